@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the SSD chunk-scan forward on one MI355X.
+
+A step is one forward of the whole op (`ssd_chunk_scan_fwd`: stages 1-4 on one stream) over one
+batch of seeded synthetic inputs already resident in HBM.  Default workload: the policy shape
+(batch 256, seqlen 2048, 8 heads, headdim 32, dstate 64, one group, chunk 128, bf16 inputs with
+fp32 accumulation, final states returned).  Prints ONE JSON line:
+
+  value        timesteps*batch/s of the whole forward (wall clock around K steps)
+  roofline     the slowest stage kernel: algorithmic bytes per launch / its mean duration,
+               measured with HIP events on the launch stream over a second timed region of K
+               steps in which the four stages are issued one by one through their own entry
+               points; all four stages are listed under "stages"
+  stream_step  the single-timestep update at batch 4096: latency and GB/s
+  cpu_baseline the plain-C oracle (sequential recurrence, float32, OpenMP) timed on this
+               box's host cores on a bounded batch slice of the same workload
+
+Timing follows the reference harness (warm-up calls, device sync, timed calls, device sync,
+mean per call: benchmarks/src/main.rs:140-166; stream step = prefill once then timed single
+steps: main.rs:168-200).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="policy_bf16")
+    ap.add_argument("--batch", type=int, default=None, help="override the workload's batch")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-stream-step", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    return ap.parse_args()
+
+
+def wall_time_steps(fn, steps, torch):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; the path shards along batch without "
+              "communication, so --gpus N>1 is not measured here", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from trading_bot_0_amd import ssd
+    from trading_bot_0_amd.synthetic import (WORKLOADS, algorithmic_bytes_fwd, make_inputs, stage_bytes,
+                                             stage_flops, step_bytes)
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    ssd.load_library()   # raises if the HIP library is not built: there is no other path
+    torch.cuda.set_device(0)
+    w = WORKLOADS[args.workload]
+    if args.batch:
+        w = w.with_batch(args.batch)
+    inp = make_inputs(w, seed=0, device="cuda")
+    x, dt, A, Bm, Cm, D, init = (inp[k] for k in ("x", "dt", "A", "B", "C", "D", "init"))
+    ws = torch.empty(ssd.workspace_bytes(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk),
+                     dtype=torch.uint8, device="cuda")
+    y = torch.empty_like(x)
+    final = torch.empty((w.batch, w.nheads, w.headdim, w.dstate), dtype=torch.float32, device="cuda")
+
+    def forward():
+        ssd.ssd_chunk_scan(x, dt, A, Bm, Cm, D, chunk=w.chunk, initial_states=init, workspace=ws, out=y,
+                           final_out=final)
+
+    for _ in range(args.warmup):
+        forward()
+    sec = wall_time_steps(forward, args.steps, torch)
+    value = w.units / sec
+
+    # ---- second timed region: the four stages one by one, HIP events between them -------------
+    dA, d32 = ssd.chunk_cumsum(dt, A, w.chunk)
+    S = ssd.chunk_state(x, Bm, dA, d32)
+
+    lib = ssd.load_library()
+    from ctypes import byref
+    dims = ssd.SsdDims(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk)
+    code = ssd.SSD_DTYPE_BF16 if w.dtype == "bf16" else ssd.SSD_DTYPE_F32
+    stream = torch.cuda.current_stream().cuda_stream
+    ip = None if init is None else init.data_ptr()
+
+    def k1():
+        return lib.ssd_chunk_cumsum_fwd(byref(dims), code, dt.data_ptr(), A.data_ptr(), dA.data_ptr(),
+                                        d32.data_ptr(), stream)
+
+    def k2():
+        return lib.ssd_chunk_state_fwd(byref(dims), code, x.data_ptr(), Bm.data_ptr(), dA.data_ptr(),
+                                       d32.data_ptr(), S.data_ptr(), stream)
+
+    def k3():
+        return lib.ssd_state_passing_fwd(byref(dims), S.data_ptr(), dA.data_ptr(), ip, S.data_ptr(),
+                                         final.data_ptr(), stream)
+
+    def k4():
+        return lib.ssd_chunk_scan_stage_fwd(byref(dims), code, x.data_ptr(), Bm.data_ptr(), Cm.data_ptr(),
+                                            dA.data_ptr(), d32.data_ptr(), S.data_ptr(), D.data_ptr(),
+                                            y.data_ptr(), stream)
+
+    stage_fns = [("chunk_cumsum", k1), ("chunk_state", k2), ("state_passing", k3), ("chunk_scan", k4)]
+    for _ in range(max(2, args.warmup // 2)):
+        for _, fn in stage_fns:
+            assert fn() == 0, ssd.last_error(lib)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    for i in range(args.steps):
+        ev[i][0].record()
+        for j, (_, fn) in enumerate(stage_fns):
+            fn()
+            ev[i][j + 1].record()
+    torch.cuda.synchronize()
+    sb, sf = stage_bytes(w), stage_flops(w)
+    stages = {}
+    for j, (name, _) in enumerate(stage_fns):
+        ms = sum(ev[i][j].elapsed_time(ev[i][j + 1]) for i in range(args.steps)) / args.steps
+        gbs = sb[name] / (ms * 1e-3) / 1e9
+        stages[name] = {"ms": round(ms, 5), "alg_bytes": sb[name], "GBps": round(gbs, 1),
+                        "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
+        if name in sf:
+            tf = sf[name] / (ms * 1e-3) / 1e12
+            stages[name]["dense_TFLOPs"] = round(tf, 1)
+            stages[name]["mfma_frac"] = round(tf / MFMA_BF16_PEAK_TFLOPS, 4)
+    dom = max(stages, key=lambda k: stages[k]["ms"])
+    roofline = {"kernel": dom, "bound": "hbm", "achieved": stages[dom]["GBps"], "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": stages[dom]["hbm_frac"], "traffic": None}
+
+    out = {
+        "metric": "SSD scan timesteps*batch/s at policy shape" if args.workload == "policy_bf16"
+                  else f"SSD scan timesteps*batch/s ({args.workload})",
+        "value": value, "unit": "timesteps*batch/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w.dtype, "data": "synthetic",
+        "config": {"workload": w.name, "batch": w.batch, "seqlen": w.seqlen, "nheads": w.nheads,
+                   "headdim": w.headdim, "dstate": w.dstate, "ngroups": w.ngroups, "chunk": w.chunk},
+        "forward_alg_bytes": algorithmic_bytes_fwd(w),
+        "forward_hbm_frac": round(algorithmic_bytes_fwd(w) / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "roofline": roofline, "stages": stages,
+        "stages_ms_sum": round(sum(s["ms"] for s in stages.values()), 5),
+    }
+
+    # ---- streaming step at batch 4096 ---------------------------------------------------------
+    if not args.no_stream_step:
+        sw = WORKLOADS["streamed_bf16"]
+        del inp, x, Bm, Cm, y, S, ws
+        torch.cuda.empty_cache()
+        si = make_inputs(sw, seed=0, device="cuda", seqlen=sw.stream_steps)
+        state = torch.zeros((sw.batch, sw.nheads, sw.headdim, sw.dstate), dtype=torch.float32, device="cuda")
+        xs = [si["x"][:, t].contiguous() for t in range(sw.stream_steps)]
+        ds = [si["dt"][:, t].contiguous() for t in range(sw.stream_steps)]
+        bs = [si["B"][:, t].contiguous() for t in range(sw.stream_steps)]
+        cs = [si["C"][:, t].contiguous() for t in range(sw.stream_steps)]
+        ys = torch.empty_like(xs[0])
+        for t in range(8):
+            ssd.ssd_step(state, xs[t], ds[t], si["A"], bs[t], cs[t], si["D"], out=ys)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for t in range(sw.stream_steps):
+            ssd.ssd_step(state, xs[t], ds[t], si["A"], bs[t], cs[t], si["D"], out=ys)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / sw.stream_steps
+        gbs = step_bytes(sw) / (us * 1e-6) / 1e9
+        out["stream_step"] = {"batch": sw.batch, "steps": sw.stream_steps, "us_per_step": round(us, 2),
+                              "alg_bytes": step_bytes(sw), "GBps": round(gbs, 1),
+                              "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
+
+    # ---- CPU baseline: the C oracle on a bounded batch slice ---------------------------------
+    if not args.no_cpu_baseline:
+        import numpy as np
+        from oracle import c_oracle
+        threads = min(16, os.cpu_count() or 1)
+        cpu = make_inputs(w.with_batch(max(threads, 16)), seed=0, device="cpu")
+        a = {k: (None if v is None else v.float().numpy()) for k, v in cpu.items()}
+
+        def run(nb):
+            t0 = time.perf_counter()
+            c_oracle.ssd_sequential_c(a["x"][:nb], a["dt"][:nb], a["A"], a["B"][:nb], a["C"][:nb], a["D"],
+                                      None if a["init"] is None else a["init"][:nb], dtype=np.float32,
+                                      nthreads=threads)
+            return time.perf_counter() - t0
+
+        nb0 = a["x"].shape[0]
+        t_probe = run(nb0)
+        reps = max(1, min(int(args.cpu_seconds / max(t_probe, 1e-3)), 200))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            run(nb0)
+        t_cpu = (time.perf_counter() - t0) / reps
+        out["cpu_baseline"] = {"value": nb0 * w.seqlen / t_cpu, "unit": "timesteps*batch/s", "cores": threads,
+                               "kind": "port",
+                               "sample": f"plain-C sequential recurrence, float32, OpenMP {threads} threads, "
+                                         f"batch slice {nb0} of {w.batch} at full seqlen, {reps} repetitions, "
+                                         f"{t_cpu * 1e3:.1f} ms each"}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,126 @@
+/*
+ * libssd_hip -- C ABI of the MI355X (gfx950) Mamba-2 SSD chunk-scan forward and the
+ * single-timestep streaming update.
+ *
+ * What each entry point replaces in CarsonBurke/trading_bot_0: the SSD op itself is no longer
+ * in that tree (only its benchmark rows survive, benchmark_results/bench_20260112_070055.json:
+ * 7,16,25,34), so the citations name the slot each call fills and the FFI conventions it
+ * follows.  Conventions are those of the tree's own extern "C" boundary, the vendored
+ * torch-sys shim:
+ *   - errors never cross the ABI as exceptions; a failing call returns non-zero and leaves a
+ *     malloc'd message in a thread-local slot fetched (and cleared) by
+ *     ssd_get_and_reset_last_err(), which the caller frees with free()
+ *     (vendor/torch-sys-0.25.0/libtch/torch_api.h:18-24,33; torch_api.cpp:32,84-88;
+ *     polled from Rust at trading_bots/src/torch/cuda/graph.rs:107-119);
+ *   - tensors stay owned by the caller and arrive as raw device pointers, the value of
+ *     Tensor::data_ptr() (vendor/torch-sys-0.25.0/src/lib.rs:38, libtch/torch_api.cpp:180);
+ *     the library retains nothing between calls;
+ *   - all work is enqueued on the stream handed in (NULL = the legacy default stream), with no
+ *     allocation and no synchronisation, so a call can sit inside the reference's captured
+ *     update (trading_bots/src/torch/train/update.rs:206-330; torch_api.cpp:408-464);
+ *   - every entry point is re-entrant: no global mutable state, unlike the FA4 bridge that
+ *     needs a process-wide lock (trading_bots/src/torch/fa4.rs:11,50-55).
+ *
+ * Tensor layouts (all contiguous row-major, last stride 1; every pointer 16-byte aligned):
+ *   x, y        [batch, seqlen, nheads, headdim]      element type = dtype
+ *   dt          [batch, seqlen, nheads]               dtype; already positive, no softplus/bias
+ *   A, D        [nheads]                              float32; A < 0; D may be NULL
+ *   Bm, Cm      [batch, seqlen, ngroups, dstate]      dtype; head h uses group h/(nheads/ngroups)
+ *   states      [batch, nheads, headdim, dstate]      float32 (initial, final, streaming)
+ *   dA_cs, dt32 [batch, nheads, nchunks, chunk]       float32 (stage 1 outputs)
+ *   chunk states[batch, nchunks, nheads, headdim, dstate] float32 (stages 2-4)
+ * Recurrence: h_t = exp(dt_t A_h) h_{t-1} + dt_t x_t (outer) B_t ; y_t = h_t . C_t + D_h x_t.
+ *
+ * Supported shapes: dstate in {16,32,64,128}; headdim a multiple of 8, <= 64; chunk in
+ * {32,64,128,256}; nheads % ngroups == 0; the LDS tile of stage 4 must fit 160 KiB (all bf16
+ * shapes do; float32 up to headdim 64 / dstate 64 / chunk 256 or dstate 128 / chunk 128).
+ * seqlen need not be a multiple of chunk: the ragged tail behaves as dt = 0 padding.
+ */
+#ifndef SSD_HIP_H
+#define SSD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SSD_DTYPE_F32 0  /* all tensors float32 */
+#define SSD_DTYPE_BF16 1 /* x, dt, Bm, Cm, y bfloat16; A, D, states, accumulators float32 */
+
+#define SSD_OK 0
+#define SSD_ERR_INVALID 1     /* NULL/misaligned pointer, non-positive or inconsistent dims */
+#define SSD_ERR_UNSUPPORTED 2 /* shape outside the kernels' tile set */
+#define SSD_ERR_WORKSPACE 3   /* workspace smaller than ssd_workspace_bytes() */
+#define SSD_ERR_RUNTIME 4     /* the HIP runtime rejected a launch */
+
+typedef struct ssd_dims {
+    int64_t batch, seqlen, nheads, headdim, dstate, ngroups, chunk;
+} ssd_dims;
+
+typedef struct ssd_step_dims {
+    int64_t batch, nheads, headdim, dstate, ngroups;
+} ssd_step_dims;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ssd_version(void);
+
+/* Thread-local last error, malloc'd; NULL when none.  Same contract as get_and_reset_last_err
+ * (vendor/torch-sys-0.25.0/libtch/torch_api.h:33, torch_api.cpp:84-88). */
+char *ssd_get_and_reset_last_err(void);
+
+/* Bytes of scratch ssd_chunk_scan_fwd needs for these dims.  The reference lets ATen allocate
+ * op temporaries; a capturable op cannot, so the caller owns the buffer (the Rust side would
+ * hold it as a Tensor::empty, cf. the persistent rollout buffers at
+ * trading_bots/src/torch/train/trainer.rs:622-944). */
+int ssd_workspace_bytes(const ssd_dims *dims, size_t *out_bytes);
+
+/* Whole forward: stages 1-4 on one stream.  Fills y and, when non-NULL, final_states.
+ * Slot: the temporal encoder's sequence mixer, TradingModel::patch_trunk
+ * (trading_bots/src/torch/model/trading_model.rs:589-606), reached from the batched replay
+ * forward (trading_bots/src/torch/model/stream/replay.rs:83-114) and from prefix
+ * initialisation of a stream (trading_bots/src/torch/model/stream/live.rs:322-360);
+ * historical benchmark rows mamba2_forward_train / mamba2_infer_prefill
+ * (benchmark_results/bench_20260112_070055.json:7,25). */
+int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt,
+                       const float *A, const void *Bm, const void *Cm, const float *D,
+                       const float *initial_states, void *y, float *final_states,
+                       void *workspace, size_t workspace_bytes, void *hip_stream);
+
+/* Stage 1: per-chunk inclusive cumulative sum of dt*A and dt as float32, both [B,H,nc,Q]. */
+int ssd_chunk_cumsum_fwd(const ssd_dims *dims, int dtype, const void *dt, const float *A,
+                         float *dA_cs, float *dt32, void *hip_stream);
+
+/* Stage 2: per-chunk states S[b,c,h,p,n] = sum_l exp(dA_cs[Q-1]-dA_cs[l]) dt[l] x[l,p] B[l,n]. */
+int ssd_chunk_state_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm,
+                        const float *dA_cs, const float *dt32, float *chunk_states,
+                        void *hip_stream);
+
+/* Stage 3: sequential recurrence over chunks.  prev_states[c] receives the state entering
+ * chunk c and may alias chunk_states (in place); final_states and initial_states may be NULL. */
+int ssd_state_passing_fwd(const ssd_dims *dims, const float *chunk_states, const float *dA_cs,
+                          const float *initial_states, float *prev_states, float *final_states,
+                          void *hip_stream);
+
+/* Stage 4: intra-chunk masked (C B^T o decay) x plus the C.h readout of the entering state
+ * plus D x. */
+int ssd_chunk_scan_stage_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm,
+                             const void *Cm, const float *dA_cs, const float *dt32,
+                             const float *prev_states, const float *D, void *y,
+                             void *hip_stream);
+
+/* One recurrent update, in place on state [B,H,P,N]:  x,y [B,H,P]; dt [B,H]; Bm,Cm [B,G,N].
+ * Slot: the per-bar streaming step step_uniform_stream_state_on_device
+ * (trading_bots/src/torch/model/stream/live.rs:228-244), called per bar from
+ * trading_bots/src/torch/infer/offline.rs:124-125 and per rollout step from
+ * trading_bots/src/torch/train/rollout.rs:209-235; historical row mamba2_infer_step
+ * (benchmark_results/bench_20260112_070055.json:34). */
+int ssd_step_fwd(const ssd_step_dims *dims, int dtype, float *state, const void *x,
+                 const void *dt, const float *A, const void *Bm, const void *Cm, const float *D,
+                 void *y, void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SSD_HIP_H */

@@ -1,0 +1,126 @@
+"""The C-ABI library loads without a GPU, exports every symbol include/ssd_hip.h declares, and
+rejects bad arguments with a code and a message before touching the device (the reference's
+wrappers validate first and bail with a message, trading_bots/src/torch/fa4.rs:145-191)."""
+import ctypes
+import re
+from ctypes import byref, c_size_t
+from pathlib import Path
+
+import pytest
+
+from trading_bot_0_amd import ssd
+
+REPO = Path(__file__).resolve().parent.parent
+FAKE = 0x1000  # aligned, never dereferenced: validation fails before any launch
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return ssd.load_library()
+
+
+def declared_symbols():
+    text = (REPO / "include" / "ssd_hip.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ssd_\w+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(lib):
+    names = declared_symbols()
+    assert sorted(names) == sorted(ssd.EXPORTED_SYMBOLS)
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_version_and_empty_error_slot(lib):
+    assert lib.ssd_version() >= 100
+    assert ssd.last_error(lib) is None
+
+
+def dims(**kw):
+    d = dict(batch=2, seqlen=256, nheads=4, headdim=32, dstate=64, ngroups=1, chunk=128)
+    d.update(kw)
+    return ssd.SsdDims(*[d[k] for k in ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "chunk")])
+
+
+def test_workspace_bytes_formula(lib):
+    out = c_size_t(0)
+    assert lib.ssd_workspace_bytes(byref(dims()), byref(out)) == 0
+    B, H, nc, Q, P, N = 2, 4, 2, 128, 32, 64
+    assert out.value == 2 * B * H * nc * Q * 4 + B * nc * H * P * N * 4
+    # ragged seqlen rounds the chunk count up
+    assert lib.ssd_workspace_bytes(byref(dims(seqlen=257)), byref(out)) == 0
+    assert out.value == 2 * B * H * 3 * Q * 4 + B * 3 * H * P * N * 4
+
+
+@pytest.mark.parametrize("kw,code,needle", [
+    (dict(batch=0), 1, "positive"),
+    (dict(seqlen=-5), 1, "positive"),
+    (dict(nheads=6, ngroups=4), 1, "divisible"),
+    (dict(dstate=48), 2, "dstate"),
+    (dict(headdim=12), 2, "headdim"),
+    (dict(headdim=128), 2, "headdim"),
+    (dict(chunk=100), 2, "chunk"),
+])
+def test_bad_dims_are_rejected_with_message(lib, kw, code, needle):
+    out = c_size_t(0)
+    assert lib.ssd_workspace_bytes(byref(dims(**kw)), byref(out)) == code
+    msg = ssd.last_error(lib)
+    assert msg and needle in msg
+    assert ssd.last_error(lib) is None  # fetching clears the slot
+
+
+def test_float32_lds_limit(lib):
+    d = dims(headdim=64, dstate=128, chunk=256)
+    rc = lib.ssd_chunk_cumsum_fwd(byref(d), 0, FAKE, FAKE, FAKE, FAKE, None)
+    assert rc == 2 and "LDS" in ssd.last_error(lib)
+    out = c_size_t(0)
+    assert lib.ssd_workspace_bytes(byref(d), byref(out)) == 0  # fine in bf16
+
+
+def test_null_misaligned_and_dtype(lib):
+    d = dims()
+    args = [FAKE] * 4 + [FAKE, None, None, FAKE, None, FAKE]  # x dt A B C D init y final ws
+    assert lib.ssd_chunk_scan_fwd(byref(d), 1, None, *args[1:], 1 << 30, None) == 1
+    assert "x must not be NULL" in ssd.last_error(lib)
+    bad = list(args)
+    bad[3] = FAKE + 2
+    assert lib.ssd_chunk_scan_fwd(byref(d), 1, *bad, 1 << 30, None) == 1
+    assert "16-byte aligned" in ssd.last_error(lib)
+    assert lib.ssd_chunk_scan_fwd(byref(d), 7, *args, 1 << 30, None) == 1
+    assert "dtype" in ssd.last_error(lib)
+    assert lib.ssd_chunk_scan_fwd(byref(d), 1, *args, 16, None) == 3
+    assert "workspace" in ssd.last_error(lib)
+    assert lib.ssd_chunk_scan_fwd(None, 1, *args, 1 << 30, None) == 1
+    sd = ssd.SsdStepDims(4, 8, 32, 64, 3)
+    assert lib.ssd_step_fwd(byref(sd), 1, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, None) == 1
+    assert "divisible" in ssd.last_error(lib)
+    sd = ssd.SsdStepDims(4, 8, 32, 64, 1)
+    assert lib.ssd_step_fwd(byref(sd), 1, None, FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, None) == 1
+    assert "state must not be NULL" in ssd.last_error(lib)
+
+
+def test_error_slot_is_thread_local(lib):
+    import threading
+    out = c_size_t(0)
+    assert lib.ssd_workspace_bytes(byref(dims(batch=0)), byref(out)) == 1
+    seen = []
+    t = threading.Thread(target=lambda: seen.append(ssd.last_error(lib)))
+    t.start()
+    t.join()
+    assert seen == [None]
+    assert "positive" in ssd.last_error(lib)
+
+
+def test_host_wrappers_validate_before_calling():
+    import torch
+    x = torch.zeros(2, 64, 4, 32)
+    with pytest.raises(ValueError, match="must be on the GPU"):
+        ssd.ssd_chunk_scan(x, torch.zeros(2, 64, 4), torch.zeros(4), torch.zeros(2, 64, 1, 64),
+                           torch.zeros(2, 64, 1, 64), chunk=32)
+    with pytest.raises(ValueError, match="rank-4"):
+        ssd.ssd_chunk_scan(x[0], torch.zeros(2, 64, 4), torch.zeros(4), torch.zeros(2, 64, 1, 64),
+                           torch.zeros(2, 64, 1, 64), chunk=32)
+    with pytest.raises(ValueError, match="float32 or bfloat16"):
+        ssd.ssd_chunk_scan(x.half(), torch.zeros(2, 64, 4), torch.zeros(4), torch.zeros(2, 64, 1, 64),
+                           torch.zeros(2, 64, 1, 64), chunk=32)

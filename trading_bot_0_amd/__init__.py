@@ -1,0 +1,14 @@
+"""MI355X-native Mamba-2 SSD chunk-scan forward and streaming step (hand-written gfx950 HIP
+kernels behind the C ABI in include/ssd_hip.h)."""
+from .ssd import (  # noqa: F401
+    SsdError,
+    chunk_cumsum,
+    chunk_scan_stage,
+    chunk_state,
+    load_library,
+    ssd_chunk_scan,
+    ssd_step,
+    state_passing,
+    workspace_bytes,
+)
+from .stream_state import SsdStreamState  # noqa: F401

@@ -1,0 +1,39 @@
+// Internal interface between the C ABI (ssd_api.cpp) and the gfx950 kernels (ssd_kernels.hip).
+// Shapes arrive here already validated; launchers only pick a template instance and a grid.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace ssd {
+
+struct ScanShape {
+    int B, L, H, P, N, G, Q, nc;
+};
+
+struct StepShape {
+    int B, H, P, N, G;
+};
+
+constexpr size_t kLdsLimitBytes = 160 * 1024;  // LDS per workgroup on gfx950
+
+// Dynamic LDS the stage-2 / stage-4 workgroup needs (elem_bytes = 2 for bf16, 4 for float).
+size_t chunk_state_lds_bytes(const ScanShape &s, int elem_bytes);
+size_t chunk_scan_lds_bytes(const ScanShape &s, int elem_bytes);
+
+hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A,
+                               float *dA_cs, float *dt32, hipStream_t stream);
+hipError_t launch_chunk_state(const ScanShape &s, int dtype, const void *x, const void *Bm,
+                              const float *dA_cs, const float *dt32, float *states,
+                              hipStream_t stream);
+hipError_t launch_state_passing(const ScanShape &s, const float *states, const float *dA_cs,
+                                const float *init, float *prev, float *final_states,
+                                hipStream_t stream);
+hipError_t launch_chunk_scan(const ScanShape &s, int dtype, const void *x, const void *Bm,
+                             const void *Cm, const float *dA_cs, const float *dt32,
+                             const float *prev, const float *D, void *y, hipStream_t stream);
+hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *x, const void *dt,
+                       const float *A, const void *Bm, const void *Cm, const float *D, void *y,
+                       hipStream_t stream);
+
+}  // namespace ssd

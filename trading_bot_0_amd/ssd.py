@@ -1,0 +1,329 @@
+"""Host-side operator interface of the SSD path: the functions a model calls, over torch-ROCm
+tensors, bound to libssd_hip.so through its C ABI with ctypes.
+
+The shape of this module mirrors how the reference wraps a custom kernel
+(`trading_bots/src/torch/fa4.rs:28-47` public op functions, `:145-191` validate-then-call with a
+message per violated precondition): `ssd_chunk_scan(...) -> (y, final_states)` is the batched
+op that sits in the temporal-encoder slot (`trading_bots/src/torch/model/trading_model.rs:589-606`)
+and `ssd_step(state, ...) -> y` is the per-bar streaming update
+(`trading_bots/src/torch/model/stream/live.rs:228-244`).  Tensors stay owned by the caller; raw
+device pointers are `Tensor.data_ptr()` exactly as the Rust side would pass
+(`vendor/torch-sys-0.25.0/src/lib.rs:38`).  torch is used for device memory and the current
+stream only -- there is no fallback: without the built library every call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import POINTER, Structure, byref, c_char_p, c_int, c_int64, c_size_t, c_void_p
+from typing import Optional, Tuple
+
+import torch
+
+from ._build import LIB_PATH
+
+SSD_DTYPE_F32 = 0
+SSD_DTYPE_BF16 = 1
+
+EXPORTED_SYMBOLS = (
+    "ssd_version",
+    "ssd_get_and_reset_last_err",
+    "ssd_workspace_bytes",
+    "ssd_chunk_scan_fwd",
+    "ssd_chunk_cumsum_fwd",
+    "ssd_chunk_state_fwd",
+    "ssd_state_passing_fwd",
+    "ssd_chunk_scan_stage_fwd",
+    "ssd_step_fwd",
+)
+
+
+class SsdError(RuntimeError):
+    """A call into libssd_hip returned non-zero; carries the library's message and code."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"[ssd error {code}] {message}")
+        self.code = code
+        self.message = message
+
+
+class SsdDims(Structure):
+    _fields_ = [(n, c_int64) for n in ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "chunk")]
+
+
+class SsdStepDims(Structure):
+    _fields_ = [(n, c_int64) for n in ("batch", "nheads", "headdim", "dstate", "ngroups")]
+
+
+_lib = None
+_lib_lock = threading.Lock()
+_libc = ctypes.CDLL(None)
+_libc.free.argtypes = [c_void_p]
+_libc.free.restype = None
+
+
+def load_library() -> ctypes.CDLL:
+    """Loads libssd_hip.so (after torch, so both share one HIP runtime).  Raises if it is not
+    built: the HIP path is the only path."""
+    global _lib
+    with _lib_lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+                "from the repository root (needs hipcc). There is no CPU fallback."
+            )
+        lib = ctypes.CDLL(str(LIB_PATH))
+        P = c_void_p
+        lib.ssd_version.argtypes = []
+        lib.ssd_version.restype = c_int
+        lib.ssd_get_and_reset_last_err.argtypes = []
+        lib.ssd_get_and_reset_last_err.restype = c_void_p
+        lib.ssd_workspace_bytes.argtypes = [POINTER(SsdDims), POINTER(c_size_t)]
+        lib.ssd_chunk_scan_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, c_size_t, P]
+        lib.ssd_chunk_cumsum_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P]
+        lib.ssd_chunk_state_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P]
+        lib.ssd_state_passing_fwd.argtypes = [POINTER(SsdDims), P, P, P, P, P, P]
+        lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P]
+        lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
+        for name in EXPORTED_SYMBOLS[2:]:
+            getattr(lib, name).restype = c_int
+        _lib = lib
+        return lib
+
+
+def last_error(lib: Optional[ctypes.CDLL] = None) -> Optional[str]:
+    """Fetches and clears this thread's error message (freed here, as the Rust side does with
+    libc::free, `trading_bots/src/torch/cuda/graph.rs:107-119`)."""
+    lib = lib or load_library()
+    ptr = lib.ssd_get_and_reset_last_err()
+    if not ptr:
+        return None
+    msg = ctypes.string_at(ptr).decode("utf-8", "replace")
+    _libc.free(ptr)
+    return msg
+
+
+def _check(lib, rc: int) -> None:
+    if rc != 0:
+        raise SsdError(rc, last_error(lib) or "unknown error")
+
+
+def _stream_ptr(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return SSD_DTYPE_F32
+    if t.dtype == torch.bfloat16:
+        return SSD_DTYPE_BF16
+    raise ValueError(f"SSD tensors must be float32 or bfloat16, got {t.dtype}")
+
+
+def _require(t: torch.Tensor, name: str, shape, dtype) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise ValueError(f"SSD {name} must be a tensor")
+    if not t.is_cuda:
+        raise ValueError(f"SSD {name} must be on the GPU, got {t.device}")
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f"SSD {name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    if t.dtype != dtype:
+        raise ValueError(f"SSD {name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"SSD {name} must be contiguous")
+
+
+def _scan_dims(x, Bm, chunk) -> SsdDims:
+    if x.dim() != 4:
+        raise ValueError(f"SSD x must be rank-4 [batch, seqlen, nheads, headdim], got {tuple(x.shape)}")
+    if Bm.dim() != 4:
+        raise ValueError(f"SSD B must be rank-4 [batch, seqlen, ngroups, dstate], got {tuple(Bm.shape)}")
+    Bsz, L, H, P = x.shape
+    return SsdDims(Bsz, L, H, P, Bm.shape[3], Bm.shape[2], int(chunk))
+
+
+def num_chunks(seqlen: int, chunk: int) -> int:
+    return -(-seqlen // chunk)
+
+
+def workspace_bytes(batch, seqlen, nheads, headdim, dstate, ngroups, chunk) -> int:
+    lib = load_library()
+    out = c_size_t(0)
+    _check(lib, lib.ssd_workspace_bytes(byref(SsdDims(batch, seqlen, nheads, headdim, dstate, ngroups, chunk)),
+                                        byref(out)))
+    return out.value
+
+
+def _validate_scan_inputs(x, dt, A, Bm, Cm, D, initial_states, dims: SsdDims):
+    Bsz, L, H, P, N, G = dims.batch, dims.seqlen, dims.nheads, dims.headdim, dims.dstate, dims.ngroups
+    dtype = x.dtype
+    _dtype_code(x)
+    _require(x, "x", (Bsz, L, H, P), dtype)
+    if dt is not None:
+        _require(dt, "dt", (Bsz, L, H), dtype)
+    if A is not None:
+        _require(A, "A", (H,), torch.float32)
+    _require(Bm, "B", (Bsz, L, G, N), dtype)
+    if Cm is not None:
+        _require(Cm, "C", (Bsz, L, G, N), dtype)
+    if D is not None:
+        _require(D, "D", (H,), torch.float32)
+    if initial_states is not None:
+        _require(initial_states, "initial_states", (Bsz, H, P, N), torch.float32)
+    for name, t in (("dt", dt), ("A", A), ("B", Bm), ("C", Cm), ("D", D), ("initial_states", initial_states)):
+        if t is not None and t.device != x.device:
+            raise ValueError(f"SSD {name} must be on {x.device}, got {t.device}")
+
+
+def ssd_chunk_scan(
+    x: torch.Tensor,
+    dt: torch.Tensor,
+    A: torch.Tensor,
+    Bm: torch.Tensor,
+    Cm: torch.Tensor,
+    D: Optional[torch.Tensor] = None,
+    chunk: int = 128,
+    initial_states: Optional[torch.Tensor] = None,
+    return_final_states: bool = True,
+    workspace: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+    final_out: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """SSD chunk-scan forward.  Returns (y [B,L,H,P] in x's dtype, final_states [B,H,P,N] fp32).
+
+    `workspace` (uint8, >= workspace_bytes(...)), `out` and `final_out` let a caller that runs
+    under stream capture or in a tight loop avoid any allocation."""
+    lib = load_library()
+    dims = _scan_dims(x, Bm, chunk)
+    _validate_scan_inputs(x, dt, A, Bm, Cm, D, initial_states, dims)
+    y = torch.empty_like(x) if out is None else out
+    _require(y, "out", x.shape, x.dtype)
+    final = None
+    if return_final_states:
+        shape = (dims.batch, dims.nheads, dims.headdim, dims.dstate)
+        final = torch.empty(shape, dtype=torch.float32, device=x.device) if final_out is None else final_out
+        _require(final, "final_out", shape, torch.float32)
+    need = c_size_t(0)
+    _check(lib, lib.ssd_workspace_bytes(byref(dims), byref(need)))
+    if workspace is None:
+        workspace = torch.empty(need.value, dtype=torch.uint8, device=x.device)
+    elif (not workspace.is_cuda) or workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+        raise ValueError("SSD workspace must be a contiguous uint8 GPU tensor")
+    rc = lib.ssd_chunk_scan_fwd(byref(dims), _dtype_code(x), x.data_ptr(), dt.data_ptr(), A.data_ptr(),
+                                Bm.data_ptr(), Cm.data_ptr(), _ptr(D), _ptr(initial_states), y.data_ptr(),
+                                _ptr(final), workspace.data_ptr(), workspace.numel(), _stream_ptr(x))
+    _check(lib, rc)
+    return y, final
+
+
+# ---- per-stage entry points (testing / profiling) ----------------------------------------
+
+def chunk_cumsum(dt: torch.Tensor, A: torch.Tensor, chunk: int):
+    """Stage 1 -> (dA_cs, dt32), both [B,H,nc,Q] float32."""
+    lib = load_library()
+    if dt.dim() != 3:
+        raise ValueError(f"SSD dt must be rank-3 [batch, seqlen, nheads], got {tuple(dt.shape)}")
+    Bsz, L, H = dt.shape
+    _require(dt, "dt", (Bsz, L, H), dt.dtype)
+    _require(A, "A", (H,), torch.float32)
+    nc = num_chunks(L, chunk)
+    dA = torch.empty((Bsz, H, nc, chunk), dtype=torch.float32, device=dt.device)
+    d32 = torch.empty_like(dA)
+    dims = SsdDims(Bsz, L, H, 32, 64, 1, int(chunk))  # P, N, G do not enter stage 1
+    _check(lib, lib.ssd_chunk_cumsum_fwd(byref(dims), _dtype_code(dt), dt.data_ptr(), A.data_ptr(),
+                                         dA.data_ptr(), d32.data_ptr(), _stream_ptr(dt)))
+    return dA, d32
+
+
+def chunk_state(x, Bm, dA_cs, dt32):
+    """Stage 2 -> chunk states [B,nc,H,P,N] float32."""
+    lib = load_library()
+    chunk = dA_cs.shape[-1]
+    dims = _scan_dims(x, Bm, chunk)
+    _validate_scan_inputs(x, None, None, Bm, None, None, None, dims)
+    nc = num_chunks(dims.seqlen, chunk)
+    _require(dA_cs, "dA_cs", (dims.batch, dims.nheads, nc, chunk), torch.float32)
+    _require(dt32, "dt32", (dims.batch, dims.nheads, nc, chunk), torch.float32)
+    S = torch.empty((dims.batch, nc, dims.nheads, dims.headdim, dims.dstate), dtype=torch.float32, device=x.device)
+    _check(lib, lib.ssd_chunk_state_fwd(byref(dims), _dtype_code(x), x.data_ptr(), Bm.data_ptr(),
+                                        dA_cs.data_ptr(), dt32.data_ptr(), S.data_ptr(), _stream_ptr(x)))
+    return S
+
+
+def state_passing(states, dA_cs, initial_states=None, in_place: bool = False):
+    """Stage 3 -> (prev_states [B,nc,H,P,N], final_states [B,H,P,N])."""
+    lib = load_library()
+    if states.dim() != 5:
+        raise ValueError(f"SSD chunk states must be rank-5 [batch, nchunks, nheads, headdim, dstate]")
+    Bsz, nc, H, P, N = states.shape
+    chunk = dA_cs.shape[-1]
+    _require(states, "chunk_states", (Bsz, nc, H, P, N), torch.float32)
+    _require(dA_cs, "dA_cs", (Bsz, H, nc, chunk), torch.float32)
+    if initial_states is not None:
+        _require(initial_states, "initial_states", (Bsz, H, P, N), torch.float32)
+    prev = states if in_place else torch.empty_like(states)
+    final = torch.empty((Bsz, H, P, N), dtype=torch.float32, device=states.device)
+    dims = SsdDims(Bsz, nc * chunk, H, P, N, 1, int(chunk))
+    _check(lib, lib.ssd_state_passing_fwd(byref(dims), states.data_ptr(), dA_cs.data_ptr(), _ptr(initial_states),
+                                          prev.data_ptr(), final.data_ptr(), _stream_ptr(states)))
+    return prev, final
+
+
+def chunk_scan_stage(x, Bm, Cm, dA_cs, dt32, prev_states, D=None):
+    """Stage 4 -> y [B,L,H,P]."""
+    lib = load_library()
+    chunk = dA_cs.shape[-1]
+    dims = _scan_dims(x, Bm, chunk)
+    _validate_scan_inputs(x, None, None, Bm, Cm, D, None, dims)
+    nc = num_chunks(dims.seqlen, chunk)
+    _require(dA_cs, "dA_cs", (dims.batch, dims.nheads, nc, chunk), torch.float32)
+    _require(dt32, "dt32", (dims.batch, dims.nheads, nc, chunk), torch.float32)
+    _require(prev_states, "prev_states", (dims.batch, nc, dims.nheads, dims.headdim, dims.dstate), torch.float32)
+    y = torch.empty_like(x)
+    _check(lib, lib.ssd_chunk_scan_stage_fwd(byref(dims), _dtype_code(x), x.data_ptr(), Bm.data_ptr(),
+                                             Cm.data_ptr(), dA_cs.data_ptr(), dt32.data_ptr(),
+                                             prev_states.data_ptr(), _ptr(D), y.data_ptr(), _stream_ptr(x)))
+    return y
+
+
+def ssd_step(
+    state: torch.Tensor,
+    x: torch.Tensor,
+    dt: torch.Tensor,
+    A: torch.Tensor,
+    Bm: torch.Tensor,
+    Cm: torch.Tensor,
+    D: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """One recurrent update.  `state` [B,H,P,N] fp32 is advanced in place; returns y [B,H,P]."""
+    lib = load_library()
+    if state.dim() != 4:
+        raise ValueError(f"SSD state must be rank-4 [batch, nheads, headdim, dstate], got {tuple(state.shape)}")
+    if Bm.dim() != 3:
+        raise ValueError(f"SSD step B must be rank-3 [batch, ngroups, dstate], got {tuple(Bm.shape)}")
+    Bsz, H, P, N = state.shape
+    G = Bm.shape[1]
+    dtype = x.dtype
+    _dtype_code(x)
+    _require(state, "state", (Bsz, H, P, N), torch.float32)
+    _require(x, "x", (Bsz, H, P), dtype)
+    _require(dt, "dt", (Bsz, H), dtype)
+    _require(A, "A", (H,), torch.float32)
+    _require(Bm, "B", (Bsz, G, N), dtype)
+    _require(Cm, "C", (Bsz, G, N), dtype)
+    if D is not None:
+        _require(D, "D", (H,), torch.float32)
+    y = torch.empty_like(x) if out is None else out
+    _require(y, "out", (Bsz, H, P), dtype)
+    dims = SsdStepDims(Bsz, H, P, N, G)
+    _check(lib, lib.ssd_step_fwd(byref(dims), _dtype_code(x), state.data_ptr(), x.data_ptr(), dt.data_ptr(),
+                                 A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), _ptr(D), y.data_ptr(),
+                                 _stream_ptr(x)))
+    return y
