@@ -90,8 +90,8 @@ def main():
     value = w.units / sec
 
     # ---- second timed region: the four stages one by one, HIP events between them -------------
-    dA, d32 = ssd.chunk_cumsum(dt, A, w.chunk)
-    S = ssd.chunk_state(x, Bm, dA, d32)
+    dtcs = ssd.chunk_cumsum(dt, A, w.chunk)
+    S = ssd.chunk_state(x, Bm, dtcs)
 
     lib = ssd.load_library()
     from ctypes import byref
@@ -101,21 +101,19 @@ def main():
     ip = None if init is None else init.data_ptr()
 
     def k1():
-        return lib.ssd_chunk_cumsum_fwd(byref(dims), code, dt.data_ptr(), A.data_ptr(), dA.data_ptr(),
-                                        d32.data_ptr(), stream)
+        return lib.ssd_chunk_cumsum_fwd(byref(dims), code, dt.data_ptr(), A.data_ptr(), dtcs.data_ptr(), stream)
 
     def k2():
-        return lib.ssd_chunk_state_fwd(byref(dims), code, x.data_ptr(), Bm.data_ptr(), dA.data_ptr(),
-                                       d32.data_ptr(), S.data_ptr(), stream)
+        return lib.ssd_chunk_state_fwd(byref(dims), code, x.data_ptr(), Bm.data_ptr(), dtcs.data_ptr(),
+                                       S.data_ptr(), stream)
 
     def k3():
-        return lib.ssd_state_passing_fwd(byref(dims), S.data_ptr(), dA.data_ptr(), ip, S.data_ptr(),
+        return lib.ssd_state_passing_fwd(byref(dims), S.data_ptr(), dtcs.data_ptr(), ip, S.data_ptr(),
                                          final.data_ptr(), stream)
 
     def k4():
         return lib.ssd_chunk_scan_stage_fwd(byref(dims), code, x.data_ptr(), Bm.data_ptr(), Cm.data_ptr(),
-                                            dA.data_ptr(), d32.data_ptr(), S.data_ptr(), D.data_ptr(),
-                                            y.data_ptr(), stream)
+                                            dtcs.data_ptr(), S.data_ptr(), D.data_ptr(), y.data_ptr(), stream)
 
     stage_fns = [("chunk_cumsum", k1), ("chunk_state", k2), ("state_passing", k3), ("chunk_scan", k4)]
     for _ in range(max(2, args.warmup // 2)):

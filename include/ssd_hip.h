@@ -27,7 +27,11 @@
  *   A, D        [nheads]                              float32; A < 0; D may be NULL
  *   Bm, Cm      [batch, seqlen, ngroups, dstate]      dtype; head h uses group h/(nheads/ngroups)
  *   states      [batch, nheads, headdim, dstate]      float32 (initial, final, streaming)
- *   dA_cs, dt32 [batch, nheads, nchunks, chunk]       float32 (stage 1 outputs)
+ *   dtcs        [batch, nheads, nchunks, 3, chunk]    float32 (stage 1 output): rows 0 and 1 are
+ *               log2(e) times the per-chunk inclusive cumulative sum of dt*A, as an unevaluated
+ *               pair hi + lo (later stages only use differences of it, which the pair keeps
+ *               exact to the difference's own rounding, and turn them into decays with one
+ *               exp2), row 2 is dt
  *   chunk states[batch, nchunks, nheads, headdim, dstate] float32 (stages 2-4)
  * Recurrence: h_t = exp(dt_t A_h) h_{t-1} + dt_t x_t (outer) B_t ; y_t = h_t . C_t + D_h x_t.
  *
@@ -48,6 +52,7 @@ extern "C" {
 
 #define SSD_DTYPE_F32 0  /* all tensors float32 */
 #define SSD_DTYPE_BF16 1 /* x, dt, Bm, Cm, y bfloat16; A, D, states, accumulators float32 */
+#define SSD_DTYPE_BF16_Y32 2 /* as 1, but y is written as float32 (no output rounding) */
 
 #define SSD_OK 0
 #define SSD_ERR_INVALID 1     /* NULL/misaligned pointer, non-positive or inconsistent dims */
@@ -88,27 +93,28 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
                        const float *initial_states, void *y, float *final_states,
                        void *workspace, size_t workspace_bytes, void *hip_stream);
 
-/* Stage 1: per-chunk inclusive cumulative sum of dt*A and dt as float32, both [B,H,nc,Q]. */
-int ssd_chunk_cumsum_fwd(const ssd_dims *dims, int dtype, const void *dt, const float *A,
-                         float *dA_cs, float *dt32, void *hip_stream);
+/* Stage 1: per-chunk inclusive cumulative sum of dt*A (times log2 e, hi/lo pair) and dt as float32
+ * -> dtcs. */
+int ssd_chunk_cumsum_fwd(const ssd_dims *dims, int dtype, const void *dt, const float *A, float *dtcs,
+                         void *hip_stream);
 
-/* Stage 2: per-chunk states S[b,c,h,p,n] = sum_l exp(dA_cs[Q-1]-dA_cs[l]) dt[l] x[l,p] B[l,n]. */
+/* Stage 2: per-chunk states S[b,c,h,p,n] = sum_l exp(cs[Q-1]-cs[l]) dt[l] x[l,p] B[l,n], cs the
+ * cumulative sum of dt*A inside chunk c. */
 int ssd_chunk_state_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm,
-                        const float *dA_cs, const float *dt32, float *chunk_states,
-                        void *hip_stream);
+                        const float *dtcs, float *chunk_states, void *hip_stream);
 
 /* Stage 3: sequential recurrence over chunks.  prev_states[c] receives the state entering
- * chunk c and may alias chunk_states (in place); final_states and initial_states may be NULL. */
-int ssd_state_passing_fwd(const ssd_dims *dims, const float *chunk_states, const float *dA_cs,
+ * chunk c and may alias chunk_states (in place); final_states and initial_states may be NULL
+ * and may alias each other. */
+int ssd_state_passing_fwd(const ssd_dims *dims, const float *chunk_states, const float *dtcs,
                           const float *initial_states, float *prev_states, float *final_states,
                           void *hip_stream);
 
 /* Stage 4: intra-chunk masked (C B^T o decay) x plus the C.h readout of the entering state
  * plus D x. */
 int ssd_chunk_scan_stage_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm,
-                             const void *Cm, const float *dA_cs, const float *dt32,
-                             const float *prev_states, const float *D, void *y,
-                             void *hip_stream);
+                             const void *Cm, const float *dtcs, const float *prev_states,
+                             const float *D, void *y, void *hip_stream);
 
 /* One recurrent update, in place on state [B,H,P,N]:  x,y [B,H,P]; dt [B,H]; Bm,Cm [B,G,N].
  * Slot: the per-bar streaming step step_uniform_stream_state_on_device

@@ -1,13 +1,24 @@
 """Shared helpers of the GPU parity tests: moving synthetic inputs to the device, handing the
-oracle exactly the values the kernels see, and the parity metric."""
+oracle exactly the values the kernels see, and the parity rules.
+
+Parity rules (max|out - ref| / rms(ref), ref = float64 oracle on the inputs' exact values):
+  float32 mode           <= 1e-4
+  bf16-in / fp32-acc     <= 2e-2, judged on the float32-y output of the same kernels; the bf16 y
+                         must then be exactly that result rounded once to bf16.
+Why not the plain metric on the bf16 y: storing y in bf16 costs up to 2^-8 |y| whatever computed
+it, and y's largest elements sit 10..100s of RMS out (D*x with the largest |D|; Student-t x), so
+the output format alone can exceed 2e-2 RMS.  The rule above is the stronger statement: the
+arithmetic meets the bar, and the stored y is the correctly rounded value of that arithmetic.
+"""
 import numpy as np
 import torch
 
 from oracle import c_oracle
 from oracle import ssd_oracle as orc
 
-TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}   # max|out-ref| / rms(ref), per the task's bar
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}
 ORACLE_THREADS = 16
+LOG2E = 1.4426950408889634
 
 
 def np64(t):
@@ -36,3 +47,18 @@ def assert_close(out, ref, dtype, what):
     e = rel_err(out, ref)
     assert np.isfinite(e) and e <= TOL[dtype], f"{what}: max|err|/rms = {e:.3e} > {TOL[dtype]:.0e}"
     return e
+
+
+def check_y(call, ref, dtype, what):
+    """`call(y_dtype)` runs the op and returns y.  Applies the parity rule for `dtype` (the input
+    dtype) and returns (y in the default output dtype, error of the judged output)."""
+    if dtype == torch.float32:
+        y = call(None)
+        return y, assert_close(y, ref, dtype, what)
+    y32 = call(torch.float32)
+    assert y32.dtype == torch.float32
+    e = assert_close(y32, ref, dtype, f"{what} (float32 y)")
+    y16 = call(None)
+    assert y16.dtype == torch.bfloat16
+    assert torch.equal(y16, y32.to(torch.bfloat16)), f"{what}: bf16 y is not the rounded float32 y"
+    return y16, e

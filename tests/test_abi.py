@@ -47,10 +47,10 @@ def test_workspace_bytes_formula(lib):
     out = c_size_t(0)
     assert lib.ssd_workspace_bytes(byref(dims()), byref(out)) == 0
     B, H, nc, Q, P, N = 2, 4, 2, 128, 32, 64
-    assert out.value == 2 * B * H * nc * Q * 4 + B * nc * H * P * N * 4
+    assert out.value == 3 * B * H * nc * Q * 4 + B * nc * H * P * N * 4
     # ragged seqlen rounds the chunk count up
     assert lib.ssd_workspace_bytes(byref(dims(seqlen=257)), byref(out)) == 0
-    assert out.value == 2 * B * H * 3 * Q * 4 + B * 3 * H * P * N * 4
+    assert out.value == 3 * B * H * 3 * Q * 4 + B * 3 * H * P * N * 4
 
 
 @pytest.mark.parametrize("kw,code,needle", [
@@ -72,7 +72,7 @@ def test_bad_dims_are_rejected_with_message(lib, kw, code, needle):
 
 def test_float32_lds_limit(lib):
     d = dims(headdim=64, dstate=128, chunk=256)
-    rc = lib.ssd_chunk_cumsum_fwd(byref(d), 0, FAKE, FAKE, FAKE, FAKE, None)
+    rc = lib.ssd_chunk_cumsum_fwd(byref(d), 0, FAKE, FAKE, FAKE, None)
     assert rc == 2 and "LDS" in ssd.last_error(lib)
     out = c_size_t(0)
     assert lib.ssd_workspace_bytes(byref(d), byref(out)) == 0  # fine in bf16
@@ -96,6 +96,8 @@ def test_null_misaligned_and_dtype(lib):
     assert lib.ssd_step_fwd(byref(sd), 1, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, None) == 1
     assert "divisible" in ssd.last_error(lib)
     sd = ssd.SsdStepDims(4, 8, 32, 64, 1)
+    assert lib.ssd_step_fwd(byref(sd), 3, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, None) == 1
+    assert "dtype" in ssd.last_error(lib)
     assert lib.ssd_step_fwd(byref(sd), 1, None, FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, None) == 1
     assert "state must not be NULL" in ssd.last_error(lib)
 

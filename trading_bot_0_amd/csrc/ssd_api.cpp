@@ -42,8 +42,9 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
     } while (0)
 
 int check_dtype(int dtype) {
-    if (dtype != SSD_DTYPE_F32 && dtype != SSD_DTYPE_BF16)
-        return fail(SSD_ERR_INVALID, "ssd: dtype must be 0 (float32) or 1 (bfloat16), got %d", dtype);
+    if (dtype != SSD_DTYPE_F32 && dtype != SSD_DTYPE_BF16 && dtype != SSD_DTYPE_BF16_Y32)
+        return fail(SSD_ERR_INVALID,
+                    "ssd: dtype must be 0 (float32), 1 (bfloat16) or 2 (bfloat16 with float32 y), got %d", dtype);
     return SSD_OK;
 }
 
@@ -80,7 +81,7 @@ int make_shape(const ssd_dims *d, int dtype, ssd::ScanShape *out) {
         return fail(SSD_ERR_UNSUPPORTED, "ssd: batch*nchunks*nheads or batch*seqlen exceeds 2^31-1");
     ssd::ScanShape s{(int)d->batch, (int)d->seqlen, (int)d->nheads, (int)d->headdim,
                      (int)d->dstate, (int)d->ngroups, (int)d->chunk, (int)nc};
-    const int eb = dtype == SSD_DTYPE_BF16 ? 2 : 4;
+    const int eb = dtype == SSD_DTYPE_F32 ? 4 : 2;
     if (ssd::chunk_scan_lds_bytes(s, eb) > ssd::kLdsLimitBytes || ssd::chunk_state_lds_bytes(s, eb) > ssd::kLdsLimitBytes)
         return fail(SSD_ERR_UNSUPPORTED,
                     "ssd: headdim %lld / dstate %lld / chunk %lld needs more than 160 KiB of LDS in %s mode",
@@ -90,16 +91,15 @@ int make_shape(const ssd_dims *d, int dtype, ssd::ScanShape *out) {
 }
 
 struct Workspace {
-    size_t dA_off, dt_off, st_off, total;
+    size_t dtcs_off, st_off, total;
 };
 
 Workspace carve(const ssd::ScanShape &s) {
     Workspace w;
-    const size_t row = (size_t)s.B * s.H * s.nc * s.Q * sizeof(float);
+    const size_t dtcs = (size_t)s.B * s.H * s.nc * 3 * s.Q * sizeof(float);
     const size_t st = (size_t)s.B * s.nc * s.H * s.P * s.N * sizeof(float);
-    w.dA_off = 0;
-    w.dt_off = align_up(row, 256);
-    w.st_off = w.dt_off + align_up(row, 256);
+    w.dtcs_off = 0;
+    w.st_off = align_up(dtcs, 256);
     w.total = w.st_off + align_up(st, 256);
     return w;
 }
@@ -130,61 +130,57 @@ int ssd_workspace_bytes(const ssd_dims *dims, size_t *out_bytes) {
     return SSD_OK;
 }
 
-int ssd_chunk_cumsum_fwd(const ssd_dims *dims, int dtype, const void *dt, const float *A, float *dA_cs,
-                         float *dt32, void *hip_stream) {
+int ssd_chunk_cumsum_fwd(const ssd_dims *dims, int dtype, const void *dt, const float *A, float *dtcs,
+                         void *hip_stream) {
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
     REQUIRE_PTR(dt);
     REQUIRE_PTR(A);
-    REQUIRE_PTR(dA_cs);
-    REQUIRE_PTR(dt32);
-    hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dA_cs, dt32, (hipStream_t)hip_stream);
+    REQUIRE_PTR(dtcs);
+    hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dtcs, (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "chunk_cumsum launch");
 }
 
-int ssd_chunk_state_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm, const float *dA_cs,
-                        const float *dt32, float *chunk_states, void *hip_stream) {
+int ssd_chunk_state_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm, const float *dtcs,
+                        float *chunk_states, void *hip_stream) {
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
     REQUIRE_PTR(x);
     REQUIRE_PTR(Bm);
-    REQUIRE_PTR(dA_cs);
-    REQUIRE_PTR(dt32);
+    REQUIRE_PTR(dtcs);
     REQUIRE_PTR(chunk_states);
-    hipError_t e = ssd::launch_chunk_state(s, dtype, x, Bm, dA_cs, dt32, chunk_states, (hipStream_t)hip_stream);
+    hipError_t e = ssd::launch_chunk_state(s, dtype, x, Bm, dtcs, chunk_states, (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "chunk_state launch");
 }
 
-int ssd_state_passing_fwd(const ssd_dims *dims, const float *chunk_states, const float *dA_cs,
+int ssd_state_passing_fwd(const ssd_dims *dims, const float *chunk_states, const float *dtcs,
                           const float *initial_states, float *prev_states, float *final_states,
                           void *hip_stream) {
     ssd::ScanShape s;
     if (int rc = make_shape(dims, SSD_DTYPE_BF16, &s)) return rc;
     REQUIRE_PTR(chunk_states);
-    REQUIRE_PTR(dA_cs);
+    REQUIRE_PTR(dtcs);
     REQUIRE_PTR(prev_states);
     OPTIONAL_PTR(initial_states);
     OPTIONAL_PTR(final_states);
-    hipError_t e = ssd::launch_state_passing(s, chunk_states, dA_cs, initial_states, prev_states, final_states,
+    hipError_t e = ssd::launch_state_passing(s, chunk_states, dtcs, initial_states, prev_states, final_states,
                                              (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "state_passing launch");
 }
 
 int ssd_chunk_scan_stage_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm, const void *Cm,
-                             const float *dA_cs, const float *dt32, const float *prev_states, const float *D,
-                             void *y, void *hip_stream) {
+                             const float *dtcs, const float *prev_states, const float *D, void *y,
+                             void *hip_stream) {
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
     REQUIRE_PTR(x);
     REQUIRE_PTR(Bm);
     REQUIRE_PTR(Cm);
-    REQUIRE_PTR(dA_cs);
-    REQUIRE_PTR(dt32);
+    REQUIRE_PTR(dtcs);
     REQUIRE_PTR(prev_states);
     REQUIRE_PTR(y);
     OPTIONAL_PTR(D);
-    hipError_t e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dA_cs, dt32, prev_states, D, y,
-                                          (hipStream_t)hip_stream);
+    hipError_t e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dtcs, prev_states, D, y, (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "chunk_scan launch");
 }
 
@@ -207,17 +203,16 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
     if (workspace_bytes < w.total)
         return fail(SSD_ERR_WORKSPACE, "ssd: workspace has %zu bytes, %zu needed", workspace_bytes, w.total);
     char *base = static_cast<char *>(workspace);
-    float *dA_cs = reinterpret_cast<float *>(base + w.dA_off);
-    float *dt32 = reinterpret_cast<float *>(base + w.dt_off);
+    float *dtcs = reinterpret_cast<float *>(base + w.dtcs_off);
     float *states = reinterpret_cast<float *>(base + w.st_off);
     hipStream_t st = (hipStream_t)hip_stream;
-    hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dA_cs, dt32, st);
+    hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dtcs, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_cumsum launch");
-    e = ssd::launch_chunk_state(s, dtype, x, Bm, dA_cs, dt32, states, st);
+    e = ssd::launch_chunk_state(s, dtype, x, Bm, dtcs, states, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_state launch");
-    e = ssd::launch_state_passing(s, states, dA_cs, initial_states, states, final_states, st);  // in place
+    e = ssd::launch_state_passing(s, states, dtcs, initial_states, states, final_states, st);  // in place
     if (e != hipSuccess) return hip_fail(e, "state_passing launch");
-    e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dA_cs, dt32, states, D, y, st);
+    e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dtcs, states, D, y, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_scan launch");
     return SSD_OK;
 }

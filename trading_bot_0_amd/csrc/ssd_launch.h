@@ -21,17 +21,18 @@ constexpr size_t kLdsLimitBytes = 160 * 1024;  // LDS per workgroup on gfx950
 size_t chunk_state_lds_bytes(const ScanShape &s, int elem_bytes);
 size_t chunk_scan_lds_bytes(const ScanShape &s, int elem_bytes);
 
+// dtype: 0 = float32, 1 = bf16, 2 = bf16 inputs with float32 y (stage 4 only; stages 1-2 treat it as 1).
+// dtcs is the stage-1 output [B,H,nc,3,Q] float32: cumulative dt*A as a hi/lo pair, then dt.
 hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A,
-                               float *dA_cs, float *dt32, hipStream_t stream);
+                               float *dtcs, hipStream_t stream);
 hipError_t launch_chunk_state(const ScanShape &s, int dtype, const void *x, const void *Bm,
-                              const float *dA_cs, const float *dt32, float *states,
-                              hipStream_t stream);
-hipError_t launch_state_passing(const ScanShape &s, const float *states, const float *dA_cs,
+                              const float *dtcs, float *states, hipStream_t stream);
+hipError_t launch_state_passing(const ScanShape &s, const float *states, const float *dtcs,
                                 const float *init, float *prev, float *final_states,
                                 hipStream_t stream);
 hipError_t launch_chunk_scan(const ScanShape &s, int dtype, const void *x, const void *Bm,
-                             const void *Cm, const float *dA_cs, const float *dt32,
-                             const float *prev, const float *D, void *y, hipStream_t stream);
+                             const void *Cm, const float *dtcs, const float *prev, const float *D,
+                             void *y, hipStream_t stream);
 hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *x, const void *dt,
                        const float *A, const void *Bm, const void *Cm, const float *D, void *y,
                        hipStream_t stream);

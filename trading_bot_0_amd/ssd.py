@@ -24,6 +24,7 @@ from ._build import LIB_PATH
 
 SSD_DTYPE_F32 = 0
 SSD_DTYPE_BF16 = 1
+SSD_DTYPE_BF16_Y32 = 2
 
 EXPORTED_SYMBOLS = (
     "ssd_version",
@@ -82,10 +83,10 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_get_and_reset_last_err.restype = c_void_p
         lib.ssd_workspace_bytes.argtypes = [POINTER(SsdDims), POINTER(c_size_t)]
         lib.ssd_chunk_scan_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, c_size_t, P]
-        lib.ssd_chunk_cumsum_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P]
-        lib.ssd_chunk_state_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P]
+        lib.ssd_chunk_cumsum_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P]
+        lib.ssd_chunk_state_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P]
         lib.ssd_state_passing_fwd.argtypes = [POINTER(SsdDims), P, P, P, P, P, P]
-        lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P]
+        lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
         for name in EXPORTED_SYMBOLS[2:]:
             getattr(lib, name).restype = c_int
@@ -124,6 +125,16 @@ def _dtype_code(t: torch.Tensor) -> int:
     if t.dtype == torch.bfloat16:
         return SSD_DTYPE_BF16
     raise ValueError(f"SSD tensors must be float32 or bfloat16, got {t.dtype}")
+
+
+def _out_code(x: torch.Tensor, y_dtype: Optional[torch.dtype]):
+    """dtype code of a call whose y is `y_dtype` (default: x's dtype)."""
+    code = _dtype_code(x)
+    if y_dtype is None or y_dtype == x.dtype:
+        return code, x.dtype
+    if x.dtype == torch.bfloat16 and y_dtype == torch.float32:
+        return SSD_DTYPE_BF16_Y32, y_dtype
+    raise ValueError(f"SSD y_dtype {y_dtype} is not available for {x.dtype} inputs")
 
 
 def _require(t: torch.Tensor, name: str, shape, dtype) -> None:
@@ -194,16 +205,19 @@ def ssd_chunk_scan(
     workspace: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
     final_out: Optional[torch.Tensor] = None,
+    y_dtype: Optional[torch.dtype] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """SSD chunk-scan forward.  Returns (y [B,L,H,P] in x's dtype, final_states [B,H,P,N] fp32).
 
     `workspace` (uint8, >= workspace_bytes(...)), `out` and `final_out` let a caller that runs
-    under stream capture or in a tight loop avoid any allocation."""
+    under stream capture or in a tight loop avoid any allocation.  `y_dtype=torch.float32` with
+    bf16 inputs writes y without the output rounding."""
     lib = load_library()
     dims = _scan_dims(x, Bm, chunk)
     _validate_scan_inputs(x, dt, A, Bm, Cm, D, initial_states, dims)
-    y = torch.empty_like(x) if out is None else out
-    _require(y, "out", x.shape, x.dtype)
+    code, y_dtype = _out_code(x, y_dtype)
+    y = torch.empty(x.shape, dtype=y_dtype, device=x.device) if out is None else out
+    _require(y, "out", x.shape, y_dtype)
     final = None
     if return_final_states:
         shape = (dims.batch, dims.nheads, dims.headdim, dims.dstate)
@@ -215,7 +229,7 @@ def ssd_chunk_scan(
         workspace = torch.empty(need.value, dtype=torch.uint8, device=x.device)
     elif (not workspace.is_cuda) or workspace.dtype != torch.uint8 or not workspace.is_contiguous():
         raise ValueError("SSD workspace must be a contiguous uint8 GPU tensor")
-    rc = lib.ssd_chunk_scan_fwd(byref(dims), _dtype_code(x), x.data_ptr(), dt.data_ptr(), A.data_ptr(),
+    rc = lib.ssd_chunk_scan_fwd(byref(dims), code, x.data_ptr(), dt.data_ptr(), A.data_ptr(),
                                 Bm.data_ptr(), Cm.data_ptr(), _ptr(D), _ptr(initial_states), y.data_ptr(),
                                 _ptr(final), workspace.data_ptr(), workspace.numel(), _stream_ptr(x))
     _check(lib, rc)
@@ -224,8 +238,8 @@ def ssd_chunk_scan(
 
 # ---- per-stage entry points (testing / profiling) ----------------------------------------
 
-def chunk_cumsum(dt: torch.Tensor, A: torch.Tensor, chunk: int):
-    """Stage 1 -> (dA_cs, dt32), both [B,H,nc,Q] float32."""
+def chunk_cumsum(dt: torch.Tensor, A: torch.Tensor, chunk: int) -> torch.Tensor:
+    """Stage 1 -> dtcs [B,H,nc,3,Q] float32: log2(e) * cumulative dt*A as (hi, lo), then dt."""
     lib = load_library()
     if dt.dim() != 3:
         raise ValueError(f"SSD dt must be rank-3 [batch, seqlen, nheads], got {tuple(dt.shape)}")
@@ -233,62 +247,62 @@ def chunk_cumsum(dt: torch.Tensor, A: torch.Tensor, chunk: int):
     _require(dt, "dt", (Bsz, L, H), dt.dtype)
     _require(A, "A", (H,), torch.float32)
     nc = num_chunks(L, chunk)
-    dA = torch.empty((Bsz, H, nc, chunk), dtype=torch.float32, device=dt.device)
-    d32 = torch.empty_like(dA)
+    dtcs = torch.empty((Bsz, H, nc, 3, chunk), dtype=torch.float32, device=dt.device)
     dims = SsdDims(Bsz, L, H, 32, 64, 1, int(chunk))  # P, N, G do not enter stage 1
     _check(lib, lib.ssd_chunk_cumsum_fwd(byref(dims), _dtype_code(dt), dt.data_ptr(), A.data_ptr(),
-                                         dA.data_ptr(), d32.data_ptr(), _stream_ptr(dt)))
-    return dA, d32
+                                         dtcs.data_ptr(), _stream_ptr(dt)))
+    return dtcs
 
 
-def chunk_state(x, Bm, dA_cs, dt32):
+def _require_dtcs(dtcs, dims: SsdDims):
+    nc = num_chunks(dims.seqlen, dims.chunk)
+    _require(dtcs, "dtcs", (dims.batch, dims.nheads, nc, 3, dims.chunk), torch.float32)
+    return nc
+
+
+def chunk_state(x, Bm, dtcs):
     """Stage 2 -> chunk states [B,nc,H,P,N] float32."""
     lib = load_library()
-    chunk = dA_cs.shape[-1]
-    dims = _scan_dims(x, Bm, chunk)
+    dims = _scan_dims(x, Bm, dtcs.shape[-1])
     _validate_scan_inputs(x, None, None, Bm, None, None, None, dims)
-    nc = num_chunks(dims.seqlen, chunk)
-    _require(dA_cs, "dA_cs", (dims.batch, dims.nheads, nc, chunk), torch.float32)
-    _require(dt32, "dt32", (dims.batch, dims.nheads, nc, chunk), torch.float32)
+    nc = _require_dtcs(dtcs, dims)
     S = torch.empty((dims.batch, nc, dims.nheads, dims.headdim, dims.dstate), dtype=torch.float32, device=x.device)
     _check(lib, lib.ssd_chunk_state_fwd(byref(dims), _dtype_code(x), x.data_ptr(), Bm.data_ptr(),
-                                        dA_cs.data_ptr(), dt32.data_ptr(), S.data_ptr(), _stream_ptr(x)))
+                                        dtcs.data_ptr(), S.data_ptr(), _stream_ptr(x)))
     return S
 
 
-def state_passing(states, dA_cs, initial_states=None, in_place: bool = False):
+def state_passing(states, dtcs, initial_states=None, in_place: bool = False):
     """Stage 3 -> (prev_states [B,nc,H,P,N], final_states [B,H,P,N])."""
     lib = load_library()
     if states.dim() != 5:
-        raise ValueError(f"SSD chunk states must be rank-5 [batch, nchunks, nheads, headdim, dstate]")
+        raise ValueError("SSD chunk states must be rank-5 [batch, nchunks, nheads, headdim, dstate]")
     Bsz, nc, H, P, N = states.shape
-    chunk = dA_cs.shape[-1]
+    chunk = dtcs.shape[-1]
     _require(states, "chunk_states", (Bsz, nc, H, P, N), torch.float32)
-    _require(dA_cs, "dA_cs", (Bsz, H, nc, chunk), torch.float32)
+    _require(dtcs, "dtcs", (Bsz, H, nc, 3, chunk), torch.float32)
     if initial_states is not None:
         _require(initial_states, "initial_states", (Bsz, H, P, N), torch.float32)
     prev = states if in_place else torch.empty_like(states)
     final = torch.empty((Bsz, H, P, N), dtype=torch.float32, device=states.device)
     dims = SsdDims(Bsz, nc * chunk, H, P, N, 1, int(chunk))
-    _check(lib, lib.ssd_state_passing_fwd(byref(dims), states.data_ptr(), dA_cs.data_ptr(), _ptr(initial_states),
+    _check(lib, lib.ssd_state_passing_fwd(byref(dims), states.data_ptr(), dtcs.data_ptr(), _ptr(initial_states),
                                           prev.data_ptr(), final.data_ptr(), _stream_ptr(states)))
     return prev, final
 
 
-def chunk_scan_stage(x, Bm, Cm, dA_cs, dt32, prev_states, D=None):
+def chunk_scan_stage(x, Bm, Cm, dtcs, prev_states, D=None, y_dtype=None):
     """Stage 4 -> y [B,L,H,P]."""
     lib = load_library()
-    chunk = dA_cs.shape[-1]
-    dims = _scan_dims(x, Bm, chunk)
+    dims = _scan_dims(x, Bm, dtcs.shape[-1])
     _validate_scan_inputs(x, None, None, Bm, Cm, D, None, dims)
-    nc = num_chunks(dims.seqlen, chunk)
-    _require(dA_cs, "dA_cs", (dims.batch, dims.nheads, nc, chunk), torch.float32)
-    _require(dt32, "dt32", (dims.batch, dims.nheads, nc, chunk), torch.float32)
+    nc = _require_dtcs(dtcs, dims)
     _require(prev_states, "prev_states", (dims.batch, nc, dims.nheads, dims.headdim, dims.dstate), torch.float32)
-    y = torch.empty_like(x)
-    _check(lib, lib.ssd_chunk_scan_stage_fwd(byref(dims), _dtype_code(x), x.data_ptr(), Bm.data_ptr(),
-                                             Cm.data_ptr(), dA_cs.data_ptr(), dt32.data_ptr(),
-                                             prev_states.data_ptr(), _ptr(D), y.data_ptr(), _stream_ptr(x)))
+    code, y_dtype = _out_code(x, y_dtype)
+    y = torch.empty(x.shape, dtype=y_dtype, device=x.device)
+    _check(lib, lib.ssd_chunk_scan_stage_fwd(byref(dims), code, x.data_ptr(), Bm.data_ptr(), Cm.data_ptr(),
+                                             dtcs.data_ptr(), prev_states.data_ptr(), _ptr(D), y.data_ptr(),
+                                             _stream_ptr(x)))
     return y
 
 
@@ -301,8 +315,10 @@ def ssd_step(
     Cm: torch.Tensor,
     D: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
+    y_dtype: Optional[torch.dtype] = None,
 ) -> torch.Tensor:
-    """One recurrent update.  `state` [B,H,P,N] fp32 is advanced in place; returns y [B,H,P]."""
+    """One recurrent update.  `state` [B,H,P,N] fp32 is advanced in place; returns y [B,H,P]
+    (x's dtype, or float32 from bf16 inputs with y_dtype=torch.float32)."""
     lib = load_library()
     if state.dim() != 4:
         raise ValueError(f"SSD state must be rank-4 [batch, nheads, headdim, dstate], got {tuple(state.shape)}")
@@ -320,10 +336,11 @@ def ssd_step(
     _require(Cm, "C", (Bsz, G, N), dtype)
     if D is not None:
         _require(D, "D", (H,), torch.float32)
-    y = torch.empty_like(x) if out is None else out
-    _require(y, "out", (Bsz, H, P), dtype)
+    code, y_dtype = _out_code(x, y_dtype)
+    y = torch.empty((Bsz, H, P), dtype=y_dtype, device=x.device) if out is None else out
+    _require(y, "out", (Bsz, H, P), y_dtype)
     dims = SsdStepDims(Bsz, H, P, N, G)
-    _check(lib, lib.ssd_step_fwd(byref(dims), _dtype_code(x), state.data_ptr(), x.data_ptr(), dt.data_ptr(),
+    _check(lib, lib.ssd_step_fwd(byref(dims), code, state.data_ptr(), x.data_ptr(), dt.data_ptr(),
                                  A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), _ptr(D), y.data_ptr(),
                                  _stream_ptr(x)))
     return y

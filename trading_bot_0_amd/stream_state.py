@@ -53,22 +53,23 @@ class SsdStreamState:
     def clone(self) -> "SsdStreamState":
         return SsdStreamState(self.state.clone(), self.initialized)
 
-    def init_from_prefix(self, x, dt, A, Bm, Cm, D=None, chunk: int = 128, workspace=None) -> torch.Tensor:
+    def init_from_prefix(self, x, dt, A, Bm, Cm, D=None, chunk: int = 128, workspace=None,
+                         y_dtype=None) -> torch.Tensor:
         """Scan a full prefix [B,L,...] and keep its final state (cf. init_from_full_on_device,
         live.rs:322-360).  Continues from the current state when already initialised.  Returns y."""
         if x.shape[0] != self.batch:
             raise ValueError(f"stream state batch size mismatch: state has {self.batch}, input has {x.shape[0]}")
         init = self.state if self.initialized else None
         y, _ = ssd.ssd_chunk_scan(x, dt, A, Bm, Cm, D, chunk=chunk, initial_states=init,
-                                  workspace=workspace, final_out=self.state)
+                                  workspace=workspace, final_out=self.state, y_dtype=y_dtype)
         self.initialized = True
         return y
 
-    def step(self, x, dt, A, Bm, Cm, D=None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def step(self, x, dt, A, Bm, Cm, D=None, out: Optional[torch.Tensor] = None, y_dtype=None) -> torch.Tensor:
         """Advance every stream by one timestep (cf. step_uniform_stream_state_on_device,
         live.rs:228-244).  x [B,H,P], dt [B,H], Bm/Cm [B,G,N]; returns y [B,H,P]."""
         if x.shape[0] != self.batch:
             raise ValueError(f"stream state batch size mismatch: state has {self.batch}, input has {x.shape[0]}")
-        y = ssd.ssd_step(self.state, x, dt, A, Bm, Cm, D, out=out)
+        y = ssd.ssd_step(self.state, x, dt, A, Bm, Cm, D, out=out, y_dtype=y_dtype)
         self.initialized = True
         return y
