@@ -27,11 +27,12 @@
  *   A, D        [nheads]                              float32; A < 0; D may be NULL
  *   Bm, Cm      [batch, seqlen, ngroups, dstate]      dtype; head h uses group h/(nheads/ngroups)
  *   states      [batch, nheads, headdim, dstate]      float32 (initial, final, streaming)
- *   dtcs        [batch, nheads, nchunks, 3, chunk]    float32 (stage 1 output): rows 0 and 1 are
+ *   dtcs        [batch, nheads, nchunks, 4, chunk]    float32 (stage 1 output): rows 0 and 1 are
  *               log2(e) times the per-chunk inclusive cumulative sum of dt*A, as an unevaluated
  *               pair hi + lo (later stages only use differences of it, which the pair keeps
  *               exact to the difference's own rounding, and turn them into decays with one
- *               exp2), row 2 is dt
+ *               exp2), row 2 is dt, row 3 is the decay from each step to the end of its chunk
+ *               times dt (the weight stage 2 applies to x)
  *   chunk states[batch, nchunks, nheads, headdim, dstate] float32 (stages 2-4)
  * Recurrence: h_t = exp(dt_t A_h) h_{t-1} + dt_t x_t (outer) B_t ; y_t = h_t . C_t + D_h x_t.
  *

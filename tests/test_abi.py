@@ -47,10 +47,10 @@ def test_workspace_bytes_formula(lib):
     out = c_size_t(0)
     assert lib.ssd_workspace_bytes(byref(dims()), byref(out)) == 0
     B, H, nc, Q, P, N = 2, 4, 2, 128, 32, 64
-    assert out.value == 3 * B * H * nc * Q * 4 + B * nc * H * P * N * 4
+    assert out.value == 4 * B * H * nc * Q * 4 + B * nc * H * P * N * 4
     # ragged seqlen rounds the chunk count up
     assert lib.ssd_workspace_bytes(byref(dims(seqlen=257)), byref(out)) == 0
-    assert out.value == 3 * B * H * 3 * Q * 4 + B * 3 * H * P * N * 4
+    assert out.value == 4 * B * H * 3 * Q * 4 + B * 3 * H * P * N * 4
 
 
 @pytest.mark.parametrize("kw,code,needle", [

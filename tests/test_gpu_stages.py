@@ -49,12 +49,13 @@ def f32dev(a):
 
 
 def dtcs_dev(mids):
-    """The oracle's float64 cumulative sum and dt in the stage-1 output layout [B,H,nc,3,Q]:
-    log2(e) * cumsum as an unevaluated float32 pair hi + lo, then dt."""
+    """The oracle's float64 cumulative sum and dt in the stage-1 output layout [B,H,nc,4,Q]:
+    log2(e) * cumsum as an unevaluated float32 pair hi + lo, dt, and the stage-2 weight."""
     al = mids["dA_cs"] * LOG2E
     hi = al.astype(np.float32)
     lo = (al - hi.astype(np.float64)).astype(np.float32)
-    return f32dev(np.stack([hi, lo, mids["dt_c"].astype(np.float32)], axis=3))
+    w = np.exp(mids["dA_cs"][..., -1:] - mids["dA_cs"]) * mids["dt_c"]
+    return f32dev(np.stack([hi, lo, mids["dt_c"].astype(np.float32), w.astype(np.float32)], axis=3))
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
@@ -70,6 +71,8 @@ def test_chunk_cumsum(shape, dtype):
     assert np.max(np.abs((hi + lo) - al)) <= 1e-11 * max(1.0, np.max(np.abs(al)))
     assert np.max(np.abs(hi - al)) <= 2.0 ** -23 * max(1.0, np.max(np.abs(al)))   # hi alone: a rounded float
     assert np.array_equal(d32, mids["dt_c"]), "dt row is an exact copy"
+    w = np.exp(mids["dA_cs"][..., -1:] - mids["dA_cs"]) * mids["dt_c"]
+    assert np.max(np.abs(got[:, :, :, 3] - w)) <= 1e-6 * np.max(w), "stage-2 weight row"
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])

@@ -96,7 +96,7 @@ struct Workspace {
 
 Workspace carve(const ssd::ScanShape &s) {
     Workspace w;
-    const size_t dtcs = (size_t)s.B * s.H * s.nc * 3 * s.Q * sizeof(float);
+    const size_t dtcs = (size_t)s.B * s.H * s.nc * 4 * s.Q * sizeof(float);
     const size_t st = (size_t)s.B * s.nc * s.H * s.P * s.N * sizeof(float);
     w.dtcs_off = 0;
     w.st_off = align_up(dtcs, 256);

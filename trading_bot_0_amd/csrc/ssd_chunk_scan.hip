@@ -1,0 +1,356 @@
+// Stage 4 of the SSD forward for gfx950: chunk_scan.  One tile per (b,c,h); each wave owns 32 output columns
+// l in [32*lb, 32*lb+32) and computes the TRANSPOSED output tile yT[p,l]:
+//   yT  = exp2(alpha[l]) * (Hc [P x N] . C^T [N x l])                   state readout
+//       + sum over s-blocks sb <= lb of  xT [P x s] . M^T [s x l]        intra-chunk
+//   M^T[s,l] = (B[s,:] . C[l,:]) * exp2(alpha[l] - alpha[s]) * dt[s]  for s <= l, else 0
+// Computing the transpose makes the 32x32 accumulator of B.C^T directly usable as the B
+// operand of the second MFMA (its lane already holds column l and 16 rows s), so the masked
+// score matrix never leaves registers; the A operand xT is read from LDS in the matching K
+// order.  C fragments for the wave's 32 columns stay in registers for both products.
+//
+// Decay factors.  Only the diagonal block (sb == lb) needs a mask and one exp2 per element
+// (mask before exp2: no inf*0).  Below the diagonal the factor separates through the first
+// row m = 32*lb of the column block, exp2(alpha[l]-alpha[s]) = exp2(alpha[l]-alpha[m]) *
+// exp2(alpha[m]-alpha[s]) with both exponents <= 0: one value per lane times a per-row table
+// (dt folded in) that the workgroup builds once in LDS.
+//
+// In bf16 mode the two operands this kernel manufactures in fp32 -- M and the entering state
+// Hc -- are fed to the MFMA as hi + lo bf16 pairs; x, B and C enter exactly as given.
+// TO is the element type of y (T, or float for bf16 inputs with float32 output).
+// The column-block index is rotated with the workgroup id so that the wave with the most
+// s-blocks does not always sit on the same SIMD.
+//
+// Persistent and software-pipelined like stage 2: the next tile's B, x, entering state, C and
+// alpha rows sit in registers while the current tile's MFMAs run.
+#include "ssd_device.h"
+
+namespace ssd {
+
+template <typename T, typename TO, int PB, int NK>  // Ppad = 32*PB >= P, N = 16*NK
+__global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict__ x, const T *__restrict__ Bm,
+                                                            const T *__restrict__ Cm,
+                                                            const float *__restrict__ dtcs,
+                                                            const float *__restrict__ prev,
+                                                            const float *__restrict__ D, TO *__restrict__ y,
+                                                            ScanShape s) {
+    constexpr int VEC = Vec16<T>::N;
+    constexpr int PARTS = Split<T>::PARTS;
+    constexpr int N = NK * 16;
+    constexpr int Ppad = PB * 32;
+    constexpr int ldb = N + lds_pad<T>();
+    // Load mapping over the 2Q threads: a thread owns one 16-byte column slot of rows l0, l0+rpp, ...
+    constexpr int bcpr = N / VEC, xcpr = Ppad / VEC;
+    constexpr int UB = bcpr / 2, UX = xcpr / 2;   // passes = Q / (2Q / slots per row); both slot counts are even
+    constexpr int hcpr = N / 4;
+    constexpr int UH = 2;                    // entering-state float4 loads per thread held across tiles
+    constexpr bool kPrefetchC = NK <= 4;     // wide states: C is fetched at the top of the tile instead
+    using XT = RowMajorTile<Ppad>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int Q = s.Q;
+    const int ldx = Q + lds_pad<T>();        // float mode: xs is transposed [Ppad][ldx]
+    const int nblk = Q / 32;
+    float *al_s = reinterpret_cast<float *>(smem);  // [3][Q]: alpha hi, alpha lo, dt
+    float *tab = al_s + 3 * Q;                      // [nblk][Q]: exp2(alpha[32k]-alpha[s])*dt[s], s < 32k
+    T *Bs = reinterpret_cast<T *>(tab + nblk * Q);  // [Q][ldb]
+    T *Hs = Bs + Q * ldb;                           // [PARTS][Ppad][ldb]
+    T *xs = Hs + PARTS * Ppad * ldb;                // bf16: [Q][Ppad] row-major; float: [Ppad][ldx]
+    const float *ah_s = al_s, *alo_s = al_s + Q, *dt_s = al_s + 2 * Q;
+
+    const int tid = threadIdx.x, nthr = 2 * Q;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, half = lane >> 5;
+    const int xrpp = nthr / xcpr, brpp = nthr / bcpr;
+    const int xl0 = tid / xcpr, xch = tid % xcpr, bl0 = tid / bcpr, bch = tid % bcpr;
+    const bool xslot = xch * VEC < s.P;      // column slots past P stay zero
+    const int xoff0 = xl0 * s.H * s.P + xch * VEC, xstep = xrpp * s.H * s.P;   // elements
+    const int boff0 = bl0 * s.G * N + bch * VEC, bstep = brpp * s.G * N;
+    const int htotal = s.P * hcpr;
+    const bool p_full = s.P == Ppad;
+
+    // ---- registers holding the next tile's inputs ----
+    float a3[2];
+    Vec16<T> bv[UB], xv[UX];
+    float4 hv[UH];
+    Frag<T> Cn[kPrefetchC ? NK : 1];
+
+    // C fragments straight from global: column l = 32*lb + r of the tile, K = n
+    auto load_c = [&](const Tile &t, int logical, int rows, Frag<T> *dst) {
+        const int l = ((wave + logical) % nblk) * 32 + r;
+        const T *crow = Cm + (((size_t)t.b * s.L + t.t0 + l) * s.G + t.g) * N + half * 8;
+        if (rows == Q) {
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) dst[kk] = load_frag(crow + kk * 16);
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) dst[kk] = (l < rows) ? load_frag(crow + kk * 16) : zero_frag<T>();
+        }
+    };
+    auto prefetch = [&](int logical) {
+        const Tile t = decode_tile(logical, s);
+        const float *arow = dtcs + ((((size_t)t.b * s.H + t.h) * s.nc + t.c) * 4) * Q;
+        a3[0] = (tid < 3 * Q) ? arow[tid] : 0.f;
+        a3[1] = (tid + nthr < 3 * Q) ? arow[tid + nthr] : 0.f;
+        const int rows = min(Q, s.L - t.t0);  // valid rows of a ragged last chunk
+        const T *bb = Bm + (((size_t)t.b * s.L + t.t0) * s.G + t.g) * N;
+        const T *xb = x + (((size_t)t.b * s.L + t.t0) * s.H + t.h) * s.P;
+        if (rows == Q) {
+#pragma unroll
+            for (int u = 0; u < UB; ++u)
+                bv[u] = load_vec16(bb + boff0 + u * bstep);
+#pragma unroll
+            for (int u = 0; u < UX; ++u) xv[u] = xslot ? load_vec16(xb + xoff0 + u * xstep) : zero_vec16<T>();
+        } else {
+#pragma unroll
+            for (int u = 0; u < UB; ++u)
+                bv[u] = (bl0 + u * brpp < rows) ? load_vec16(bb + boff0 + u * bstep) : zero_vec16<T>();
+#pragma unroll
+            for (int u = 0; u < UX; ++u)
+                xv[u] = (xslot && xl0 + u * xrpp < rows) ? load_vec16(xb + xoff0 + u * xstep) : zero_vec16<T>();
+        }
+        const float *hp = prev + ((((size_t)t.b * s.nc + t.c) * s.H + t.h) * s.P) * N;
+#pragma unroll
+        for (int u = 0; u < UH; ++u) {
+            const int idx = u * nthr + tid;
+            hv[u] = (idx < htotal) ? *reinterpret_cast<const float4 *>(hp + idx * 4) : make_float4(0, 0, 0, 0);
+        }
+        if (kPrefetchC) load_c(t, logical, rows, Cn);
+    };
+    auto put_state = [&](int idx, const float4 &h4) {
+        const int p = idx / hcpr, n4 = idx % hcpr;
+        const float v[4] = {h4.x, h4.y, h4.z, h4.w};
+        T hi[4], lo[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) Split<T>::split(v[i], hi[i], lo[i]);
+        T *dsth = Hs + p * ldb + n4 * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dsth[i] = hi[i];
+        if (PARTS == 2) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dsth[Ppad * ldb + i] = lo[i];
+        }
+    };
+
+    TileSched sched(s.B * s.nc * s.H);
+    if (sched.valid()) prefetch(sched.logical());
+    // zero the state rows no tile write covers (only when P is not a multiple of 32)
+    for (int idx = tid; idx < PARTS * (Ppad - s.P) * ldb; idx += nthr) {
+        const int part = idx / ((Ppad - s.P) * ldb), rem = idx % ((Ppad - s.P) * ldb);
+        Hs[(part * Ppad + s.P) * ldb + rem] = (T)0.f;
+    }
+
+    for (; sched.valid(); sched.advance()) {
+        const int logical = sched.logical();
+        const Tile t = decode_tile(logical, s);
+        const int rows = min(Q, s.L - t.t0);
+        const int lb = (wave + logical) % nblk;  // this wave's column block
+        const int l = lb * 32 + r;
+        Frag<T> Cf[NK];
+        if constexpr (kPrefetchC) {
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) Cf[kk] = Cn[kk];
+        } else {
+            load_c(t, logical, rows, Cf);
+        }
+
+        __syncthreads();  // the previous tile's LDS reads are done (and the zero fill is visible)
+        // ---- registers -> LDS ----
+        if (tid < 3 * Q) al_s[tid] = a3[0];
+        if (tid + nthr < 3 * Q) al_s[tid + nthr] = a3[1];
+#pragma unroll
+        for (int u = 0; u < UB; ++u)
+            *reinterpret_cast<uint4 *>(Bs + (bl0 + u * brpp) * ldb + bch * VEC) = bv[u].u;
+#pragma unroll
+        for (int u = 0; u < UX; ++u) {
+            const int sr = xl0 + u * xrpp;
+            if constexpr (is_bf16<T>) {
+                *reinterpret_cast<uint4 *>(xs + XT::off(sr, xch * VEC)) = xv[u].u;
+            } else {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) xs[(xch * VEC + i) * ldx + sr] = xv[u].e[i];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UH; ++u) {
+            const int idx = u * nthr + tid;
+            if (idx < htotal) put_state(idx, hv[u]);
+        }
+        {   // the part of the entering state the register batch does not hold (small chunk, large state)
+            const float *hp = prev + ((((size_t)t.b * s.nc + t.c) * s.H + t.h) * s.P) * N;
+            for (int idx = UH * nthr + tid; idx < htotal; idx += nthr)
+                put_state(idx, *reinterpret_cast<const float4 *>(hp + idx * 4));
+        }
+        __syncthreads();  // alpha and dt are visible
+        // decay table rows k = 1..nblk-1 (row 0 is never read)
+        for (int idx = tid; idx < nblk * Q; idx += nthr) {
+            const int k = idx / Q, sr = idx % Q;
+            if (k > 0 && sr < 32 * k) {
+                const float d = alpha_diff(ah_s[32 * k], alo_s[32 * k], ah_s[sr], alo_s[sr]);
+                tab[idx] = exp2_hw(fminf(d, 0.f)) * dt_s[sr];
+            }
+        }
+        if (sched.has_next()) prefetch(sched.next_logical());
+        __syncthreads();
+
+        const float al_hi = ah_s[l], al_lo = alo_s[l];
+        f32x16 accY[PB];
+        // state readout, scaled per output column by exp2(alpha[l]) (alpha <= 0)
+        {
+            const float el = exp2_hw(al_hi + al_lo);
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+                f32x16 a = {0};
+                const T *hrow = Hs + (pb * 32 + r) * ldb + half * 8;
+#pragma unroll
+                for (int kk = 0; kk < NK; ++kk) {
+                    a = mma32(load_frag(hrow + kk * 16), Cf[kk], a);
+                    if (PARTS == 2) a = mma32(load_frag(hrow + Ppad * ldb + kk * 16), Cf[kk], a);
+                }
+                accY[pb] = a * el;
+            }
+        }
+        // intra-chunk: s-blocks at or below this wave's column block (causal)
+        const float lane_dec = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah_s[32 * lb], alo_s[32 * lb]), 0.f));
+        const float *tab_row = tab + lb * Q;
+        for (int sb = 0; sb <= lb; ++sb) {
+            f32x16 sc = {0};
+            const T *brow = Bs + (sb * 32 + r) * ldb + half * 8;
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) sc = mma32(load_frag(brow + kk * 16), Cf[kk], sc);
+            Frag<T> mh[2], ml[2];
+            if (sb < lb) {
+#pragma unroll
+                for (int vg = 0; vg < 4; ++vg) {
+                    const int s0 = sb * 32 + 8 * vg + 4 * half;
+                    const float4 t4 = *reinterpret_cast<const float4 *>(tab_row + s0);
+                    const float tv[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int v = vg * 4 + i;
+                        T hi, lo;
+                        Split<T>::split(sc[v] * tv[i] * lane_dec, hi, lo);
+                        mh[v / 8].v[v % 8] = hi;
+                        if (PARTS == 2) ml[v / 8].v[v % 8] = lo;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int vg = 0; vg < 4; ++vg) {
+                    const int s0 = sb * 32 + 8 * vg + 4 * half;
+                    const float4 ah4 = *reinterpret_cast<const float4 *>(ah_s + s0);
+                    const float4 al4 = *reinterpret_cast<const float4 *>(alo_s + s0);
+                    const float4 dt4 = *reinterpret_cast<const float4 *>(dt_s + s0);
+                    const float ahv[4] = {ah4.x, ah4.y, ah4.z, ah4.w};
+                    const float alv[4] = {al4.x, al4.y, al4.z, al4.w};
+                    const float dtv[4] = {dt4.x, dt4.y, dt4.z, dt4.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int v = vg * 4 + i;
+                        const float arg = alpha_diff(al_hi, al_lo, ahv[i], alv[i]);
+                        const float w = (s0 + i <= l) ? exp2_hw(fminf(arg, 0.f)) * dtv[i] * sc[v] : 0.f;
+                        T hi, lo;
+                        Split<T>::split(w, hi, lo);
+                        mh[v / 8].v[v % 8] = hi;
+                        if (PARTS == 2) ml[v / 8].v[v % 8] = lo;
+                    }
+                }
+            }
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    // K order of mh[j]: rows s = sb*32 + 16j + 4*half + {0..3} and the same + 8
+                    Frag<T> xf;
+                    if constexpr (is_bf16<T>) {
+                        xf = XT::frag(xs, sb * 32 + 16 * j + 4 * half, 8, pb * 32, lane);
+                    } else {
+                        xf = load_frag_split(xs + (pb * 32 + r) * ldx + sb * 32 + 16 * j + 4 * half);
+                    }
+                    accY[pb] = mma32(xf, mh[j], accY[pb]);
+                    if (PARTS == 2) accY[pb] = mma32(xf, ml[j], accY[pb]);
+                }
+            }
+        }
+        // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]
+        if (l < rows) {
+            const float dh = D ? D[t.h] : 0.f;
+            TO *yrow = y + (((size_t)t.b * s.L + t.t0 + l) * s.H + t.h) * s.P + 4 * half;
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+#pragma unroll
+                for (int vg = 0; vg < 4; ++vg) {
+                    const int p0 = pb * 32 + 8 * vg + 4 * half;
+                    if (p_full || p0 < s.P) {
+                        float xl[4];
+                        if constexpr (is_bf16<T>) {
+                            const bf16x4 x4 = *reinterpret_cast<const bf16x4 *>(xs + XT::off(l, p0));
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) xl[i] = (float)x4[i];
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) xl[i] = xs[(p0 + i) * ldx + l];
+                        }
+                        store4<TO>(yrow + pb * 32 + 8 * vg, accY[pb][vg * 4 + 0] + dh * xl[0],
+                                   accY[pb][vg * 4 + 1] + dh * xl[1], accY[pb][vg * 4 + 2] + dh * xl[2],
+                                   accY[pb][vg * 4 + 3] + dh * xl[3]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Launchers
+// ------------------------------------------------------------------------------------------
+size_t chunk_scan_lds_bytes(const ScanShape &s, int eb) {
+    const size_t Ppad = (s.P + 31) & ~31;
+    const size_t ldb = s.N + 16 / eb, parts = eb == 2 ? 2 : 1;
+    const size_t xs = eb == 2 ? (size_t)s.Q * Ppad : Ppad * (size_t)(s.Q + 4);
+    return (size_t)s.Q * 12 + (size_t)(s.Q / 32) * s.Q * 4 + ((size_t)s.Q * ldb + parts * Ppad * ldb + xs) * eb;
+}
+
+template <typename T, typename TO, int PB, int NK>
+static hipError_t scan_launch(const ScanShape &s, const void *x, const void *Bm, const void *Cm,
+                              const float *dtcs, const float *prev, const float *D, void *y, hipStream_t st) {
+    const size_t lds = chunk_scan_lds_bytes(s, sizeof(T));
+    hipError_t e = allow_lds(chunk_scan_kernel<T, TO, PB, NK>, lds);
+    if (e != hipSuccess) return e;
+    int grid = 1;
+    e = persistent_grid(chunk_scan_kernel<T, TO, PB, NK>, 64 * (s.Q / 32), lds, s.B * s.nc * s.H, &grid);
+    if (e != hipSuccess) return e;
+    chunk_scan_kernel<T, TO, PB, NK><<<dim3(grid), dim3(64 * (s.Q / 32)), lds, st>>>(
+        static_cast<const T *>(x), static_cast<const T *>(Bm), static_cast<const T *>(Cm), dtcs, prev, D,
+        static_cast<TO *>(y), s);
+    return hipGetLastError();
+}
+
+template <typename T, typename TO, int PB>
+static hipError_t scan_dispatch_n(const ScanShape &s, const void *x, const void *Bm, const void *Cm,
+                                  const float *dtcs, const float *prev, const float *D, void *y,
+                                  hipStream_t st) {
+    switch (s.N) {
+        case 16: return scan_launch<T, TO, PB, 1>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 32: return scan_launch<T, TO, PB, 2>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 64: return scan_launch<T, TO, PB, 4>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 128: return scan_launch<T, TO, PB, 8>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <typename T, typename TO>
+static hipError_t scan_dispatch(const ScanShape &s, const void *x, const void *Bm, const void *Cm,
+                                const float *dtcs, const float *prev, const float *D, void *y, hipStream_t st) {
+    return (s.P <= 32) ? scan_dispatch_n<T, TO, 1>(s, x, Bm, Cm, dtcs, prev, D, y, st)
+                       : scan_dispatch_n<T, TO, 2>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+}
+
+hipError_t launch_chunk_scan(const ScanShape &s, int dtype, const void *x, const void *Bm, const void *Cm,
+                             const float *dtcs, const float *prev, const float *D, void *y, hipStream_t st) {
+    switch (dtype) {
+        case 0: return scan_dispatch<float, float>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 1: return scan_dispatch<__bf16, __bf16>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        default: return scan_dispatch<__bf16, float>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+    }
+}
+
+}  // namespace ssd

@@ -1,0 +1,267 @@
+// Device-side building blocks shared by the SSD kernels (gfx950 only): MFMA fragments, 16-byte
+// vectors, hi/lo bf16 splitting, row-major LDS tiles read through the transpose load, the
+// XCD-aware persistent tile schedule.
+//
+// Notation: b batch, c chunk, l/s position inside a chunk (0..Q-1), h head, g group,
+// p head-dim index, n state index, t = c*Q + l absolute timestep.
+// alpha[l] = log2(e) * sum_{i<=l} dt[i]*A is the per-chunk cumulative log2-decay, so every
+// decay factor is one v_exp_f32:  exp(sum_{s<i<=l} dt_i A) = exp2(alpha[l] - alpha[s]).
+//
+// MFMA operand convention used throughout (v_mfma_f32_32x32x16_bf16 and, in float mode,
+// eight v_mfma_f32_32x32x2_f32): a lane with r = lane%32 and half = lane/32 supplies, for the
+// A operand, 8 K-consecutive elements of row r starting at k = 8*half; for the B operand the
+// same for column r.  Accumulator register v of that lane is element
+// (row 8*(v/4) + 4*half + v%4, column r).
+#pragma once
+#include <type_traits>
+
+#include "ssd_launch.h"
+
+namespace ssd {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+template <typename T> constexpr bool is_bf16 = std::is_same<T, __bf16>::value;
+
+// ------------------------------------------------------------------------------------------
+// Fragments and 16-byte vectors
+// ------------------------------------------------------------------------------------------
+template <typename T> struct Frag;
+template <> struct Frag<__bf16> {
+    bf16x8 v;
+};
+template <> struct Frag<float> {
+    float v[8];
+};
+
+__device__ inline f32x16 mma32(const Frag<__bf16> &a, const Frag<__bf16> &b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
+}
+// Float mode: K index 8*half + i is fed to MFMA number i as its k = half; the K order is a
+// permutation of the bf16 one, which a sum does not see.
+__device__ inline f32x16 mma32(const Frag<float> &a, const Frag<float> &b, f32x16 c) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[i], b.v[i], c, 0, 0, 0);
+    return c;
+}
+
+template <typename T> struct Vec16;  // one 16-byte global/LDS transaction
+template <> struct Vec16<__bf16> {
+    static constexpr int N = 8;
+    union {
+        uint4 u;
+        __bf16 e[8];
+    };
+};
+template <> struct Vec16<float> {
+    static constexpr int N = 4;
+    union {
+        uint4 u;
+        float e[4];
+    };
+};
+
+template <typename T> __device__ inline Vec16<T> load_vec16(const T *p) {
+    Vec16<T> r;
+    r.u = *reinterpret_cast<const uint4 *>(p);
+    return r;
+}
+template <typename T> __device__ inline Vec16<T> zero_vec16() {
+    Vec16<T> r;
+    r.u = make_uint4(0, 0, 0, 0);
+    return r;
+}
+template <typename T> __device__ inline Frag<T> zero_frag() {
+    Frag<T> f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f.v[i] = (T)0.f;
+    return f;
+}
+
+// 8 consecutive elements starting at p (16-byte aligned).
+__device__ inline Frag<__bf16> load_frag(const __bf16 *p) {
+    Frag<__bf16> f;
+    f.v = *reinterpret_cast<const bf16x8 *>(p);
+    return f;
+}
+__device__ inline Frag<float> load_frag(const float *p) {
+    Frag<float> f;
+    const float4 a = *reinterpret_cast<const float4 *>(p);
+    const float4 b = *reinterpret_cast<const float4 *>(p + 4);
+    f.v[0] = a.x; f.v[1] = a.y; f.v[2] = a.z; f.v[3] = a.w;
+    f.v[4] = b.x; f.v[5] = b.y; f.v[6] = b.z; f.v[7] = b.w;
+    return f;
+}
+// Elements p[0..3] and p[8..11]: the K order in which an accumulator tile, reused directly as
+// a B operand, presents its rows (see chunk_scan_kernel).  Float mode only; bf16 uses LDS
+// transpose reads.
+__device__ inline Frag<float> load_frag_split(const float *p) {
+    Frag<float> f;
+    const float4 a = *reinterpret_cast<const float4 *>(p);
+    const float4 b = *reinterpret_cast<const float4 *>(p + 8);
+    f.v[0] = a.x; f.v[1] = a.y; f.v[2] = a.z; f.v[3] = a.w;
+    f.v[4] = b.x; f.v[5] = b.y; f.v[6] = b.z; f.v[7] = b.w;
+    return f;
+}
+
+template <typename T> __device__ inline void store4(T *p, float a, float b, float c, float d);
+template <> __device__ inline void store4<float>(float *p, float a, float b, float c, float d) {
+    *reinterpret_cast<float4 *>(p) = make_float4(a, b, c, d);
+}
+template <> __device__ inline void store4<__bf16>(__bf16 *p, float a, float b, float c, float d) {
+    bf16x4 v;
+    v[0] = (__bf16)a; v[1] = (__bf16)b; v[2] = (__bf16)c; v[3] = (__bf16)d;
+    *reinterpret_cast<bf16x4 *>(p) = v;
+}
+
+template <typename T> constexpr int lds_pad() { return 16 / (int)sizeof(T); }
+
+// exp2 as the single hardware instruction (v_exp_f32, ~1 ulp); arguments here are <= 0 and
+// results below 2^-126 flush to zero, which is the wanted limit of a vanished decay.
+__device__ inline float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
+// alpha difference from hi/lo pairs: good to the rounding of the difference itself
+__device__ inline float alpha_diff(float hi_a, float lo_a, float hi_b, float lo_b) {
+    return (hi_a - hi_b) + (lo_a - lo_b);
+}
+
+// hi/lo split of an fp32 value into two bf16 (relative error 2^-17 instead of 2^-9); in float
+// mode there is nothing to split.
+template <typename T> struct Split;
+template <> struct Split<__bf16> {
+    static constexpr int PARTS = 2;
+    static __device__ inline void split(float v, __bf16 &hi, __bf16 &lo) {
+        hi = (__bf16)v;
+        lo = (__bf16)(v - (float)hi);
+    }
+};
+template <> struct Split<float> {
+    static constexpr int PARTS = 1;
+    static __device__ inline void split(float v, float &hi, float &lo) {
+        hi = v;
+        lo = 0.f;
+    }
+};
+
+// ------------------------------------------------------------------------------------------
+// Row-major bf16 tiles in LDS read through the gfx950 transpose load.
+//
+// x and B arrive with the MFMA K axis (time) as their slow axis, but an MFMA lane needs K
+// consecutive for its row/column.  ds_read_b64_tr_b16 does that transposition inside the LDS
+// read: within each block of 16 lanes, lane 4a+b supplies the address of 4 consecutive
+// 16-bit elements of tile row (k0+a), columns c0+4b..c0+4b+3, and lane i receives the 4
+// elements tile[k0+0..3][c0+i] (measured on the device; one such read is half of an 8-deep
+// MFMA operand).  Tiles are therefore stored exactly as they come from memory, with 16-byte
+// vector writes, instead of being scattered element by element.
+//
+// COLS (elements per row) is 32, 64 or 128, i.e. 1, 2 or 4 granules of 64 bytes.  A transpose
+// read touches 4 consecutive rows x 64 bytes per 32 lanes; the granule index is XOR-swizzled
+// with the row so those four pieces fall into the four quarters of the 64 banks.
+// ------------------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_gcc;
+#define SSD_LDS_AS __attribute__((address_space(3)))
+
+template <int COLS> struct RowMajorTile {
+    static constexpr int GR = COLS / 32;
+    static __device__ inline int swz(int row) { return GR == 1 ? 0 : (GR == 2 ? ((row >> 1) & 1) : (row & 3)); }
+    // element offset of (row, col); col..col+7 stay inside one granule when col % 8 == 0
+    static __device__ inline int off(int row, int col) {
+        return row * COLS + ((((col >> 5) ^ swz(row)) << 5) | (col & 31));
+    }
+    // this lane's 4 elements tile[k0 + 0..3][c0 + lane%16 + 16*((lane/16)%2)] -- with k0 already
+    // including the lane half's K offset, that is K-consecutive data for operand row c0 + lane%32
+    static __device__ inline bf16x4 tr4(const __bf16 *tile, int k0, int c0, int lane) {
+        const int q = lane >> 4, a = (lane >> 2) & 3, b = lane & 3;
+        const __bf16 *src = tile + off(k0 + a, c0 + 16 * (q & 1) + 4 * b);
+        const bf16x4_gcc v = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SSD_LDS_AS bf16x4_gcc *)(src));
+        return __builtin_bit_cast(bf16x4, v);
+    }
+    // operand fragment: rows k0..k0+3 then k0+gap..k0+gap+3 (gap 4 = 8 consecutive K values)
+    static __device__ inline Frag<__bf16> frag(const __bf16 *tile, int k0, int gap, int c0, int lane) {
+        Frag<__bf16> f;
+        const bf16x4 lo = tr4(tile, k0, c0, lane), hi = tr4(tile, k0 + gap, c0, lane);
+        f.v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return f;
+    }
+};
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with a private L2.  Re-number them so
+// that consecutive logical ids (the heads of one (b,c) tile, which share B and C and sit in
+// the same cache lines of x) land on the same XCD at nearly the same time.
+__device__ inline int xcd_remap(int bid, int total) {
+    return (total % 8 == 0) ? (bid % 8) * (total / 8) + bid / 8 : bid;
+}
+
+// ------------------------------------------------------------------------------------------
+// Persistent tile schedule of stages 2 and 4.  The grid holds as many workgroups as the chip
+// keeps resident; each walks a fixed list of (b,c,h) tiles and fetches the next tile's inputs
+// into registers while it computes the current one, so HBM requests stay in flight through
+// the MFMA phase (with one tile per workgroup and ~4 workgroups per CU the chip alternated
+// between loading and computing and sat at a third of the HBM rate).
+// Workgroup j runs on XCD j%8; the list is cut so that at any moment the workgroups of one
+// XCD work on consecutive logical tiles, i.e. on the heads of the same (b,c).  No workgroup
+// ever waits on another: the loop bounds are fixed at launch.
+// ------------------------------------------------------------------------------------------
+struct TileSched {
+    int base, pos, step, per;
+    __device__ explicit TileSched(int total) {
+        if (total % 8 == 0 && gridDim.x % 8 == 0) {
+            per = total / 8;
+            base = (int)(blockIdx.x % 8) * per;
+            pos = blockIdx.x / 8;
+            step = gridDim.x / 8;
+        } else {
+            per = total;
+            base = 0;
+            pos = blockIdx.x;
+            step = gridDim.x;
+        }
+    }
+    __device__ bool valid() const { return pos < per; }
+    __device__ bool has_next() const { return pos + step < per; }
+    __device__ int logical() const { return base + pos; }
+    __device__ int next_logical() const { return base + pos + step; }
+    __device__ void advance() { pos += step; }
+};
+
+struct Tile {
+    int b, c, h, g, t0;
+};
+__device__ inline Tile decode_tile(int logical, const ScanShape &s) {
+    Tile t;
+    t.h = logical % s.H;
+    t.c = (logical / s.H) % s.nc;
+    t.b = logical / (s.H * s.nc);
+    t.g = t.h / (s.H / s.G);
+    t.t0 = t.c * s.Q;
+    return t;
+}
+
+
+// Workgroups of a persistent kernel: as many as stay resident on the current device, in whole
+// multiples of the 8 XCDs, never more than there are tiles.
+template <typename K>
+static inline hipError_t persistent_grid(K kernel, int block, size_t lds, int tiles, int *grid) {
+    int dev = 0, cus = 0, per_cu = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, lds);
+    if (e != hipSuccess) return e;
+    if (per_cu < 1) per_cu = 1;
+    long long g = (long long)cus * per_cu;
+    if (g > tiles) g = tiles;
+    if (g >= 8) g -= g % 8;
+    *grid = (int)(g < 1 ? 1 : g);
+    return hipSuccess;
+}
+
+template <typename K> static inline hipError_t allow_lds(K kernel, size_t bytes) {
+    if (bytes <= 64 * 1024) return hipSuccess;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+}  // namespace ssd

@@ -22,7 +22,8 @@ size_t chunk_state_lds_bytes(const ScanShape &s, int elem_bytes);
 size_t chunk_scan_lds_bytes(const ScanShape &s, int elem_bytes);
 
 // dtype: 0 = float32, 1 = bf16, 2 = bf16 inputs with float32 y (stage 4 only; stages 1-2 treat it as 1).
-// dtcs is the stage-1 output [B,H,nc,3,Q] float32: cumulative dt*A as a hi/lo pair, then dt.
+// dtcs is the stage-1 output [B,H,nc,4,Q] float32: log2(e) * cumulative dt*A as a hi/lo pair, dt, and
+// the stage-2 weight exp2(alpha[Q-1] - alpha[l]) * dt[l].
 hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A,
                                float *dtcs, hipStream_t stream);
 hipError_t launch_chunk_state(const ScanShape &s, int dtype, const void *x, const void *Bm,

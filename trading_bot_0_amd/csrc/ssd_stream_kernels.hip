@@ -1,0 +1,267 @@
+// Mamba-2 SSD forward for gfx950 (MI355X, CDNA4): the three streaming kernels.
+// Stage 1 (chunk_cumsum) is a DPP wavefront scan; stage 3 (state_passing) and stage 5 (the
+// single-timestep update) are pure HBM streams.  Stages 2 and 4 (MFMA tiles) live in
+// ssd_chunk_state.hip and ssd_chunk_scan.hip.
+#include "ssd_device.h"
+
+namespace ssd {
+
+// ------------------------------------------------------------------------------------------
+// Stage 1: chunk_cumsum.  One workgroup per (b,c): the [Q,H] tile of dt is read coalesced,
+// transposed through LDS, and every head row gets a wavefront inclusive scan of dt*A.
+//
+// Output "dtcs" [B,H,nc,4,Q] float32: rows 0/1 = alpha (the cumulative sum times log2 e) as
+// an unevaluated pair hi + lo, row 2 = dt, row 3 = the stage-2 weight
+// exp2(alpha[Q-1] - alpha[l]) * dt[l] (decay from step l to the end of the chunk).  The scan runs in float64 and is split into two
+// floats because the later stages only ever use DIFFERENCES alpha[l] - alpha[s]: with one
+// float, a large |alpha| (hundreds after a strongly decaying step) leaves an absolute error
+// of ulp(|alpha|) in a difference that may itself be small, i.e. a relative error of
+// 1e-5..1e-3 in the decay factor.  (hi_l - hi_s) + (lo_l - lo_s) keeps the difference good to
+// its own ulp.
+// ------------------------------------------------------------------------------------------
+template <int CTRL, int ROWMASK> __device__ inline double dpp_move(double v) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROWMASK, 0xf, false);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROWMASK, 0xf, false);
+    return __hiloint2double(hi, lo);  // lanes the row mask disables, or with no source lane, get +0.0
+}
+// Inclusive sum across the 64 lanes with DPP data movement: shifts inside rows of 16, then the
+// row totals are broadcast into the following rows (row_bcast:15 / row_bcast:31).
+__device__ inline double wave_inclusive_scan(double v) {
+    v += dpp_move<0x111, 0xf>(v);  // row_shr:1
+    v += dpp_move<0x112, 0xf>(v);  // row_shr:2
+    v += dpp_move<0x114, 0xf>(v);  // row_shr:4
+    v += dpp_move<0x118, 0xf>(v);  // row_shr:8
+    v += dpp_move<0x142, 0xa>(v);  // row_bcast:15 -> rows 1,3
+    v += dpp_move<0x143, 0xc>(v);  // row_bcast:31 -> rows 2,3
+    return v;
+}
+
+template <typename T, int EPL>  // EPL = elements per lane = max(Q/64, 1)
+__global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__ dt,
+                                                           const float *__restrict__ A,
+                                                           float *__restrict__ dtcs, ScanShape s) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    float *tile = reinterpret_cast<float *>(smem);  // [H][Q+1]
+    const int ldt = s.Q + 1;
+    const int b = blockIdx.x / s.nc, c = blockIdx.x % s.nc;
+    const int t0 = c * s.Q;
+    for (int idx = threadIdx.x; idx < s.Q * s.H; idx += blockDim.x) {
+        const int l = idx / s.H, h = idx % s.H;
+        const int t = t0 + l;
+        const float v = (t < s.L) ? (float)dt[((size_t)b * s.L + t) * s.H + h] : 0.f;
+        tile[h * ldt + l] = v;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    constexpr double kLog2e = 1.4426950408889634;
+    for (int h = wave; h < s.H; h += nwaves) {
+        const double a = (double)A[h];
+        float dtv[EPL];
+        double cs[EPL];
+        double run = 0.0;
+        const int l0 = lane * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            dtv[e] = (l0 + e < s.Q) ? tile[h * ldt + l0 + e] : 0.f;
+            run += (double)dtv[e] * a;
+            cs[e] = run;
+        }
+        const double incl = wave_inclusive_scan(run);
+        const double excl = incl - run;
+        // chunk total = the last lane's inclusive sum (lanes past Q carry zeros)
+        const double total = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(incl), 63),
+                                              __builtin_amdgcn_readlane(__double2loint(incl), 63));
+        if (l0 < s.Q) {
+            float *row = dtcs + ((((size_t)b * s.H + h) * s.nc + c) * 4) * s.Q + l0;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const double cum = cs[e] + excl;
+                const double al = cum * kLog2e;
+                const float hi = (float)al;
+                row[e] = hi;
+                row[s.Q + e] = (float)(al - (double)hi);
+                row[2 * s.Q + e] = dtv[e];
+                row[3 * s.Q + e] = exp2_hw(fminf((float)((total - cum) * kLog2e), 0.f)) * dtv[e];
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Stage 3: state_passing.  One lane per float4 of the [P,N] state of one (b,h); the chunk
+// loop is the only sequential axis.  All chunk loads of a batch of chunks are issued before
+// the dependent multiply-adds so the recurrence does not serialise memory latency.
+// prev may alias states: each lane reads its element of chunk c before overwriting it.
+// ------------------------------------------------------------------------------------------
+constexpr int kPassUnroll = 8;
+
+__global__ __launch_bounds__(256) void state_passing_kernel(const float *states, const float *__restrict__ dtcs,
+                                                            const float *init, float *prev,
+                                                            float *final_states, ScanShape s,
+                                                            long long total) {
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const int pn4 = s.P * s.N / 4;
+    const int bh = (int)(gid / pn4), idx = (int)(gid % pn4);
+    const int b = bh / s.H, h = bh % s.H;
+    const size_t chunk_stride = (size_t)s.H * pn4;  // in float4
+    const float4 *src = reinterpret_cast<const float4 *>(states) + ((size_t)b * s.nc * s.H + h) * pn4 + idx;
+    float4 *dst = reinterpret_cast<float4 *>(prev) + ((size_t)b * s.nc * s.H + h) * pn4 + idx;
+    const float *a_end = dtcs + ((size_t)bh * s.nc) * 4 * s.Q + (s.Q - 1);  // alpha_hi at the chunk end
+    const size_t a_stride = (size_t)4 * s.Q;
+    float4 st = init ? reinterpret_cast<const float4 *>(init)[(size_t)bh * pn4 + idx] : make_float4(0, 0, 0, 0);
+    int c = 0;
+    for (; c + kPassUnroll <= s.nc; c += kPassUnroll) {
+        float4 sv[kPassUnroll];
+        float dec[kPassUnroll];
+#pragma unroll
+        for (int i = 0; i < kPassUnroll; ++i) {
+            sv[i] = src[(size_t)(c + i) * chunk_stride];
+            dec[i] = exp2_hw(a_end[(size_t)(c + i) * a_stride]);
+        }
+#pragma unroll
+        for (int i = 0; i < kPassUnroll; ++i) {
+            dst[(size_t)(c + i) * chunk_stride] = st;
+            st.x = dec[i] * st.x + sv[i].x;
+            st.y = dec[i] * st.y + sv[i].y;
+            st.z = dec[i] * st.z + sv[i].z;
+            st.w = dec[i] * st.w + sv[i].w;
+        }
+    }
+    for (; c < s.nc; ++c) {
+        const float4 sv = src[(size_t)c * chunk_stride];
+        const float dec = exp2_hw(a_end[(size_t)c * a_stride]);
+        dst[(size_t)c * chunk_stride] = st;
+        st.x = dec * st.x + sv.x;
+        st.y = dec * st.y + sv.y;
+        st.z = dec * st.z + sv.z;
+        st.w = dec * st.w + sv.w;
+    }
+    if (final_states) reinterpret_cast<float4 *>(final_states)[(size_t)bh * pn4 + idx] = st;
+}
+
+// ------------------------------------------------------------------------------------------
+// Stage 5: single-timestep update, in place.  One wave per (b,h); NL = N/4 lanes cover one
+// state row with a float4 each, 64/NL rows per pass.  The row dot-product with C is reduced
+// across the NL lanes with xor-shuffles.  TO is the element type of y.
+// ------------------------------------------------------------------------------------------
+template <typename T, typename TO, int NL>
+__global__ __launch_bounds__(256) void step_kernel(float *__restrict__ state, const T *__restrict__ x,
+                                                   const T *__restrict__ dt, const float *__restrict__ A,
+                                                   const T *__restrict__ Bm, const T *__restrict__ Cm,
+                                                   const float *__restrict__ D, TO *__restrict__ y, StepShape s) {
+    constexpr int N = NL * 4;
+    constexpr int RPP = 64 / NL;  // rows per pass
+    constexpr int UN = 4;         // passes whose loads are issued together
+    const int lane = threadIdx.x & 63;
+    const long long bh = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (bh >= (long long)s.B * s.H) return;
+    const int b = (int)(bh / s.H), h = (int)(bh % s.H);
+    const int g = h / (s.H / s.G);
+    const int nl = lane % NL, rl = lane / NL;
+    const float dtv = (float)dt[bh];
+    const float decay = expf(dtv * A[h]);
+    const float dh = D ? D[h] : 0.f;
+    float bv[4], cv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        bv[i] = (float)Bm[((size_t)b * s.G + g) * N + nl * 4 + i] * dtv;
+        cv[i] = (float)Cm[((size_t)b * s.G + g) * N + nl * 4 + i];
+    }
+    float4 *st = reinterpret_cast<float4 *>(state) + (size_t)bh * s.P * NL;
+    const T *xr = x + (size_t)bh * s.P;
+    TO *yr = y + (size_t)bh * s.P;
+    for (int p0 = 0; p0 < s.P; p0 += RPP * UN) {
+        float4 hv[UN];
+        float xv[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int p = p0 + u * RPP + rl;
+            if (p < s.P) {
+                hv[u] = st[(size_t)p * NL + nl];
+                xv[u] = (float)xr[p];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int p = p0 + u * RPP + rl;
+            float part = 0.f;
+            if (p < s.P) {
+                float4 v = hv[u];
+                v.x = decay * v.x + xv[u] * bv[0];
+                v.y = decay * v.y + xv[u] * bv[1];
+                v.z = decay * v.z + xv[u] * bv[2];
+                v.w = decay * v.w + xv[u] * bv[3];
+                st[(size_t)p * NL + nl] = v;
+                part = v.x * cv[0] + v.y * cv[1] + v.z * cv[2] + v.w * cv[3];
+            }
+#pragma unroll
+            for (int m = NL / 2; m >= 1; m >>= 1) part += __shfl_xor(part, m, 64);
+            if (p < s.P && nl == 0) yr[p] = (TO)(part + dh * xv[u]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Launchers
+// ------------------------------------------------------------------------------------------
+template <typename T>
+static hipError_t cumsum_dispatch(const ScanShape &s, const void *dt, const float *A, float *dtcs,
+                                  hipStream_t st) {
+    const dim3 grid(s.B * s.nc), block(256);
+    const size_t lds = (size_t)s.H * (s.Q + 1) * sizeof(float);
+    const T *d = static_cast<const T *>(dt);
+    if (s.Q <= 64) {
+        chunk_cumsum_kernel<T, 1><<<grid, block, lds, st>>>(d, A, dtcs, s);
+    } else if (s.Q == 128) {
+        chunk_cumsum_kernel<T, 2><<<grid, block, lds, st>>>(d, A, dtcs, s);
+    } else {
+        chunk_cumsum_kernel<T, 4><<<grid, block, lds, st>>>(d, A, dtcs, s);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A, float *dtcs,
+                               hipStream_t st) {
+    return dtype ? cumsum_dispatch<__bf16>(s, dt, A, dtcs, st) : cumsum_dispatch<float>(s, dt, A, dtcs, st);
+}
+
+hipError_t launch_state_passing(const ScanShape &s, const float *states, const float *dtcs, const float *init,
+                                float *prev, float *final_states, hipStream_t st) {
+    const long long total = (long long)s.B * s.H * (s.P * s.N / 4);
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    state_passing_kernel<<<dim3(blocks), dim3(256), 0, st>>>(states, dtcs, init, prev, final_states, s, total);
+    return hipGetLastError();
+}
+
+template <typename T, typename TO>
+static hipError_t step_dispatch(const StepShape &s, float *state, const void *x, const void *dt,
+                                const float *A, const void *Bm, const void *Cm, const float *D, void *y,
+                                hipStream_t st) {
+    const long long pairs = (long long)s.B * s.H;
+    const dim3 grid((unsigned)((pairs + 3) / 4)), block(256);
+    const T *xx = static_cast<const T *>(x), *dd = static_cast<const T *>(dt);
+    const T *bb = static_cast<const T *>(Bm), *cc = static_cast<const T *>(Cm);
+    TO *yy = static_cast<TO *>(y);
+    switch (s.N) {
+        case 16: step_kernel<T, TO, 4><<<grid, block, 0, st>>>(state, xx, dd, A, bb, cc, D, yy, s); break;
+        case 32: step_kernel<T, TO, 8><<<grid, block, 0, st>>>(state, xx, dd, A, bb, cc, D, yy, s); break;
+        case 64: step_kernel<T, TO, 16><<<grid, block, 0, st>>>(state, xx, dd, A, bb, cc, D, yy, s); break;
+        case 128: step_kernel<T, TO, 32><<<grid, block, 0, st>>>(state, xx, dd, A, bb, cc, D, yy, s); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *x, const void *dt,
+                       const float *A, const void *Bm, const void *Cm, const float *D, void *y,
+                       hipStream_t st) {
+    switch (dtype) {
+        case 0: return step_dispatch<float, float>(s, state, x, dt, A, Bm, Cm, D, y, st);
+        case 1: return step_dispatch<__bf16, __bf16>(s, state, x, dt, A, Bm, Cm, D, y, st);
+        default: return step_dispatch<__bf16, float>(s, state, x, dt, A, Bm, Cm, D, y, st);
+    }
+}
+
+}  // namespace ssd

@@ -239,7 +239,8 @@ def ssd_chunk_scan(
 # ---- per-stage entry points (testing / profiling) ----------------------------------------
 
 def chunk_cumsum(dt: torch.Tensor, A: torch.Tensor, chunk: int) -> torch.Tensor:
-    """Stage 1 -> dtcs [B,H,nc,3,Q] float32: log2(e) * cumulative dt*A as (hi, lo), then dt."""
+    """Stage 1 -> dtcs [B,H,nc,4,Q] float32: log2(e) * cumulative dt*A as (hi, lo), dt, and the
+    stage-2 weight exp(cs[Q-1] - cs[l]) * dt[l]."""
     lib = load_library()
     if dt.dim() != 3:
         raise ValueError(f"SSD dt must be rank-3 [batch, seqlen, nheads], got {tuple(dt.shape)}")
@@ -247,7 +248,7 @@ def chunk_cumsum(dt: torch.Tensor, A: torch.Tensor, chunk: int) -> torch.Tensor:
     _require(dt, "dt", (Bsz, L, H), dt.dtype)
     _require(A, "A", (H,), torch.float32)
     nc = num_chunks(L, chunk)
-    dtcs = torch.empty((Bsz, H, nc, 3, chunk), dtype=torch.float32, device=dt.device)
+    dtcs = torch.empty((Bsz, H, nc, 4, chunk), dtype=torch.float32, device=dt.device)
     dims = SsdDims(Bsz, L, H, 32, 64, 1, int(chunk))  # P, N, G do not enter stage 1
     _check(lib, lib.ssd_chunk_cumsum_fwd(byref(dims), _dtype_code(dt), dt.data_ptr(), A.data_ptr(),
                                          dtcs.data_ptr(), _stream_ptr(dt)))
@@ -256,7 +257,7 @@ def chunk_cumsum(dt: torch.Tensor, A: torch.Tensor, chunk: int) -> torch.Tensor:
 
 def _require_dtcs(dtcs, dims: SsdDims):
     nc = num_chunks(dims.seqlen, dims.chunk)
-    _require(dtcs, "dtcs", (dims.batch, dims.nheads, nc, 3, dims.chunk), torch.float32)
+    _require(dtcs, "dtcs", (dims.batch, dims.nheads, nc, 4, dims.chunk), torch.float32)
     return nc
 
 
@@ -280,7 +281,7 @@ def state_passing(states, dtcs, initial_states=None, in_place: bool = False):
     Bsz, nc, H, P, N = states.shape
     chunk = dtcs.shape[-1]
     _require(states, "chunk_states", (Bsz, nc, H, P, N), torch.float32)
-    _require(dtcs, "dtcs", (Bsz, H, nc, 3, chunk), torch.float32)
+    _require(dtcs, "dtcs", (Bsz, H, nc, 4, chunk), torch.float32)
     if initial_states is not None:
         _require(initial_states, "initial_states", (Bsz, H, P, N), torch.float32)
     prev = states if in_place else torch.empty_like(states)
