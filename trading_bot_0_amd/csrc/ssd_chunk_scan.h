@@ -20,35 +20,85 @@
 // The column-block index is rotated with the workgroup id so that the wave with the most
 // s-blocks does not always sit on the same SIMD.
 //
-// Persistent and software-pipelined like stage 2: the next tile's B, x, entering state, C and
-// alpha rows sit in registers while the current tile's MFMAs run.
+// Persistent and software-pipelined like stage 2: the next tile's B, x, entering state and
+// alpha rows sit in registers while the current tile's MFMAs run.  Everything that shapes the
+// inner code (head-dim blocks, state width, chunk length) is a template parameter.
+// y leaves in 16-byte pieces: the two lanes that hold one output column swap halves of their
+// values (v_permlane32_swap) so that each stores 8 consecutive head-dim elements.
+#pragma once
 #include "ssd_device.h"
 
 namespace ssd {
 
-template <typename T, typename TO, int PB, int NK>  // Ppad = 32*PB >= P, N = 16*NK
-__global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict__ x, const T *__restrict__ Bm,
-                                                            const T *__restrict__ Cm,
-                                                            const float *__restrict__ dtcs,
-                                                            const float *__restrict__ prev,
-                                                            const float *__restrict__ D, TO *__restrict__ y,
-                                                            ScanShape s) {
+__device__ inline void swap_halves(unsigned &x, unsigned &y) {
+    // x[lanes 32..63] <-> y[lanes 0..31]
+    const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+    x = r[0];
+    y = r[1];
+}
+__device__ inline unsigned pack_bf16x2(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+    bf16x2 v;
+    v[0] = (__bf16)a;
+    v[1] = (__bf16)b;
+    return __builtin_bit_cast(unsigned, v);
+}
+
+// One output column block of 32 head-dim values per lane pair: o[v] is element
+// p = 8*(v/4) + 4*half + v%4 of column l.  Writes p = 16*half .. 16*half+15 of row `yrow`
+// (yrow already points at the column's row and at head-dim offset 32*pb).
+template <typename TO> __device__ inline void store_column(TO *yrow, float (&o)[16], int half, int pvalid, bool row_ok);
+template <> __device__ inline void store_column<__bf16>(__bf16 *yrow, float (&o)[16], int half, int pvalid, bool row_ok) {
+    unsigned X[4], Y[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        X[k] = pack_bf16x2(o[2 * k], o[2 * k + 1]);          // p-groups 0 and 1 (v = 0..7)
+        Y[k] = pack_bf16x2(o[8 + 2 * k], o[8 + 2 * k + 1]);  // p-groups 2 and 3 (v = 8..15)
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) swap_halves(X[k], Y[k]);
+    if (row_ok) {
+        const int p0 = 16 * half;
+        if (p0 + 8 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0) = make_uint4(X[0], X[1], Y[0], Y[1]);
+        if (p0 + 16 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 8) = make_uint4(X[2], X[3], Y[2], Y[3]);
+    }
+}
+template <> __device__ inline void store_column<float>(float *yrow, float (&o)[16], int half, int pvalid, bool row_ok) {
+    unsigned X[8], Y[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        X[k] = __float_as_uint(o[k]);
+        Y[k] = __float_as_uint(o[8 + k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) swap_halves(X[k], Y[k]);
+    if (row_ok) {
+        const int p0 = 16 * half;
+        if (p0 + 4 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0) = make_uint4(X[0], X[1], X[2], X[3]);
+        if (p0 + 8 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 4) = make_uint4(Y[0], Y[1], Y[2], Y[3]);
+        if (p0 + 12 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 8) = make_uint4(X[4], X[5], X[6], X[7]);
+        if (p0 + 16 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 12) = make_uint4(Y[4], Y[5], Y[6], Y[7]);
+    }
+}
+
+template <typename T, typename TO, int PB, int NK, int QB>  // Ppad = 32*PB >= P, N = 16*NK, Q = 32*QB
+__global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >= 4) ? 3 : 2) void chunk_scan_kernel(
+    const T *__restrict__ x, const T *__restrict__ Bm, const T *__restrict__ Cm, const float *__restrict__ dtcs,
+    const float *__restrict__ prev, const float *__restrict__ D, TO *__restrict__ y, ScanShape s) {
     constexpr int VEC = Vec16<T>::N;
     constexpr int PARTS = Split<T>::PARTS;
-    constexpr int N = NK * 16;
-    constexpr int Ppad = PB * 32;
+    constexpr int N = NK * 16, Ppad = PB * 32, Q = QB * 32, nthr = 64 * QB, nblk = QB;
     constexpr int ldb = N + lds_pad<T>();
+    constexpr int ldx = Q + lds_pad<T>();    // float mode: xs is transposed [Ppad][ldx]
     // Load mapping over the 2Q threads: a thread owns one 16-byte column slot of rows l0, l0+rpp, ...
     constexpr int bcpr = N / VEC, xcpr = Ppad / VEC;
-    constexpr int UB = bcpr / 2, UX = xcpr / 2;   // passes = Q / (2Q / slots per row); both slot counts are even
+    constexpr int brpp = nthr / bcpr, xrpp = nthr / xcpr;
+    constexpr int UB = bcpr / 2, UX = xcpr / 2;   // passes = Q / rows per pass; both slot counts are even
     constexpr int hcpr = N / 4;
-    constexpr int UH = 2;                    // entering-state float4 loads per thread held across tiles
-    constexpr bool kPrefetchC = NK <= 4;     // wide states: C is fetched at the top of the tile instead
+    constexpr int UHfull = (Ppad * hcpr + nthr - 1) / nthr;
+    constexpr int UH = UHfull < 4 ? UHfull : 4;   // entering-state float4 loads per thread held across tiles
     using XT = RowMajorTile<Ppad>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int Q = s.Q;
-    const int ldx = Q + lds_pad<T>();        // float mode: xs is transposed [Ppad][ldx]
-    const int nblk = Q / 32;
     float *al_s = reinterpret_cast<float *>(smem);  // [3][Q]: alpha hi, alpha lo, dt
     float *tab = al_s + 3 * Q;                      // [nblk][Q]: exp2(alpha[32k]-alpha[s])*dt[s], s < 32k
     T *Bs = reinterpret_cast<T *>(tab + nblk * Q);  // [Q][ldb]
@@ -56,35 +106,19 @@ __global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict_
     T *xs = Hs + PARTS * Ppad * ldb;                // bf16: [Q][Ppad] row-major; float: [Ppad][ldx]
     const float *ah_s = al_s, *alo_s = al_s + Q, *dt_s = al_s + 2 * Q;
 
-    const int tid = threadIdx.x, nthr = 2 * Q;
+    const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, half = lane >> 5;
-    const int xrpp = nthr / xcpr, brpp = nthr / bcpr;
     const int xl0 = tid / xcpr, xch = tid % xcpr, bl0 = tid / bcpr, bch = tid % bcpr;
     const bool xslot = xch * VEC < s.P;      // column slots past P stay zero
     const int xoff0 = xl0 * s.H * s.P + xch * VEC, xstep = xrpp * s.H * s.P;   // elements
     const int boff0 = bl0 * s.G * N + bch * VEC, bstep = brpp * s.G * N;
     const int htotal = s.P * hcpr;
-    const bool p_full = s.P == Ppad;
 
     // ---- registers holding the next tile's inputs ----
     float a3[2];
     Vec16<T> bv[UB], xv[UX];
     float4 hv[UH];
-    Frag<T> Cn[kPrefetchC ? NK : 1];
-
-    // C fragments straight from global: column l = 32*lb + r of the tile, K = n
-    auto load_c = [&](const Tile &t, int logical, int rows, Frag<T> *dst) {
-        const int l = ((wave + logical) % nblk) * 32 + r;
-        const T *crow = Cm + (((size_t)t.b * s.L + t.t0 + l) * s.G + t.g) * N + half * 8;
-        if (rows == Q) {
-#pragma unroll
-            for (int kk = 0; kk < NK; ++kk) dst[kk] = load_frag(crow + kk * 16);
-        } else {
-#pragma unroll
-            for (int kk = 0; kk < NK; ++kk) dst[kk] = (l < rows) ? load_frag(crow + kk * 16) : zero_frag<T>();
-        }
-    };
     auto prefetch = [&](int logical) {
         const Tile t = decode_tile(logical, s);
         const float *arow = dtcs + ((((size_t)t.b * s.H + t.h) * s.nc + t.c) * 4) * Q;
@@ -95,8 +129,7 @@ __global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict_
         const T *xb = x + (((size_t)t.b * s.L + t.t0) * s.H + t.h) * s.P;
         if (rows == Q) {
 #pragma unroll
-            for (int u = 0; u < UB; ++u)
-                bv[u] = load_vec16(bb + boff0 + u * bstep);
+            for (int u = 0; u < UB; ++u) bv[u] = load_vec16(bb + boff0 + u * bstep);
 #pragma unroll
             for (int u = 0; u < UX; ++u) xv[u] = xslot ? load_vec16(xb + xoff0 + u * xstep) : zero_vec16<T>();
         } else {
@@ -107,26 +140,27 @@ __global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict_
             for (int u = 0; u < UX; ++u)
                 xv[u] = (xslot && xl0 + u * xrpp < rows) ? load_vec16(xb + xoff0 + u * xstep) : zero_vec16<T>();
         }
-        const float *hp = prev + ((((size_t)t.b * s.nc + t.c) * s.H + t.h) * s.P) * N;
+        const float4 *hp = reinterpret_cast<const float4 *>(prev + ((((size_t)t.b * s.nc + t.c) * s.H + t.h) * s.P) * N);
 #pragma unroll
         for (int u = 0; u < UH; ++u) {
             const int idx = u * nthr + tid;
-            hv[u] = (idx < htotal) ? *reinterpret_cast<const float4 *>(hp + idx * 4) : make_float4(0, 0, 0, 0);
+            hv[u] = (idx < htotal) ? hp[idx] : make_float4(0, 0, 0, 0);
         }
-        if (kPrefetchC) load_c(t, logical, rows, Cn);
     };
     auto put_state = [&](int idx, const float4 &h4) {
         const int p = idx / hcpr, n4 = idx % hcpr;
         const float v[4] = {h4.x, h4.y, h4.z, h4.w};
-        T hi[4], lo[4];
+        if constexpr (is_bf16<T>) {
+            __bf16 hi[4], lo[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) Split<T>::split(v[i], hi[i], lo[i]);
-        T *dsth = Hs + p * ldb + n4 * 4;
+            for (int i = 0; i < 4; ++i) Split<T>::split(v[i], hi[i], lo[i]);
+            bf16x4 h4v, l4v;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dsth[i] = hi[i];
-        if (PARTS == 2) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) dsth[Ppad * ldb + i] = lo[i];
+            for (int i = 0; i < 4; ++i) { h4v[i] = hi[i]; l4v[i] = lo[i]; }
+            *reinterpret_cast<bf16x4 *>(Hs + p * ldb + n4 * 4) = h4v;
+            *reinterpret_cast<bf16x4 *>(Hs + (Ppad + p) * ldb + n4 * 4) = l4v;
+        } else {
+            *reinterpret_cast<float4 *>(Hs + p * ldb + n4 * 4) = h4;
         }
     };
 
@@ -144,12 +178,17 @@ __global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict_
         const int rows = min(Q, s.L - t.t0);
         const int lb = (wave + logical) % nblk;  // this wave's column block
         const int l = lb * 32 + r;
+        // C fragments straight from global: column l of the tile, K = n
         Frag<T> Cf[NK];
-        if constexpr (kPrefetchC) {
+        {
+            const T *crow = Cm + (((size_t)t.b * s.L + t.t0 + l) * s.G + t.g) * N + half * 8;
+            if (rows == Q) {
 #pragma unroll
-            for (int kk = 0; kk < NK; ++kk) Cf[kk] = Cn[kk];
-        } else {
-            load_c(t, logical, rows, Cf);
+                for (int kk = 0; kk < NK; ++kk) Cf[kk] = load_frag(crow + kk * 16);
+            } else {
+#pragma unroll
+                for (int kk = 0; kk < NK; ++kk) Cf[kk] = (l < rows) ? load_frag(crow + kk * 16) : zero_frag<T>();
+            }
         }
 
         __syncthreads();  // the previous tile's LDS reads are done (and the zero fill is visible)
@@ -174,18 +213,21 @@ __global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict_
             const int idx = u * nthr + tid;
             if (idx < htotal) put_state(idx, hv[u]);
         }
-        {   // the part of the entering state the register batch does not hold (small chunk, large state)
-            const float *hp = prev + ((((size_t)t.b * s.nc + t.c) * s.H + t.h) * s.P) * N;
-            for (int idx = UH * nthr + tid; idx < htotal; idx += nthr)
-                put_state(idx, *reinterpret_cast<const float4 *>(hp + idx * 4));
+        if constexpr (UHfull > UH) {  // the part of the entering state the register batch does not hold
+            const float4 *hp = reinterpret_cast<const float4 *>(prev + ((((size_t)t.b * s.nc + t.c) * s.H + t.h) * s.P) * N);
+            for (int idx = UH * nthr + tid; idx < htotal; idx += nthr) put_state(idx, hp[idx]);
         }
         __syncthreads();  // alpha and dt are visible
         // decay table rows k = 1..nblk-1 (row 0 is never read)
-        for (int idx = tid; idx < nblk * Q; idx += nthr) {
-            const int k = idx / Q, sr = idx % Q;
-            if (k > 0 && sr < 32 * k) {
-                const float d = alpha_diff(ah_s[32 * k], alo_s[32 * k], ah_s[sr], alo_s[sr]);
-                tab[idx] = exp2_hw(fminf(d, 0.f)) * dt_s[sr];
+        if constexpr (nblk > 1) {
+#pragma unroll
+            for (int i = 0; i < (nblk * Q) / nthr; ++i) {
+                const int idx = i * nthr + tid;
+                const int k = idx / Q, sr = idx % Q;
+                if (k > 0 && sr < 32 * k) {
+                    const float d = alpha_diff(ah_s[32 * k], alo_s[32 * k], ah_s[sr], alo_s[sr]);
+                    tab[idx] = exp2_hw(fminf(d, 0.f)) * dt_s[sr];
+                }
             }
         }
         if (sched.has_next()) prefetch(sched.next_logical());
@@ -227,7 +269,7 @@ __global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict_
                     for (int i = 0; i < 4; ++i) {
                         const int v = vg * 4 + i;
                         T hi, lo;
-                        Split<T>::split(sc[v] * tv[i] * lane_dec, hi, lo);
+                        Split<T>::split(sc[v] * (tv[i] * lane_dec), hi, lo);
                         mh[v / 8].v[v % 8] = hi;
                         if (PARTS == 2) ml[v / 8].v[v % 8] = lo;
                     }
@@ -271,57 +313,62 @@ __global__ __launch_bounds__(512, 2) void chunk_scan_kernel(const T *__restrict_
             }
         }
         // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]
-        if (l < rows) {
+        {
             const float dh = D ? D[t.h] : 0.f;
-            TO *yrow = y + (((size_t)t.b * s.L + t.t0 + l) * s.H + t.h) * s.P + 4 * half;
+            TO *yrow = y + (((size_t)t.b * s.L + t.t0 + l) * s.H + t.h) * s.P;
 #pragma unroll
             for (int pb = 0; pb < PB; ++pb) {
+                float o[16];
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
                     const int p0 = pb * 32 + 8 * vg + 4 * half;
-                    if (p_full || p0 < s.P) {
-                        float xl[4];
-                        if constexpr (is_bf16<T>) {
-                            const bf16x4 x4 = *reinterpret_cast<const bf16x4 *>(xs + XT::off(l, p0));
+                    float xl[4];
+                    if constexpr (is_bf16<T>) {
+                        const bf16x4 x4 = *reinterpret_cast<const bf16x4 *>(xs + XT::off(l, p0));
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) xl[i] = (float)x4[i];
-                        } else {
+                        for (int i = 0; i < 4; ++i) xl[i] = (float)x4[i];
+                    } else {
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) xl[i] = xs[(p0 + i) * ldx + l];
-                        }
-                        store4<TO>(yrow + pb * 32 + 8 * vg, accY[pb][vg * 4 + 0] + dh * xl[0],
-                                   accY[pb][vg * 4 + 1] + dh * xl[1], accY[pb][vg * 4 + 2] + dh * xl[2],
-                                   accY[pb][vg * 4 + 3] + dh * xl[3]);
+                        for (int i = 0; i < 4; ++i) xl[i] = xs[(p0 + i) * ldx + l];
                     }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) o[vg * 4 + i] = accY[pb][vg * 4 + i] + dh * xl[i];
                 }
+                store_column<TO>(yrow + pb * 32, o, half, s.P - pb * 32, l < rows);
             }
         }
     }
 }
 
 // ------------------------------------------------------------------------------------------
-// Launchers
+// Launchers (one translation unit per input/output type pair instantiates scan_dispatch)
 // ------------------------------------------------------------------------------------------
-size_t chunk_scan_lds_bytes(const ScanShape &s, int eb) {
-    const size_t Ppad = (s.P + 31) & ~31;
-    const size_t ldb = s.N + 16 / eb, parts = eb == 2 ? 2 : 1;
-    const size_t xs = eb == 2 ? (size_t)s.Q * Ppad : Ppad * (size_t)(s.Q + 4);
-    return (size_t)s.Q * 12 + (size_t)(s.Q / 32) * s.Q * 4 + ((size_t)s.Q * ldb + parts * Ppad * ldb + xs) * eb;
-}
-
-template <typename T, typename TO, int PB, int NK>
+template <typename T, typename TO, int PB, int NK, int QB>
 static hipError_t scan_launch(const ScanShape &s, const void *x, const void *Bm, const void *Cm,
                               const float *dtcs, const float *prev, const float *D, void *y, hipStream_t st) {
     const size_t lds = chunk_scan_lds_bytes(s, sizeof(T));
-    hipError_t e = allow_lds(chunk_scan_kernel<T, TO, PB, NK>, lds);
+    hipError_t e = allow_lds(chunk_scan_kernel<T, TO, PB, NK, QB>, lds);
     if (e != hipSuccess) return e;
     int grid = 1;
-    e = persistent_grid(chunk_scan_kernel<T, TO, PB, NK>, 64 * (s.Q / 32), lds, s.B * s.nc * s.H, &grid);
+    e = persistent_grid(chunk_scan_kernel<T, TO, PB, NK, QB>, 64 * QB, lds, s.B * s.nc * s.H, &grid);
     if (e != hipSuccess) return e;
-    chunk_scan_kernel<T, TO, PB, NK><<<dim3(grid), dim3(64 * (s.Q / 32)), lds, st>>>(
+    chunk_scan_kernel<T, TO, PB, NK, QB><<<dim3(grid), dim3(64 * QB), lds, st>>>(
         static_cast<const T *>(x), static_cast<const T *>(Bm), static_cast<const T *>(Cm), dtcs, prev, D,
         static_cast<TO *>(y), s);
     return hipGetLastError();
+}
+
+template <typename T, typename TO, int PB, int NK>
+static hipError_t scan_dispatch_q(const ScanShape &s, const void *x, const void *Bm, const void *Cm,
+                                  const float *dtcs, const float *prev, const float *D, void *y,
+                                  hipStream_t st) {
+    switch (s.Q) {
+        case 32: return scan_launch<T, TO, PB, NK, 1>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 64: return scan_launch<T, TO, PB, NK, 2>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 128: return scan_launch<T, TO, PB, NK, 4>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 256: return scan_launch<T, TO, PB, NK, 8>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 template <typename T, typename TO, int PB>
@@ -329,28 +376,19 @@ static hipError_t scan_dispatch_n(const ScanShape &s, const void *x, const void 
                                   const float *dtcs, const float *prev, const float *D, void *y,
                                   hipStream_t st) {
     switch (s.N) {
-        case 16: return scan_launch<T, TO, PB, 1>(s, x, Bm, Cm, dtcs, prev, D, y, st);
-        case 32: return scan_launch<T, TO, PB, 2>(s, x, Bm, Cm, dtcs, prev, D, y, st);
-        case 64: return scan_launch<T, TO, PB, 4>(s, x, Bm, Cm, dtcs, prev, D, y, st);
-        case 128: return scan_launch<T, TO, PB, 8>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 16: return scan_dispatch_q<T, TO, PB, 1>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 32: return scan_dispatch_q<T, TO, PB, 2>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 64: return scan_dispatch_q<T, TO, PB, 4>(s, x, Bm, Cm, dtcs, prev, D, y, st);
+        case 128: return scan_dispatch_q<T, TO, PB, 8>(s, x, Bm, Cm, dtcs, prev, D, y, st);
         default: return hipErrorInvalidValue;
     }
 }
 
 template <typename T, typename TO>
-static hipError_t scan_dispatch(const ScanShape &s, const void *x, const void *Bm, const void *Cm,
-                                const float *dtcs, const float *prev, const float *D, void *y, hipStream_t st) {
+hipError_t scan_dispatch(const ScanShape &s, const void *x, const void *Bm, const void *Cm, const float *dtcs,
+                         const float *prev, const float *D, void *y, hipStream_t st) {
     return (s.P <= 32) ? scan_dispatch_n<T, TO, 1>(s, x, Bm, Cm, dtcs, prev, D, y, st)
                        : scan_dispatch_n<T, TO, 2>(s, x, Bm, Cm, dtcs, prev, D, y, st);
-}
-
-hipError_t launch_chunk_scan(const ScanShape &s, int dtype, const void *x, const void *Bm, const void *Cm,
-                             const float *dtcs, const float *prev, const float *D, void *y, hipStream_t st) {
-    switch (dtype) {
-        case 0: return scan_dispatch<float, float>(s, x, Bm, Cm, dtcs, prev, D, y, st);
-        case 1: return scan_dispatch<__bf16, __bf16>(s, x, Bm, Cm, dtcs, prev, D, y, st);
-        default: return scan_dispatch<__bf16, float>(s, x, Bm, Cm, dtcs, prev, D, y, st);
-    }
 }
 
 }  // namespace ssd
