@@ -41,6 +41,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-stream-step", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain elementwise kernel over 256 MiB in / 256 MiB out three times, the known-size "
+                         "reference that rocprofv3's FETCH_SIZE / WRITE_SIZE readings are scaled by")
     return ap.parse_args()
 
 
@@ -83,6 +86,14 @@ def main():
     def forward():
         ssd.ssd_chunk_scan(x, dt, A, Bm, Cm, D, chunk=w.chunk, initial_states=init, workspace=ws, out=y,
                            final_out=final)
+
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)   # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         forward()

@@ -107,7 +107,8 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
     const float *ah_s = al_s, *alo_s = al_s + Q, *dt_s = al_s + 2 * Q;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and known to be
     const int r = lane & 31, half = lane >> 5;
     const int xl0 = tid / xcpr, xch = tid % xcpr, bl0 = tid / bcpr, bch = tid % bcpr;
     const bool xslot = xch * VEC < s.P;      // column slots past P stay zero
@@ -287,8 +288,9 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int v = vg * 4 + i;
-                        const float arg = alpha_diff(al_hi, al_lo, ahv[i], alv[i]);
-                        const float w = (s0 + i <= l) ? exp2_hw(fminf(arg, 0.f)) * dtv[i] * sc[v] : 0.f;
+                        // masked entries get exp2(-inf) = 0: a select on the exponent, no branch
+                        const float arg = fminf(alpha_diff(al_hi, al_lo, ahv[i], alv[i]), 0.f);
+                        const float w = exp2_hw((s0 + i <= l) ? arg : -INFINITY) * dtv[i] * sc[v];
                         T hi, lo;
                         Split<T>::split(w, hi, lo);
                         mh[v / 8].v[v % 8] = hi;

@@ -37,7 +37,8 @@ __global__ __launch_bounds__(64 * PB * ((NK + 1) / 2)) void chunk_state_kernel(
     T *bs = xs + (is_bf16<T> ? PARTS * Q * Ppad : Ppad * ldq);  // bf16: [Q][Npad]; float: [Npad][ldq]
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and known to be
     const int r = lane & 31, half = lane >> 5;
     const int pb = wave / NB, nb = wave % NB;
     const int xl0 = tid / xcpr, xch = tid % xcpr, bl0 = tid / bcpr, bch = tid % bcpr;
