@@ -9,8 +9,8 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
   value        timesteps*batch/s of the whole forward (wall clock around K steps)
   roofline     the slowest stage kernel: algorithmic bytes per launch / its mean duration,
                measured with HIP events on the launch stream over a second timed region of K
-               steps in which the four stages are issued one by one through their own entry
-               points; all four stages are listed under "stages"
+               steps in which the stage kernels the forward launches are issued one by one
+               through their own entry points; all of them are listed under "stages"
   stream_step  the single-timestep update at batch 4096: latency and GB/s
   cpu_baseline the plain-C oracle (sequential recurrence, float32, OpenMP) timed on this
                box's host cores on a bounded batch slice of the same workload
@@ -126,11 +126,20 @@ def main():
         return lib.ssd_chunk_scan_stage_fwd(byref(dims), code, x.data_ptr(), Bm.data_ptr(), Cm.data_ptr(),
                                             dtcs.data_ptr(), S.data_ptr(), D.data_ptr(), y.data_ptr(), stream)
 
-    stage_fns = [("chunk_cumsum", k1), ("chunk_state", k2), ("state_passing", k3), ("chunk_scan", k4)]
+    def k23():
+        return lib.ssd_chunk_state_passing_fwd(byref(dims), code, x.data_ptr(), Bm.data_ptr(), dtcs.data_ptr(), ip,
+                                               S.data_ptr(), final.data_ptr(), stream)
+
+    # the stages the whole-forward entry point launches for this shape: with at least 512 (batch, head)
+    # sequences it runs stages 2 and 3 as one kernel
+    if w.batch * w.nheads >= 512:
+        stage_fns = [("chunk_cumsum", k1), ("chunk_state_passing", k23), ("chunk_scan", k4)]
+    else:
+        stage_fns = [("chunk_cumsum", k1), ("chunk_state", k2), ("state_passing", k3), ("chunk_scan", k4)]
     for _ in range(max(2, args.warmup // 2)):
         for _, fn in stage_fns:
             assert fn() == 0, ssd.last_error(lib)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(stage_fns) + 1)] for _ in range(args.steps)]
     torch.cuda.synchronize()
     for i in range(args.steps):
         ev[i][0].record()

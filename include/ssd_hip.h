@@ -104,6 +104,14 @@ int ssd_chunk_cumsum_fwd(const ssd_dims *dims, int dtype, const void *dt, const 
 int ssd_chunk_state_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm,
                         const float *dtcs, float *chunk_states, void *hip_stream);
 
+/* Stages 2 and 3 in one pass: prev_states[c] receives the state entering chunk c, final_states the state
+ * after the last chunk; the per-chunk states stay on chip.  Parallel over (batch, head) sequences only;
+ * ssd_chunk_scan_fwd uses it when there are enough of them.  initial_states / final_states may be NULL
+ * and may alias each other. */
+int ssd_chunk_state_passing_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm,
+                                const float *dtcs, const float *initial_states, float *prev_states,
+                                float *final_states, void *hip_stream);
+
 /* Stage 3: sequential recurrence over chunks.  prev_states[c] receives the state entering
  * chunk c and may alias chunk_states (in place); final_states and initial_states may be NULL
  * and may alias each other. */

@@ -99,6 +99,34 @@ def test_state_passing(shape, with_init, in_place):
     assert_close(final, mids["final"], torch.float32, "final states")
 
 
+@pytest.mark.parametrize("with_init", [False, True])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("shape", SHAPES + [(40, 384, 16, 32, 64, 2, 128)])
+def test_chunk_state_passing_fused(shape, dtype, with_init):
+    """Stages 2+3 in one pass: states entering each chunk and the final state, against the oracle and
+    against the two separate stages."""
+    skip_if_unsupported(shape, dtype)
+    w, dev, o, mids = build(shape, dtype, init_std=0.5 if with_init else 0.0)
+    dtcs = dtcs_dev(mids)
+    prev, final = ssd.chunk_state_passing(dev["x"], dev["B"], dtcs, dev["init"])
+    torch.cuda.synchronize()
+    assert_close(prev, mids["prev"], DT[dtype], "fused prev states")
+    assert_close(final, mids["final"], DT[dtype], "fused final states")
+    prev2, final2 = ssd.state_passing(ssd.chunk_state(dev["x"], dev["B"], dtcs), dtcs, dev["init"])
+    assert rel_err(prev, np64(prev2)) <= 1e-5 and rel_err(final, np64(final2)) <= 1e-5
+    if with_init:   # the final state may be written over the initial one
+        buf = dev["init"].clone()
+        lib = ssd.load_library()
+        from ctypes import byref
+        dims = ssd.SsdDims(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk)
+        rc = lib.ssd_chunk_state_passing_fwd(byref(dims), 1 if dtype == "bf16" else 0, dev["x"].data_ptr(),
+                                             dev["B"].data_ptr(), dtcs.data_ptr(), buf.data_ptr(), prev2.data_ptr(),
+                                             buf.data_ptr(), None)
+        assert rc == 0, ssd.last_error(lib)
+        torch.cuda.synchronize()
+        assert torch.equal(buf, final) and torch.equal(prev2, prev)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_chunk_scan_stage(shape, dtype):

@@ -5,6 +5,7 @@ from .ssd import (  # noqa: F401
     chunk_cumsum,
     chunk_scan_stage,
     chunk_state,
+    chunk_state_passing,
     load_library,
     ssd_chunk_scan,
     ssd_step,

@@ -90,6 +90,10 @@ int make_shape(const ssd_dims *d, int dtype, ssd::ScanShape *out) {
     return SSD_OK;
 }
 
+// The fused stage 2+3 kernel parallelises over (batch, head) sequences only; below this many sequences
+// the separate stages, which parallelise over chunks as well, fill the chip better.
+constexpr int64_t kFusedStatePassingMinSequences = 512;
+
 struct Workspace {
     size_t dtcs_off, st_off, total;
 };
@@ -153,6 +157,22 @@ int ssd_chunk_state_fwd(const ssd_dims *dims, int dtype, const void *x, const vo
     return e == hipSuccess ? SSD_OK : hip_fail(e, "chunk_state launch");
 }
 
+int ssd_chunk_state_passing_fwd(const ssd_dims *dims, int dtype, const void *x, const void *Bm, const float *dtcs,
+                                const float *initial_states, float *prev_states, float *final_states,
+                                void *hip_stream) {
+    ssd::ScanShape s;
+    if (int rc = make_shape(dims, dtype, &s)) return rc;
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(Bm);
+    REQUIRE_PTR(dtcs);
+    REQUIRE_PTR(prev_states);
+    OPTIONAL_PTR(initial_states);
+    OPTIONAL_PTR(final_states);
+    hipError_t e = ssd::launch_chunk_state_scan(s, dtype, x, Bm, dtcs, initial_states, prev_states, final_states,
+                                                (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "chunk_state_passing launch");
+}
+
 int ssd_state_passing_fwd(const ssd_dims *dims, const float *chunk_states, const float *dtcs,
                           const float *initial_states, float *prev_states, float *final_states,
                           void *hip_stream) {
@@ -208,10 +228,16 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
     hipStream_t st = (hipStream_t)hip_stream;
     hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dtcs, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_cumsum launch");
-    e = ssd::launch_chunk_state(s, dtype, x, Bm, dtcs, states, st);
-    if (e != hipSuccess) return hip_fail(e, "chunk_state launch");
-    e = ssd::launch_state_passing(s, states, dtcs, initial_states, states, final_states, st);  // in place
-    if (e != hipSuccess) return hip_fail(e, "state_passing launch");
+    if ((int64_t)s.B * s.H >= kFusedStatePassingMinSequences) {
+        // enough (b,h) sequences to fill the chip: stages 2 and 3 in one pass, states carried on chip
+        e = ssd::launch_chunk_state_scan(s, dtype, x, Bm, dtcs, initial_states, states, final_states, st);
+        if (e != hipSuccess) return hip_fail(e, "chunk_state_passing launch");
+    } else {
+        e = ssd::launch_chunk_state(s, dtype, x, Bm, dtcs, states, st);
+        if (e != hipSuccess) return hip_fail(e, "chunk_state launch");
+        e = ssd::launch_state_passing(s, states, dtcs, initial_states, states, final_states, st);  // in place
+        if (e != hipSuccess) return hip_fail(e, "state_passing launch");
+    }
     e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dtcs, states, D, y, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_scan launch");
     return SSD_OK;

@@ -192,7 +192,7 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
             }
         }
 
-        __syncthreads();  // the previous tile's LDS reads are done (and the zero fill is visible)
+        block_sync_lds();  // the previous tile's LDS reads are done (and the zero fill is visible)
         // ---- registers -> LDS ----
         if (tid < 3 * Q) al_s[tid] = a3[0];
         if (tid + nthr < 3 * Q) al_s[tid + nthr] = a3[1];
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
             const float4 *hp = reinterpret_cast<const float4 *>(prev + ((((size_t)t.b * s.nc + t.c) * s.H + t.h) * s.P) * N);
             for (int idx = UH * nthr + tid; idx < htotal; idx += nthr) put_state(idx, hp[idx]);
         }
-        __syncthreads();  // alpha and dt are visible
+        block_sync_lds();  // alpha and dt are visible
         // decay table rows k = 1..nblk-1 (row 0 is never read)
         if constexpr (nblk > 1) {
 #pragma unroll
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
             }
         }
         if (sched.has_next()) prefetch(sched.next_logical());
-        __syncthreads();
+        block_sync_lds();
 
         const float al_hi = ah_s[l], al_lo = alo_s[l];
         f32x16 accY[PB];

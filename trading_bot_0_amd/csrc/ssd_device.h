@@ -186,6 +186,15 @@ template <int COLS> struct RowMajorTile {
     }
 };
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, and
+// on gfx9 loads and stores share one counter, so it drains every outstanding global load -- among
+// them the next tile's prefetch, which must stay in flight across the barrier.  The tile loops
+// share nothing through global memory inside a launch, so waiting for LDS (and scalar) operations
+// is all the barrier needs.
+__device__ inline void block_sync_lds() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs, each with a private L2.  Re-number them so
 // that consecutive logical ids (the heads of one (b,c) tile, which share B and C and sit in
 // the same cache lines of x) land on the same XCD at nearly the same time.
@@ -250,6 +259,12 @@ static inline hipError_t persistent_grid(K kernel, int block, size_t lds, int ti
     if (e != hipSuccess) return e;
     e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, lds);
     if (e != hipSuccess) return e;
+    // The occupancy query counts a workgroup whose LDS fills the CU to the last byte; measured, that
+    // one does not become resident, and a persistent grid larger than residency runs a second round.
+    if (lds > 0) {
+        const int by_lds = (int)(kLdsLimitBytes / (lds + 1024));
+        if (per_cu > by_lds) per_cu = by_lds;
+    }
     if (per_cu < 1) per_cu = 1;
     long long g = (long long)cus * per_cu;
     if (g > tiles) g = tiles;

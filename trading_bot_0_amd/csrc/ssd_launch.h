@@ -28,6 +28,10 @@ hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, co
                                float *dtcs, hipStream_t stream);
 hipError_t launch_chunk_state(const ScanShape &s, int dtype, const void *x, const void *Bm,
                               const float *dtcs, float *states, hipStream_t stream);
+// stages 2+3 in one pass: writes the state entering each chunk into `prev` and the final state
+hipError_t launch_chunk_state_scan(const ScanShape &s, int dtype, const void *x, const void *Bm,
+                                   const float *dtcs, const float *init, float *prev, float *final_states,
+                                   hipStream_t stream);
 hipError_t launch_state_passing(const ScanShape &s, const float *states, const float *dtcs,
                                 const float *init, float *prev, float *final_states,
                                 hipStream_t stream);

@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "ssd_chunk_cumsum_fwd",
     "ssd_chunk_state_fwd",
     "ssd_state_passing_fwd",
+    "ssd_chunk_state_passing_fwd",
     "ssd_chunk_scan_stage_fwd",
     "ssd_step_fwd",
 )
@@ -86,6 +87,7 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_chunk_cumsum_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P]
         lib.ssd_chunk_state_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P]
         lib.ssd_state_passing_fwd.argtypes = [POINTER(SsdDims), P, P, P, P, P, P]
+        lib.ssd_chunk_state_passing_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P]
         lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
         for name in EXPORTED_SYMBOLS[2:]:
@@ -271,6 +273,20 @@ def chunk_state(x, Bm, dtcs):
     _check(lib, lib.ssd_chunk_state_fwd(byref(dims), _dtype_code(x), x.data_ptr(), Bm.data_ptr(),
                                         dtcs.data_ptr(), S.data_ptr(), _stream_ptr(x)))
     return S
+
+
+def chunk_state_passing(x, Bm, dtcs, initial_states=None):
+    """Stages 2+3 in one pass -> (prev_states [B,nc,H,P,N], final_states [B,H,P,N])."""
+    lib = load_library()
+    dims = _scan_dims(x, Bm, dtcs.shape[-1])
+    _validate_scan_inputs(x, None, None, Bm, None, None, initial_states, dims)
+    nc = _require_dtcs(dtcs, dims)
+    prev = torch.empty((dims.batch, nc, dims.nheads, dims.headdim, dims.dstate), dtype=torch.float32, device=x.device)
+    final = torch.empty((dims.batch, dims.nheads, dims.headdim, dims.dstate), dtype=torch.float32, device=x.device)
+    _check(lib, lib.ssd_chunk_state_passing_fwd(byref(dims), _dtype_code(x), x.data_ptr(), Bm.data_ptr(),
+                                                dtcs.data_ptr(), _ptr(initial_states), prev.data_ptr(),
+                                                final.data_ptr(), _stream_ptr(x)))
+    return prev, final
 
 
 def state_passing(states, dtcs, initial_states=None, in_place: bool = False):

@@ -128,6 +128,10 @@ def stage_bytes(w: Workload) -> dict:
         "chunk_cumsum": (e + 8) * blh,
         "chunk_state": e * (blh * P + Bsz * L * G * N) + 8 * blh + 4 * st,
         "state_passing": 8 * st + 4 * Bsz * H * nc + 4 * Bsz * H * P * N * (1 + has_init),
+        # stages 2+3 in one pass: stage 2's traffic (the chunk-state buffer is written once, with the state
+        # entering each chunk) plus the chunk decays and the initial / final states
+        "chunk_state_passing": e * (blh * P + Bsz * L * G * N) + 8 * blh + 4 * st + 4 * Bsz * H * nc
+                               + 4 * Bsz * H * P * N * (1 + has_init),
         "chunk_scan": e * (2 * blh * P + 2 * Bsz * L * G * N) + 8 * blh + 4 * st,
     }
 
@@ -137,6 +141,7 @@ def stage_flops(w: Workload) -> dict:
     Bsz, L, H, P, N, G, Q = w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk
     return {
         "chunk_state": 2 * Bsz * L * H * N * P,
+        "chunk_state_passing": 2 * Bsz * L * H * N * P,
         "chunk_scan": 2 * Bsz * L * (G * Q * N + H * Q * P + H * N * P),
     }
 
