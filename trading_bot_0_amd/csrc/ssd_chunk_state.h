@@ -190,7 +190,9 @@ __global__ __launch_bounds__(64 * PB * ((NK + 1) / 2)) void chunk_state_kernel(
                     for_rows([&](int v, int o) { acc[v] = ib[o]; });
                 }
             }
-            for_rows([&](int v, int o) { out[o] = acc[v]; });  // the state entering chunk c
+            // the state entering chunk 0 is the initial state; later chunks' entering states are
+            // written at the end of the tile before (after the MFMAs, when the prefetch has landed)
+            if (t.c == 0) for_rows([&](int v, int o) { out[o] = acc[v]; });
             acc = acc * exp2_hw(a_end);
         } else {
 #pragma unroll
@@ -210,7 +212,10 @@ __global__ __launch_bounds__(64 * PB * ((NK + 1) / 2)) void chunk_state_kernel(
             for (int ks = 0; ks < Q; ks += 16) acc = mma32(load_frag(arow_p + ks), load_frag(brow_p + ks), acc);
         }
         if constexpr (SCAN) {
-            if (t.c == s.nc - 1 && final_states) {
+            if (t.c < s.nc - 1) {
+                float *nx = out + (size_t)s.H * s.P * N;  // chunk c+1 of the same (b,h)
+                for_rows([&](int v, int o) { nx[o] = acc[v]; });
+            } else if (final_states) {
                 float *fb = final_states + ((size_t)t.b * s.H + t.h) * s.P * N + blk;
                 for_rows([&](int v, int o) { fb[o] = acc[v]; });
             }
