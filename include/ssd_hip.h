@@ -112,6 +112,17 @@ int ssd_chunk_state_passing_fwd(const ssd_dims *dims, int dtype, const void *x, 
                                 const float *dtcs, const float *initial_states, float *prev_states,
                                 float *final_states, void *hip_stream);
 
+/* The whole forward in one kernel and one pass over the inputs (bf16 inputs only): a wave keeps the running
+ * state of 32 head-dim columns of one (batch, head) in registers while it walks the chunks, so no workspace
+ * is needed and nothing but x, dt, B, C is read and y, final_states written.  Same arguments and results as
+ * ssd_chunk_scan_fwd.  Parallel over (batch, head) sequences only; ssd_chunk_scan_fwd takes this path by
+ * itself when there are enough of them.  SSD_ERR_UNSUPPORTED unless dtype is bf16 (1 or 2), headdim is a
+ * multiple of 32, dstate is 32 or 64, chunk is 64 or 128 and (nheads/ngroups)*(headdim/32) is a multiple
+ * of 4.  Replaces the same slot as ssd_chunk_scan_fwd (model/trading_model.rs:589-606). */
+int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
+                               const void *Bm, const void *Cm, const float *D, const float *initial_states,
+                               void *y, float *final_states, void *hip_stream);
+
 /* Stage 3: sequential recurrence over chunks.  prev_states[c] receives the state entering
  * chunk c and may alias chunk_states (in place); final_states and initial_states may be NULL
  * and may alias each other. */

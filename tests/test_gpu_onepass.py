@@ -1,0 +1,111 @@
+"""The one-pass forward (one kernel, running state in registers) through the C ABI against the float64
+oracle: the shapes that pick each of its template instances, ragged tails, initial states, strong decay
+(the exact diagonal path), and agreement with the staged kernels."""
+import pytest
+import torch
+
+from trading_bot_0_amd import SsdError, ssd_chunk_scan, ssd_chunk_scan_onepass
+from trading_bot_0_amd.synthetic import WORKLOADS, Workload, make_inputs
+
+from _util import assert_close, check_y, oracle_scan, rel_err, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def run(dev, chunk, **kw):
+    y, final = ssd_chunk_scan_onepass(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=chunk,
+                                      initial_states=dev["init"], **kw)
+    torch.cuda.synchronize()
+    return y, final
+
+
+def check(w, seed=0, seqlen=None, drop_D=False):
+    cpu = make_inputs(w, seed=seed, seqlen=seqlen)
+    if drop_D:
+        cpu["D"] = None
+    dev = to_dev(cpu)
+    yr, fr = oracle_scan(cpu, with_D=not drop_D)
+    finals = []
+
+    def call(yd):
+        y, f = run(dev, w.chunk, y_dtype=yd)
+        finals.append(f)
+        return y
+
+    y, ey = check_y(call, yr, w.torch_dtype, f"{w.name} y")
+    assert all(torch.equal(f, finals[0]) for f in finals)
+    ef = assert_close(finals[0], fr, w.torch_dtype, f"{w.name} final")
+    print(f"one-pass {w.name} B={w.batch} L={seqlen or w.seqlen} H={w.nheads} P={w.headdim} N={w.dstate} "
+          f"G={w.ngroups} Q={w.chunk}: err_y={ey:.2e} err_final={ef:.2e}")
+    return dev, y, finals[0]
+
+
+SHAPES = {
+    # name: (batch, seqlen, nheads, headdim, dstate, ngroups, chunk)  -> instance picked
+    "policy": (2, 1024, 8, 32, 64, 1, 128),          # N=64 Q=128, 8 waves
+    "two_groups": (2, 512, 8, 32, 64, 2, 128),       # 4 units per group: 4 waves
+    "wide_head": (2, 512, 4, 64, 64, 1, 128),        # two 32-column units per head
+    "small_state": (2, 512, 8, 32, 32, 1, 128),      # N=32
+    "short_chunk": (2, 512, 8, 32, 64, 1, 64),       # Q=64
+    "small_state_short_chunk": (3, 256, 4, 32, 32, 1, 64),   # N=32 Q=64, 4 waves
+    "many_units": (1, 384, 16, 64, 64, 2, 128),      # 16 units per group: two workgroups per (batch, group)
+}
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+def test_shapes_against_oracle(name):
+    b, l, h, p, n, g, q = SHAPES[name]
+    check(Workload(name, b, l, h, p, n, g, q), seed=1)
+
+
+@pytest.mark.parametrize("seqlen", [1, 31, 128, 129, 300, 1000])
+def test_ragged_lengths(seqlen):
+    check(Workload("ragged", 2, seqlen, 8, 32, 64, 1, 128, init_std=0.5), seed=seqlen)
+
+
+def test_no_skip_term_and_initial_state():
+    check(Workload("no_D", 2, 384, 8, 32, 64, 1, 128, init_std=1.0), seed=3, drop_D=True)
+
+
+def test_strong_decay_takes_the_exact_diagonal_path():
+    # |A| up to 64 with dt up to ~6: whole blocks decay by far more than 2^-120
+    check(WORKLOADS["decay_extreme"].with_batch(2), seed=5, seqlen=1024)
+    check(Workload("all_large_dt", 2, 256, 8, 32, 64, 1, 128, a_log_range=(32.0, 64.0), dt_law="mixture",
+                   x_law="student-t3"), seed=6)
+
+
+def test_policy_workload_at_oracle_size():
+    check(WORKLOADS["policy_bf16"].with_batch(4))
+
+
+def test_agrees_with_the_staged_kernels():
+    w = WORKLOADS["policy_bf16"].with_batch(4)      # too few sequences for the automatic choice
+    dev = to_dev(make_inputs(w, seed=11, seqlen=640))
+    y1, f1 = run(dev, w.chunk, y_dtype=torch.float32)
+    y2, f2 = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                            y_dtype=torch.float32)
+    assert rel_err(y1, y2.double().cpu().numpy()) <= 1e-3
+    assert rel_err(f1, f2.double().cpu().numpy()) <= 1e-3
+
+
+def test_chunk_scan_takes_the_one_pass_path_for_large_batches():
+    w = WORKLOADS["policy_bf16"].with_batch(128)     # 128 workgroups of 8 units
+    dev = to_dev(make_inputs(w, seed=2, seqlen=256))
+    y1, f1 = run(dev, w.chunk)
+    y2, f2 = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk)
+    assert torch.equal(y1, y2) and torch.equal(f1, f2)
+
+
+def test_unsupported_shapes_are_refused():
+    cases = [
+        WORKLOADS["plumbing_f32"],                                  # float32 inputs
+        Workload("p16", 2, 128, 8, 16, 64, 1, 128),                 # headdim not a multiple of 32
+        Workload("n128", 2, 256, 8, 32, 128, 1, 128),               # state too wide for the accumulators
+        Workload("q256", 2, 256, 8, 32, 64, 1, 256),
+        Workload("units2", 2, 128, 2, 32, 64, 1, 128),              # 2 units per group
+    ]
+    for w in cases:
+        dev = to_dev(make_inputs(w, seed=0))
+        with pytest.raises(SsdError) as ei:
+            run(dev, w.chunk)
+        assert ei.value.code == 2, w.name

@@ -93,6 +93,9 @@ int make_shape(const ssd_dims *d, int dtype, ssd::ScanShape *out) {
 // The fused stage 2+3 kernel parallelises over (batch, head) sequences only; below this many sequences
 // the separate stages, which parallelise over chunks as well, fill the chip better.
 constexpr int64_t kFusedStatePassingMinSequences = 512;
+// The one-pass kernel runs one workgroup per 8 units of 32 head-dim columns and is parallel over sequences
+// only; below this many workgroups the staged kernels (parallel over chunks too) fill the chip better.
+constexpr int64_t kOnePassMinWorkgroups = 96;
 
 struct Workspace {
     size_t dtcs_off, st_off, total;
@@ -226,7 +229,13 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
     float *dtcs = reinterpret_cast<float *>(base + w.dtcs_off);
     float *states = reinterpret_cast<float *>(base + w.st_off);
     hipStream_t st = (hipStream_t)hip_stream;
-    hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dtcs, st);
+    hipError_t e;
+    if (ssd::fused_scan_waves(s, dtype) == 8 &&
+        (int64_t)s.B * s.H * (s.P / 32) / 8 >= kOnePassMinWorkgroups) {
+        e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, y, final_states, st);
+        return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
+    }
+    e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dtcs, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_cumsum launch");
     if ((int64_t)s.B * s.H >= kFusedStatePassingMinSequences) {
         // enough (b,h) sequences to fill the chip: stages 2 and 3 in one pass, states carried on chip
@@ -241,6 +250,29 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
     e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dtcs, states, D, y, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_scan launch");
     return SSD_OK;
+}
+
+int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
+                               const void *Bm, const void *Cm, const float *D, const float *initial_states,
+                               void *y, float *final_states, void *hip_stream) {
+    ssd::ScanShape s;
+    if (int rc = make_shape(dims, dtype, &s)) return rc;
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(dt);
+    REQUIRE_PTR(A);
+    REQUIRE_PTR(Bm);
+    REQUIRE_PTR(Cm);
+    REQUIRE_PTR(y);
+    OPTIONAL_PTR(D);
+    OPTIONAL_PTR(initial_states);
+    OPTIONAL_PTR(final_states);
+    if (ssd::fused_scan_waves(s, dtype) == 0)
+        return fail(SSD_ERR_UNSUPPORTED,
+                    "ssd: the one-pass scan needs bf16 inputs, headdim a multiple of 32, dstate 32 or 64, chunk 64 "
+                    "or 128 and (nheads/ngroups)*(headdim/32) a multiple of 4");
+    hipError_t e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, y, final_states,
+                                          (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
 }
 
 int ssd_step_fwd(const ssd_step_dims *dims, int dtype, float *state, const void *x, const void *dt,

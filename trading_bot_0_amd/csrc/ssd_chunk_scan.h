@@ -30,57 +30,6 @@
 
 namespace ssd {
 
-__device__ inline void swap_halves(unsigned &x, unsigned &y) {
-    // x[lanes 32..63] <-> y[lanes 0..31]
-    const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
-    x = r[0];
-    y = r[1];
-}
-__device__ inline unsigned pack_bf16x2(float a, float b) {
-    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-    bf16x2 v;
-    v[0] = (__bf16)a;
-    v[1] = (__bf16)b;
-    return __builtin_bit_cast(unsigned, v);
-}
-
-// One output column block of 32 head-dim values per lane pair: o[v] is element
-// p = 8*(v/4) + 4*half + v%4 of column l.  Writes p = 16*half .. 16*half+15 of row `yrow`
-// (yrow already points at the column's row and at head-dim offset 32*pb).
-template <typename TO> __device__ inline void store_column(TO *yrow, float (&o)[16], int half, int pvalid, bool row_ok);
-template <> __device__ inline void store_column<__bf16>(__bf16 *yrow, float (&o)[16], int half, int pvalid, bool row_ok) {
-    unsigned X[4], Y[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        X[k] = pack_bf16x2(o[2 * k], o[2 * k + 1]);          // p-groups 0 and 1 (v = 0..7)
-        Y[k] = pack_bf16x2(o[8 + 2 * k], o[8 + 2 * k + 1]);  // p-groups 2 and 3 (v = 8..15)
-    }
-#pragma unroll
-    for (int k = 0; k < 4; ++k) swap_halves(X[k], Y[k]);
-    if (row_ok) {
-        const int p0 = 16 * half;
-        if (p0 + 8 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0) = make_uint4(X[0], X[1], Y[0], Y[1]);
-        if (p0 + 16 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 8) = make_uint4(X[2], X[3], Y[2], Y[3]);
-    }
-}
-template <> __device__ inline void store_column<float>(float *yrow, float (&o)[16], int half, int pvalid, bool row_ok) {
-    unsigned X[8], Y[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        X[k] = __float_as_uint(o[k]);
-        Y[k] = __float_as_uint(o[8 + k]);
-    }
-#pragma unroll
-    for (int k = 0; k < 8; ++k) swap_halves(X[k], Y[k]);
-    if (row_ok) {
-        const int p0 = 16 * half;
-        if (p0 + 4 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0) = make_uint4(X[0], X[1], X[2], X[3]);
-        if (p0 + 8 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 4) = make_uint4(Y[0], Y[1], Y[2], Y[3]);
-        if (p0 + 12 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 8) = make_uint4(X[4], X[5], X[6], X[7]);
-        if (p0 + 16 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 12) = make_uint4(Y[4], Y[5], Y[6], Y[7]);
-    }
-}
-
 template <typename T, typename TO, int PB, int NK, int QB>  // Ppad = 32*PB >= P, N = 16*NK, Q = 32*QB
 __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >= 4) ? 3 : 2) void chunk_scan_kernel(
     const T *__restrict__ x, const T *__restrict__ Bm, const T *__restrict__ Cm, const float *__restrict__ dtcs,

@@ -186,6 +186,81 @@ template <int COLS> struct RowMajorTile {
     }
 };
 
+// ------------------------------------------------------------------------------------------
+// Wavefront inclusive scan in float64 (DPP data movement)
+// ------------------------------------------------------------------------------------------
+template <int CTRL, int ROWMASK> __device__ inline double dpp_move(double v) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROWMASK, 0xf, false);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROWMASK, 0xf, false);
+    return __hiloint2double(hi, lo);  // lanes the row mask disables, or with no source lane, get +0.0
+}
+// Inclusive sum across the 64 lanes with DPP data movement: shifts inside rows of 16, then the
+// row totals are broadcast into the following rows (row_bcast:15 / row_bcast:31).
+__device__ inline double wave_inclusive_scan(double v) {
+    v += dpp_move<0x111, 0xf>(v);  // row_shr:1
+    v += dpp_move<0x112, 0xf>(v);  // row_shr:2
+    v += dpp_move<0x114, 0xf>(v);  // row_shr:4
+    v += dpp_move<0x118, 0xf>(v);  // row_shr:8
+    v += dpp_move<0x142, 0xa>(v);  // row_bcast:15 -> rows 1,3
+    v += dpp_move<0x143, 0xc>(v);  // row_bcast:31 -> rows 2,3
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------
+// Output columns of a transposed 32x32 accumulator tile, stored 16 bytes at a time
+// ------------------------------------------------------------------------------------------
+__device__ inline void swap_halves(unsigned &x, unsigned &y) {
+    // x[lanes 32..63] <-> y[lanes 0..31]
+    const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+    x = r[0];
+    y = r[1];
+}
+__device__ inline unsigned pack_bf16x2(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+    bf16x2 v;
+    v[0] = (__bf16)a;
+    v[1] = (__bf16)b;
+    return __builtin_bit_cast(unsigned, v);
+}
+
+// One output column block of 32 head-dim values per lane pair: o[v] is element
+// p = 8*(v/4) + 4*half + v%4 of column l.  Writes p = 16*half .. 16*half+15 of row `yrow`
+// (yrow already points at the column's row and at head-dim offset 32*pb).
+template <typename TO> __device__ inline void store_column(TO *yrow, float (&o)[16], int half, int pvalid, bool row_ok);
+template <> __device__ inline void store_column<__bf16>(__bf16 *yrow, float (&o)[16], int half, int pvalid, bool row_ok) {
+    unsigned X[4], Y[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        X[k] = pack_bf16x2(o[2 * k], o[2 * k + 1]);          // p-groups 0 and 1 (v = 0..7)
+        Y[k] = pack_bf16x2(o[8 + 2 * k], o[8 + 2 * k + 1]);  // p-groups 2 and 3 (v = 8..15)
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) swap_halves(X[k], Y[k]);
+    if (row_ok) {
+        const int p0 = 16 * half;
+        if (p0 + 8 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0) = make_uint4(X[0], X[1], Y[0], Y[1]);
+        if (p0 + 16 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 8) = make_uint4(X[2], X[3], Y[2], Y[3]);
+    }
+}
+template <> __device__ inline void store_column<float>(float *yrow, float (&o)[16], int half, int pvalid, bool row_ok) {
+    unsigned X[8], Y[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        X[k] = __float_as_uint(o[k]);
+        Y[k] = __float_as_uint(o[8 + k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) swap_halves(X[k], Y[k]);
+    if (row_ok) {
+        const int p0 = 16 * half;
+        if (p0 + 4 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0) = make_uint4(X[0], X[1], X[2], X[3]);
+        if (p0 + 8 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 4) = make_uint4(Y[0], Y[1], Y[2], Y[3]);
+        if (p0 + 12 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 8) = make_uint4(X[4], X[5], X[6], X[7]);
+        if (p0 + 16 <= pvalid) *reinterpret_cast<uint4 *>(yrow + p0 + 12) = make_uint4(Y[4], Y[5], Y[6], Y[7]);
+    }
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, and
 // on gfx9 loads and stores share one counter, so it drains every outstanding global load -- among
 // them the next tile's prefetch, which must stay in flight across the barrier.  The tile loops

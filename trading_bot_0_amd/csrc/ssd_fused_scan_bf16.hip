@@ -1,0 +1,29 @@
+// One-pass forward, bf16 inputs and bf16 y; also the shape test and the entry the C ABI calls.
+#include "ssd_fused_scan.h"
+
+namespace ssd {
+
+hipError_t launch_fused_scan_y32(const ScanShape &, int, const void *, const void *, const float *, const void *,
+                                 const void *, const float *, const float *, void *, float *, hipStream_t);
+
+int fused_scan_waves(const ScanShape &s, int dtype) {
+    if (dtype == 0) return 0;                         // float inputs take the staged kernels
+    if (s.P % 32 != 0) return 0;
+    if (s.N != 32 && s.N != 64) return 0;             // the state block must fit the accumulators
+    if (s.Q != 64 && s.Q != 128) return 0;
+    const int units = (s.H / s.G) * (s.P / 32);
+    const int waves = (units % 8 == 0) ? 8 : ((units % 4 == 0) ? 4 : 0);
+    if (waves == 0 || fused_scan_lds_bytes(s.N, s.Q, waves) > kLdsLimitBytes) return 0;
+    return waves;
+}
+
+hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const void *dt, const float *A,
+                             const void *Bm, const void *Cm, const float *D, const float *init, void *y,
+                             float *final_states, hipStream_t st) {
+    const int waves = fused_scan_waves(s, dtype);
+    if (waves == 0) return hipErrorInvalidValue;
+    if (dtype == 2) return launch_fused_scan_y32(s, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
+    return fused_dispatch<__bf16>(s, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
+}
+
+}  // namespace ssd

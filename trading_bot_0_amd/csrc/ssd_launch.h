@@ -38,6 +38,12 @@ hipError_t launch_state_passing(const ScanShape &s, const float *states, const f
 hipError_t launch_chunk_scan(const ScanShape &s, int dtype, const void *x, const void *Bm,
                              const void *Cm, const float *dtcs, const float *prev, const float *D,
                              void *y, hipStream_t stream);
+// The whole forward in one pass (bf16 inputs): no workspace, nothing but x, dt, B, C read and y, final written.
+// fused_scan_waves is 0 when the shape cannot run there, else the waves per workgroup it would use.
+int fused_scan_waves(const ScanShape &s, int dtype);
+hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const void *dt, const float *A,
+                             const void *Bm, const void *Cm, const float *D, const float *init, void *y,
+                             float *final_states, hipStream_t stream);
 hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *x, const void *dt,
                        const float *A, const void *Bm, const void *Cm, const float *D, void *y,
                        hipStream_t stream);

@@ -19,24 +19,6 @@ namespace ssd {
 // 1e-5..1e-3 in the decay factor.  (hi_l - hi_s) + (lo_l - lo_s) keeps the difference good to
 // its own ulp.
 // ------------------------------------------------------------------------------------------
-template <int CTRL, int ROWMASK> __device__ inline double dpp_move(double v) {
-    int lo = __double2loint(v), hi = __double2hiint(v);
-    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROWMASK, 0xf, false);
-    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROWMASK, 0xf, false);
-    return __hiloint2double(hi, lo);  // lanes the row mask disables, or with no source lane, get +0.0
-}
-// Inclusive sum across the 64 lanes with DPP data movement: shifts inside rows of 16, then the
-// row totals are broadcast into the following rows (row_bcast:15 / row_bcast:31).
-__device__ inline double wave_inclusive_scan(double v) {
-    v += dpp_move<0x111, 0xf>(v);  // row_shr:1
-    v += dpp_move<0x112, 0xf>(v);  // row_shr:2
-    v += dpp_move<0x114, 0xf>(v);  // row_shr:4
-    v += dpp_move<0x118, 0xf>(v);  // row_shr:8
-    v += dpp_move<0x142, 0xa>(v);  // row_bcast:15 -> rows 1,3
-    v += dpp_move<0x143, 0xc>(v);  // row_bcast:31 -> rows 2,3
-    return v;
-}
-
 template <typename T, int EPL>  // EPL = elements per lane = max(Q/64, 1)
 __global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__ dt,
                                                            const float *__restrict__ A,

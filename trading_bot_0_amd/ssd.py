@@ -35,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "ssd_chunk_state_fwd",
     "ssd_state_passing_fwd",
     "ssd_chunk_state_passing_fwd",
+    "ssd_chunk_scan_onepass_fwd",
     "ssd_chunk_scan_stage_fwd",
     "ssd_step_fwd",
 )
@@ -88,6 +89,7 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_chunk_state_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P]
         lib.ssd_state_passing_fwd.argtypes = [POINTER(SsdDims), P, P, P, P, P, P]
         lib.ssd_chunk_state_passing_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P]
+        lib.ssd_chunk_scan_onepass_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
         for name in EXPORTED_SYMBOLS[2:]:
@@ -234,6 +236,41 @@ def ssd_chunk_scan(
     rc = lib.ssd_chunk_scan_fwd(byref(dims), code, x.data_ptr(), dt.data_ptr(), A.data_ptr(),
                                 Bm.data_ptr(), Cm.data_ptr(), _ptr(D), _ptr(initial_states), y.data_ptr(),
                                 _ptr(final), workspace.data_ptr(), workspace.numel(), _stream_ptr(x))
+    _check(lib, rc)
+    return y, final
+
+
+def ssd_chunk_scan_onepass(
+    x: torch.Tensor,
+    dt: torch.Tensor,
+    A: torch.Tensor,
+    Bm: torch.Tensor,
+    Cm: torch.Tensor,
+    D: Optional[torch.Tensor] = None,
+    chunk: int = 128,
+    initial_states: Optional[torch.Tensor] = None,
+    return_final_states: bool = True,
+    out: Optional[torch.Tensor] = None,
+    final_out: Optional[torch.Tensor] = None,
+    y_dtype: Optional[torch.dtype] = None,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """The forward as one kernel and one pass over the inputs (bf16 only, no workspace); same results
+    as ssd_chunk_scan, which takes this path by itself when the batch is large enough.  Raises
+    SsdError(unsupported) for shapes the one-pass kernel does not cover."""
+    lib = load_library()
+    dims = _scan_dims(x, Bm, chunk)
+    _validate_scan_inputs(x, dt, A, Bm, Cm, D, initial_states, dims)
+    code, y_dtype = _out_code(x, y_dtype)
+    y = torch.empty(x.shape, dtype=y_dtype, device=x.device) if out is None else out
+    _require(y, "out", x.shape, y_dtype)
+    final = None
+    if return_final_states:
+        shape = (dims.batch, dims.nheads, dims.headdim, dims.dstate)
+        final = torch.empty(shape, dtype=torch.float32, device=x.device) if final_out is None else final_out
+        _require(final, "final_out", shape, torch.float32)
+    rc = lib.ssd_chunk_scan_onepass_fwd(byref(dims), code, x.data_ptr(), dt.data_ptr(), A.data_ptr(),
+                                        Bm.data_ptr(), Cm.data_ptr(), _ptr(D), _ptr(initial_states),
+                                        y.data_ptr(), _ptr(final), _stream_ptr(x))
     _check(lib, rc)
     return y, final
 
