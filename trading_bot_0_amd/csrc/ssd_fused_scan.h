@@ -12,7 +12,8 @@
 //            decay tables in its private LDS rows (see below)
 //   phase 1  for each block of 32 output columns l (lb = 0 .. Q/32-1), yT[p,l] =
 //              E[l] * ( exp2(alpha[32 lb]) * (H . C^T)                     state readout
-//                       + sum_{s-blocks sb <= lb} xT . (B.C^T o F_lb) )    intra-chunk
+//                       + sum_{s-blocks sb < lb} xT . (B.C^T o F_lb) )     intra-chunk, below the diagonal
+//              + xT . (B.C^T o mask o E[l] F_lb)                           diagonal block
 //            with E[l] = exp2(alpha[l] - alpha[32 lb]) and F_lb[s] = exp2(alpha[32 lb] - alpha[s]) dt[s];
 //            + D x in the epilogue.  The state is the A operand straight from its accumulator
 //            registers (hi + lo bf16), in the register order of the accumulator, which fixes the
@@ -88,10 +89,29 @@ __device__ inline float readlane_f(float v, int src_lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
 }
 
+// hi + lo bf16 pairs of two products a0*f0 and a1*f1 (f = 1 to split plain values): hi is the product
+// rounded to bf16, lo the rounded remainder, which the fused multiply-add gets from the exact product.
+// Four VALU instructions per element: multiply, half a pack, one shift or mask, fma, half a pack.
+__device__ inline void split_pair(float a0, float f0, float a1, float f1, unsigned &hi, unsigned &lo) {
+    hi = pack_bf16x2(a0 * f0, a1 * f1);
+    asm("" : "+v"(hi));  // keep the packed pair as the source of both halves (else the low half is converted twice)
+    const float h0 = __uint_as_float(hi << 16), h1 = __uint_as_float(hi & 0xffff0000u);
+    lo = pack_bf16x2(__builtin_fmaf(a0, f0, -h0), __builtin_fmaf(a1, f1, -h1));
+}
+struct FragBits {  // an operand fragment as four packed pairs
+    unsigned u[4];
+    __device__ inline Frag<__bf16> frag() const {
+        typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+        u32x4 v = {u[0], u[1], u[2], u[3]};
+        Frag<__bf16> f;
+        f.v = __builtin_bit_cast(bf16x8, v);
+        return f;
+    }
+};
+
 constexpr float kFastDiagSpan = 120.f;  // log2-decay across a diagonal block up to which E*F is safe
 
-// Dynamic LDS of one workgroup: B and C tiles, one x tile per wave, (5 + Q/32) float rows and 16 block
-// scalars per wave.
+// LDS of one workgroup: B and C tiles, one x tile per wave, (5 + Q/32) float rows and 16 block scalars per wave.
 constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
     return (size_t)2 * Q * N * 2 + (size_t)waves * ((size_t)Q * 32 * 2 + (size_t)(5 + Q / 32) * Q * 4 + 64);
 }
@@ -104,21 +124,24 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     using T = __bf16;
     constexpr int N = 16 * NK, NB = NK / 2, Q = 32 * QB, nthr = 64 * WAVES;
     constexpr int EPL = Q >= 64 ? Q / 64 : 1;  // chunk positions per lane in the scan
-    constexpr int BSL = Q * N / 8;             // 16-byte pieces of a B (or C) tile
+    constexpr int BPR = N / 8;                 // 16-byte pieces per B (or C) row
+    constexpr int BSL = Q * BPR;               // pieces of a B (or C) tile
     constexpr int UBC = (BSL + nthr - 1) / nthr;
+    constexpr int BRP = nthr / BPR;            // B rows per pass of the workgroup (a multiple of 32)
     constexpr int XPR = WAVES * 4;             // 16-byte pieces of one timestep's x for the workgroup
-    constexpr int UX = Q * XPR / nthr;         // = Q / 16
+    constexpr int UX = Q / 16;                 // passes of 16 rows
+    static_assert(BRP % 32 == 0 && nthr / XPR == 16, "staging offsets rely on the swizzle period of 32 rows");
     using XT = ChunkTile<32>;
     using BT = ChunkTile<N>;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // static, so that LDS addresses are compile-time offsets
+    __shared__ __attribute__((aligned(16))) unsigned char smem[fused_scan_lds_bytes(N, Q, WAVES)];
     T *Bs = reinterpret_cast<T *>(smem);  // [Q][N]
     T *Cs = Bs + Q * N;                   // [Q][N]
     T *xs_all = Cs + Q * N;               // [WAVES][Q][32]
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63;
+    const int lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r = lane & 31, half = lane >> 5;
     T *xs = xs_all + wave * (Q * 32);
     float *wf = reinterpret_cast<float *>(xs_all + WAVES * Q * 32) + wave * ((5 + QB) * Q + 16);
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
@@ -144,16 +167,28 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     const double a_h = (double)A[h];
 
     // ---- registers holding the next chunk's inputs ----
-    // A thread's pieces sit at fixed 32-bit element offsets from the chunk's first row.
-    const int bc_row0 = tid / (N / 8), bc_off0 = bc_row0 * s.G * N + (tid % (N / 8)) * 8;
-    const int bc_step = (nthr / (N / 8)) * s.G * N, bc_rstep = nthr / (N / 8);
-    const int x_row0 = tid / XPR, x_off0 = x_row0 * HP + (tid % XPR) * 8, x_step = (nthr / XPR) * HP;
-    const int dt_off0 = lane * EPL * s.H;
+    // A thread's pieces sit at one fixed 32-bit element offset from a pointer that is uniform per pass.
+    // Offsets and LDS addresses are recomputed from the thread index where they are used (a few
+    // instructions per chunk) instead of being carried through the MFMA phases in registers; the
+    // empty asm keeps the compiler from hoisting them out of the chunk loop again.
+    // The same goes for every LDS address derived from the lane index: each phase starts from its own
+    // opaque copy, so its swizzled offsets live only as long as the phase (hoisted out of the chunk loop
+    // they would occupy a hundred registers through all phases).
+    auto opaque_tid = [&]() {
+        int t = tid;
+        asm volatile("" : "+v"(t));
+        return t;
+    };
     uint4 bq[UBC], cq[UBC], xq[UX];
     unsigned short dq[EPL];
     auto prefetch = [&](int c) {
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
+        const int tv = opaque_tid();
+        const int bc_row0 = tv / BPR, x_row0 = tv / XPR;
+        const unsigned bc_off0 = bc_row0 * s.G * N + (tv % BPR) * 8;
+        const unsigned x_off0 = x_row0 * HP + (tv % XPR) * 8;
+        const unsigned dt_off0 = (tv & 63) * EPL * s.H;
         const T *bp = Bb + (size_t)t0 * s.G * N, *cp = Cb + (size_t)t0 * s.G * N;
         const T *xp = xb + (size_t)t0 * HP, *dp = dtb + (size_t)t0 * s.H;
         // (a conditional expression over *ptr and a zero constant would become a load through a selected
@@ -166,35 +201,34 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         if (rows == Q) {
 #pragma unroll
             for (int u = 0; u < UBC; ++u) {
-                const bool ok = BSL % nthr == 0 || tid + u * nthr < BSL;
-                bq[u] = ld16(bp + bc_off0 + u * bc_step, ok);
-                cq[u] = ld16(cp + bc_off0 + u * bc_step, ok);
+                const bool ok = BSL % nthr == 0 || tv + u * nthr < BSL;
+                bq[u] = ld16(bp + (size_t)u * BRP * s.G * N + bc_off0, ok);
+                cq[u] = ld16(cp + (size_t)u * BRP * s.G * N + bc_off0, ok);
             }
 #pragma unroll
-            for (int u = 0; u < UX; ++u) xq[u] = *reinterpret_cast<const uint4 *>(xp + x_off0 + u * x_step);
+            for (int u = 0; u < UX; ++u) xq[u] = *reinterpret_cast<const uint4 *>(xp + (size_t)u * 16 * HP + x_off0);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
-                dq[e] = (Q >= 64 || lane < Q) ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
+                dq[e] = (Q >= 64 || (tv & 63) < Q) ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
         } else {  // ragged last chunk: rows past the sequence read as zero (dt = 0 makes them no-ops)
 #pragma unroll
             for (int u = 0; u < UBC; ++u) {
-                const bool ok = (BSL % nthr == 0 || tid + u * nthr < BSL) && bc_row0 + u * bc_rstep < rows;
-                bq[u] = ld16(bp + bc_off0 + u * bc_step, ok);
-                cq[u] = ld16(cp + bc_off0 + u * bc_step, ok);
+                const bool ok = (BSL % nthr == 0 || tv + u * nthr < BSL) && bc_row0 + u * BRP < rows;
+                bq[u] = ld16(bp + (size_t)u * BRP * s.G * N + bc_off0, ok);
+                cq[u] = ld16(cp + (size_t)u * BRP * s.G * N + bc_off0, ok);
             }
 #pragma unroll
-            for (int u = 0; u < UX; ++u)
-                xq[u] = ld16(xp + x_off0 + u * x_step, x_row0 + u * (nthr / XPR) < rows);
+            for (int u = 0; u < UX; ++u) xq[u] = ld16(xp + (size_t)u * 16 * HP + x_off0, x_row0 + u * 16 < rows);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
-                dq[e] = (lane * EPL + e < rows) ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
+                dq[e] = ((tv & 63) * EPL + e < rows) ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
         }
     };
 
     // ---- running state of this unit: st[nb][v] = H[p = r, n = 32 nb + 8 (v/4) + 4 half + v%4] ----
     f32x16 st[NB];
     {
-        const float *ib = init ? init + (((size_t)b * s.H + h) * s.P + pb * 32 + r) * N + 4 * half : nullptr;
+        const float *ib = init ? init + (((size_t)b * s.H + h) * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5) : nullptr;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
@@ -214,24 +248,35 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         const int rows = min(Q, s.L - t0);
         block_sync_lds();  // every wave is done reading the previous chunk's tiles
         // ---- registers -> LDS tiles ----
+        // where the pieces go: the swizzle repeats every 32 rows, so all passes of a thread share the
+        // offsets of its first (B, C) or first two (x: passes are 16 rows apart) rows
+        const int tw = opaque_tid();
+        int bw[2], xw[2][2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            bw[hf] = BT::off(tw / BPR, (tw % BPR) * 8 + 4 * hf);
+#pragma unroll
+            for (int par = 0; par < 2; ++par)
+                xw[par][hf] = ((tw % XPR) / 4) * (Q * 32) + XT::off(tw / XPR + 16 * par, ((tw % XPR) % 4) * 8 + 4 * hf);
+        }
 #pragma unroll
         for (int u = 0; u < UBC; ++u) {
-            const int idx = tid + u * nthr;
-            if (BSL % nthr == 0 || idx < BSL) {
-                const int row = idx / (N / 8), ch = idx % (N / 8);
-                BT::put16(Bs, row, ch * 8, bq[u]);
-                BT::put16(Cs, row, ch * 8, cq[u]);
+            if (BSL % nthr == 0 || tw + u * nthr < BSL) {
+                *reinterpret_cast<uint2 *>(Bs + bw[0] + u * BRP * N) = make_uint2(bq[u].x, bq[u].y);
+                *reinterpret_cast<uint2 *>(Bs + bw[1] + u * BRP * N) = make_uint2(bq[u].z, bq[u].w);
+                *reinterpret_cast<uint2 *>(Cs + bw[0] + u * BRP * N) = make_uint2(cq[u].x, cq[u].y);
+                *reinterpret_cast<uint2 *>(Cs + bw[1] + u * BRP * N) = make_uint2(cq[u].z, cq[u].w);
             }
         }
 #pragma unroll
         for (int u = 0; u < UX; ++u) {
-            const int idx = tid + u * nthr;
-            const int row = idx / XPR, piece = idx % XPR;
-            XT::put16(xs_all + (piece / 4) * (Q * 32), row, (piece % 4) * 8, xq[u]);
+            *reinterpret_cast<uint2 *>(xs_all + xw[u & 1][0] + (u >> 1) * 1024) = make_uint2(xq[u].x, xq[u].y);
+            *reinterpret_cast<uint2 *>(xs_all + xw[u & 1][1] + (u >> 1) * 1024) = make_uint2(xq[u].z, xq[u].w);
         }
         // ---- scan of dt*A over the chunk and the decay tables of this unit ----
-        float a_end;       // exp2(alpha[Q-1]): the chunk's total decay
+        float a_end;  // exp2(alpha[Q-1]): the chunk's total decay
         {
+            const int lane = tw & 63;
             constexpr double kLog2e = 1.4426950408889634;
             float dtv[EPL], hi[EPL], lo[EPL];
             double cs[EPL], run = 0.0;
@@ -289,17 +334,40 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 
         // ---- phase 1: outputs of this chunk from the state entering it ----
         {
+            const int lane = opaque_tid() & 63;
+            const int r = lane & 31, half = lane >> 5;
             Frag<T> Hhi[NK], Hlo[NK];
 #pragma unroll
             for (int kk = 0; kk < NK; ++kk) {
+                FragBits fh, fl;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    T vh, vl;
-                    Split<T>::split(st[kk / 2][8 * (kk % 2) + i], vh, vl);
-                    Hhi[kk].v[i] = vh;
-                    Hlo[kk].v[i] = vl;
+                for (int i = 0; i < 4; ++i) {
+                    const int v = 8 * (kk % 2) + 2 * i;
+                    split_pair(st[kk / 2][v], 1.f, st[kk / 2][v + 1], 1.f, fh.u[i], fl.u[i]);
                 }
+                Hhi[kk] = fh.frag();
+                Hlo[kk] = fl.frag();
             }
+            // masked, decayed scores of one s-block as hi/lo operands; fv = the block's four F vectors
+            auto make_m = [&](const f32x16 &sc, const float4 (&fv)[4], bool masked, Frag<T>(&mh)[2], Frag<T>(&ml)[2]) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    FragBits fh, fl;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {  // accumulator registers v = 8 j + 2 k, + 1
+                        const int v = 8 * j + 2 * k, vg = v / 4, i = v % 4;
+                        const float f0 = i == 0 ? fv[vg].x : fv[vg].z, f1 = i == 0 ? fv[vg].y : fv[vg].w;
+                        float s0 = sc[v], s1 = sc[v + 1];
+                        if (masked) {  // causal mask inside the diagonal block: row 8 vg + 4 half + i <= column r
+                            s0 = (8 * vg + 4 * half + i <= r) ? s0 : 0.f;
+                            s1 = (8 * vg + 4 * half + i + 1 <= r) ? s1 : 0.f;
+                        }
+                        split_pair(s0, f0, s1, f1, fh.u[k], fl.u[k]);
+                    }
+                    mh[j] = fh.frag();
+                    ml[j] = fl.frag();
+                }
+            };
 #pragma unroll 1
             for (int lb = 0; lb < QB; ++lb) {
                 const int l = lb * 32 + r;
@@ -316,131 +384,104 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
                 }
                 acc = acc * blk_s[lb];
                 const float *F_row = F_s + lb * Q;
-                auto scores = [&](int sb) {
+                // one s-block.  On the separable path the diagonal block is one more term of the sum that E[l]
+                // scales at the end; on the exact path the sum is scaled first and the block carries its full factors.
+                auto block = [&](int sb, bool diag) {
+                    Frag<T> Bf[NK];
+#pragma unroll
+                    for (int kk = 0; kk < NK; ++kk) Bf[kk] = BT::split_frag(Bs, sb * 32 + r, 16 * kk + 4 * half);
                     f32x16 sc = {0};
 #pragma unroll
-                    for (int kk = 0; kk < NK; ++kk)
-                        sc = mma32(BT::split_frag(Bs, sb * 32 + r, 16 * kk + 4 * half), Cf[kk], sc);
-                    return sc;
-                };
-                auto accumulate = [&](int sb, const Frag<T>(&mh)[2], const Frag<T>(&ml)[2]) {
+                    for (int kk = 0; kk < NK; ++kk) sc = mma32(Bf[kk], Cf[kk], sc);
+                    // requested while the score MFMAs run
+                    Frag<T> xf[2];
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)  // K order of mh[j]: rows 32 sb + 16 j + 4 half + {0..3} and the same + 8
+                        xf[j] = XT::frag(xs, sb * 32 + 16 * j + 4 * half, 8, 0, lane);
+                    float4 fv[4];
+                    if (!diag || fast) {
+#pragma unroll
+                        for (int vg = 0; vg < 4; ++vg) fv[vg] = *reinterpret_cast<const float4 *>(F_row + sb * 32 + 8 * vg + 4 * half);
+                    }
+                    float El = 1.f;
+                    if (diag) {
+                        El = E_s[l];
+                        if (!fast) {
+                            acc = acc * El;
+                            const float al_hi = ah_s[l], al_lo = alo_s[l];
+#pragma unroll
+                            for (int vg = 0; vg < 4; ++vg) {
+                                const int s0 = lb * 32 + 8 * vg + 4 * half;
+                                const float4 ah4 = *reinterpret_cast<const float4 *>(ah_s + s0);
+                                const float4 al4 = *reinterpret_cast<const float4 *>(alo_s + s0);
+                                const float4 dt4 = *reinterpret_cast<const float4 *>(dt_s + s0);
+                                // exponents clamped at 0: entries above the diagonal stay finite and are masked below
+                                fv[vg].x = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah4.x, al4.x), 0.f)) * dt4.x;
+                                fv[vg].y = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah4.y, al4.y), 0.f)) * dt4.y;
+                                fv[vg].z = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah4.z, al4.z), 0.f)) * dt4.z;
+                                fv[vg].w = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah4.w, al4.w), 0.f)) * dt4.w;
+                            }
+                        }
+                    }
+                    Frag<T> mh[2], ml[2];
+                    make_m(sc, fv, diag, mh, ml);
 #pragma unroll
                     for (int j = 0; j < 2; ++j) {
-                        // K order of mh[j]: rows s = 32 sb + 16 j + 4 half + {0..3} and the same + 8
-                        const Frag<T> xf = XT::frag(xs, sb * 32 + 16 * j + 4 * half, 8, 0, lane);
-                        acc = mma32(xf, mh[j], acc);
-                        acc = mma32(xf, ml[j], acc);
+                        acc = mma32(xf[j], mh[j], acc);
+                        acc = mma32(xf[j], ml[j], acc);
                     }
+                    if (diag && fast) acc = acc * El;  // everything summed so far shares the factor E[l]
                 };
-#pragma unroll 1
-                for (int sb = 0; sb < lb; ++sb) {
-                    const f32x16 sc = scores(sb);
-                    Frag<T> mh[2], ml[2];
+                // compile-time block index: every LDS address is a lane offset plus an immediate
+#pragma unroll
+                for (int sb = 0; sb < QB - 1; ++sb)
+                    if (sb < lb) block(sb, false);
+                block(lb, true);
+                // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]
+                {
+                    const int le = opaque_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
+                    float o[16];
 #pragma unroll
                     for (int vg = 0; vg < 4; ++vg) {
-                        const float4 f4 = *reinterpret_cast<const float4 *>(F_row + sb * 32 + 8 * vg + 4 * half);
-                        const float fv[4] = {f4.x, f4.y, f4.z, f4.w};
+                        const bf16x4 x4 = XT::row4(xs, ll, 8 * vg + 4 * he);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const int v = vg * 4 + i;
-                            T vh, vl;
-                            Split<T>::split(sc[v] * fv[i], vh, vl);
-                            mh[v / 8].v[v % 8] = vh;
-                            ml[v / 8].v[v % 8] = vl;
-                        }
+                        for (int i = 0; i < 4; ++i) o[vg * 4 + i] = acc[vg * 4 + i] + dh * (float)x4[i];
                     }
-                    accumulate(sb, mh, ml);
+                    store_column<TO>(yb + (size_t)(t0 + ll) * HP, o, he, 32, ll < rows);
                 }
-                {   // diagonal block
-                    const f32x16 sc = scores(lb);
-                    const float El = E_s[l];
-                    Frag<T> mh[2], ml[2];
-                    if (fast) {
-#pragma unroll
-                        for (int vg = 0; vg < 4; ++vg) {
-                            const float4 f4 = *reinterpret_cast<const float4 *>(F_row + lb * 32 + 8 * vg + 4 * half);
-                            const float fv[4] = {f4.x, f4.y, f4.z, f4.w};
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) {
-                                const int v = vg * 4 + i;
-                                const float wv = (8 * vg + 4 * half + i <= r) ? sc[v] * fv[i] : 0.f;
-                                T vh, vl;
-                                Split<T>::split(wv, vh, vl);
-                                mh[v / 8].v[v % 8] = vh;
-                                ml[v / 8].v[v % 8] = vl;
-                            }
-                        }
-                        accumulate(lb, mh, ml);
-                        acc = acc * El;
-                    } else {
-                        acc = acc * El;
-                        const float al_hi = ah_s[l], al_lo = alo_s[l];
-#pragma unroll
-                        for (int vg = 0; vg < 4; ++vg) {
-                            const int s0 = lb * 32 + 8 * vg + 4 * half;
-                            const float4 ah4 = *reinterpret_cast<const float4 *>(ah_s + s0);
-                            const float4 al4 = *reinterpret_cast<const float4 *>(alo_s + s0);
-                            const float4 dt4 = *reinterpret_cast<const float4 *>(dt_s + s0);
-                            const float ahv[4] = {ah4.x, ah4.y, ah4.z, ah4.w};
-                            const float alv[4] = {al4.x, al4.y, al4.z, al4.w};
-                            const float dtv4[4] = {dt4.x, dt4.y, dt4.z, dt4.w};
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) {
-                                const int v = vg * 4 + i;
-                                // masked entries get exp2(-inf) = 0: a select on the exponent
-                                const float arg = fminf(alpha_diff(al_hi, al_lo, ahv[i], alv[i]), 0.f);
-                                const float wv = exp2_hw((s0 + i <= l) ? arg : -INFINITY) * dtv4[i] * sc[v];
-                                T vh, vl;
-                                Split<T>::split(wv, vh, vl);
-                                mh[v / 8].v[v % 8] = vh;
-                                ml[v / 8].v[v % 8] = vl;
-                            }
-                        }
-                        accumulate(lb, mh, ml);
-                    }
-                }
-                // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]
-                float o[16];
-#pragma unroll
-                for (int vg = 0; vg < 4; ++vg) {
-                    const bf16x4 x4 = XT::row4(xs, l, 8 * vg + 4 * half);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) o[vg * 4 + i] = acc[vg * 4 + i] + dh * (float)x4[i];
-                }
-                store_column<TO>(yb + (size_t)(t0 + l) * HP, o, half, 32, l < rows);
             }
         }
 
         // ---- phase 2: the state leaving this chunk ----
         if (!EARLY && c + 1 < s.nc) prefetch(c + 1);
+        const int lane = opaque_tid() & 63, half = lane >> 5;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) st[nb] = st[nb] * a_end;
-#pragma unroll 2
+#pragma unroll
         for (int ks = 0; ks < Q; ks += 16) {
             const int k0 = ks + 8 * half;
             const Frag<T> xr = XT::frag(xs, k0, 4, 0, lane);  // x[l = k0..k0+7, p = r]
+            Frag<T> bf[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) bf[nb] = BT::frag(Bs, k0, 4, nb * 32, lane);  // B[l = k0..k0+7, n = 32 nb + r]
             const float4 wa = *reinterpret_cast<const float4 *>(w_s + k0);
             const float4 wb = *reinterpret_cast<const float4 *>(w_s + k0 + 4);
             const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
-            Frag<T> xh, xl;
+            FragBits xh, xl;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                T vh, vl;
-                Split<T>::split(wv[i] * (float)xr.v[i], vh, vl);
-                xh.v[i] = vh;
-                xl.v[i] = vl;
-            }
+            for (int i = 0; i < 4; ++i)
+                split_pair((float)xr.v[2 * i], wv[2 * i], (float)xr.v[2 * i + 1], wv[2 * i + 1], xh.u[i], xl.u[i]);
+            const Frag<T> xhf = xh.frag(), xlf = xl.frag();
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                const Frag<T> bf = BT::frag(Bs, k0, 4, nb * 32, lane);  // B[l = k0..k0+7, n = 32 nb + r]
-                st[nb] = mma32(bf, xh, st[nb]);
-                st[nb] = mma32(bf, xl, st[nb]);
+                st[nb] = mma32(bf[nb], xhf, st[nb]);
+                st[nb] = mma32(bf[nb], xlf, st[nb]);
             }
         }
     }
 
     if (final_states) {
-        float *fb = final_states + (((size_t)b * s.H + h) * s.P + pb * 32 + r) * N + 4 * half;
+        float *fb = final_states + (((size_t)b * s.H + h) * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
@@ -459,12 +500,9 @@ static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt
                                const void *Cm, const float *D, const float *init, void *y, float *final_states,
                                hipStream_t st) {
     constexpr bool EARLY = false;
-    const size_t lds = fused_scan_lds_bytes(16 * NK, 32 * QB, WAVES);
-    hipError_t e = allow_lds(fused_scan_kernel<TO, NK, QB, WAVES, EARLY>, lds);
-    if (e != hipSuccess) return e;
     const int units = (s.H / s.G) * (s.P / 32);
     const int grid = s.B * s.G * (units / WAVES);
-    fused_scan_kernel<TO, NK, QB, WAVES, EARLY><<<dim3(grid), dim3(64 * WAVES), lds, st>>>(
+    fused_scan_kernel<TO, NK, QB, WAVES, EARLY><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
         static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
         static_cast<const __bf16 *>(Cm), D, init, static_cast<TO *>(y), final_states, s);
     return hipGetLastError();
