@@ -123,6 +123,10 @@ int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, c
                                const void *Bm, const void *Cm, const float *D, const float *initial_states,
                                void *y, float *final_states, void *hip_stream);
 
+/* *is_onepass = 1 if ssd_chunk_scan_fwd runs these dims as the one-pass kernel (its workspace is then not
+ * touched), 0 if as the staged kernels.  A plan query like ssd_workspace_bytes; no reference counterpart. */
+int ssd_chunk_scan_is_onepass(const ssd_dims *dims, int dtype, int *is_onepass);
+
 /* Stage 3: sequential recurrence over chunks.  prev_states[c] receives the state entering
  * chunk c and may alias chunk_states (in place); final_states and initial_states may be NULL
  * and may alias each other. */

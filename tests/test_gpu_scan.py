@@ -219,3 +219,17 @@ def test_policy_shape_full_size_properties():
     assert torch.equal(y1, y[:, :h]), "first half does not depend on the future"
     assert ((y2.float() - y[:, h:].float()).abs() <= 2.0 ** -7 * y[:, h:].float().abs() + 1e-3).all()
     assert rel_err(f2, np64(final)) <= 1e-4
+
+
+def test_prepared_call_matches_the_plain_call():
+    from trading_bot_0_amd import PreparedChunkScan
+    w = WORKLOADS["policy_bf16"].with_batch(3)
+    dev = to_dev(make_inputs(w, seed=4, seqlen=500))
+    y0, f0 = run(dev, w.chunk)
+    call = PreparedChunkScan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk)
+    for _ in range(3):          # same buffers every time
+        y1, f1 = call()
+        torch.cuda.synchronize()
+        assert torch.equal(y0, y1) and torch.equal(f0, f1)
+    with pytest.raises(ValueError):
+        PreparedChunkScan(dev["x"], dev["dt"][:, :-1], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk)

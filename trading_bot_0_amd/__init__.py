@@ -1,6 +1,7 @@
 """MI355X-native Mamba-2 SSD chunk-scan forward and streaming step (hand-written gfx950 HIP
 kernels behind the C ABI in include/ssd_hip.h)."""
 from .ssd import (  # noqa: F401
+    PreparedChunkScan,
     SsdError,
     chunk_cumsum,
     chunk_scan_stage,

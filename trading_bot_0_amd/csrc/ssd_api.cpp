@@ -111,6 +111,10 @@ Workspace carve(const ssd::ScanShape &s) {
     return w;
 }
 
+bool takes_one_pass(const ssd::ScanShape &s, int dtype) {
+    return ssd::fused_scan_waves(s, dtype) == 8 && (int64_t)s.B * s.H * (s.P / 32) / 8 >= kOnePassMinWorkgroups;
+}
+
 int hip_fail(hipError_t e, const char *what) {
     return fail(SSD_ERR_RUNTIME, "ssd: %s failed: %s", what, hipGetErrorString(e));
 }
@@ -230,8 +234,7 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
     float *states = reinterpret_cast<float *>(base + w.st_off);
     hipStream_t st = (hipStream_t)hip_stream;
     hipError_t e;
-    if (ssd::fused_scan_waves(s, dtype) == 8 &&
-        (int64_t)s.B * s.H * (s.P / 32) / 8 >= kOnePassMinWorkgroups) {
+    if (takes_one_pass(s, dtype)) {
         e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, y, final_states, st);
         return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
     }
@@ -249,6 +252,14 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
     }
     e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dtcs, states, D, y, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_scan launch");
+    return SSD_OK;
+}
+
+int ssd_chunk_scan_is_onepass(const ssd_dims *dims, int dtype, int *is_onepass) {
+    if (is_onepass == nullptr) return fail(SSD_ERR_INVALID, "ssd: is_onepass must not be NULL");
+    ssd::ScanShape s;
+    if (int rc = make_shape(dims, dtype, &s)) return rc;
+    *is_onepass = takes_one_pass(s, dtype) ? 1 : 0;
     return SSD_OK;
 }
 

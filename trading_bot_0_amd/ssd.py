@@ -36,6 +36,7 @@ EXPORTED_SYMBOLS = (
     "ssd_state_passing_fwd",
     "ssd_chunk_state_passing_fwd",
     "ssd_chunk_scan_onepass_fwd",
+    "ssd_chunk_scan_is_onepass",
     "ssd_chunk_scan_stage_fwd",
     "ssd_step_fwd",
 )
@@ -90,6 +91,7 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_state_passing_fwd.argtypes = [POINTER(SsdDims), P, P, P, P, P, P]
         lib.ssd_chunk_state_passing_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P]
         lib.ssd_chunk_scan_onepass_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P]
+        lib.ssd_chunk_scan_is_onepass.argtypes = [POINTER(SsdDims), c_int, POINTER(c_int)]
         lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
         for name in EXPORTED_SYMBOLS[2:]:
@@ -238,6 +240,57 @@ def ssd_chunk_scan(
                                 _ptr(final), workspace.data_ptr(), workspace.numel(), _stream_ptr(x))
     _check(lib, rc)
     return y, final
+
+
+class PreparedChunkScan:
+    """ssd_chunk_scan with everything but the launch done once: shapes validated, outputs and workspace
+    allocated, argument pointers fixed.  Calling it launches the forward on the current stream of the
+    inputs' device and returns (y, final_states); the tensors it was built from must stay alive and in
+    place.  For loops that call the op with the same buffers (benchmarks, graph capture, a serving loop):
+    per call it costs one foreign call, where ssd_chunk_scan spends tens of microseconds in Python."""
+
+    def __init__(self, x, dt, A, Bm, Cm, D=None, chunk=128, initial_states=None, return_final_states=True,
+                 workspace=None, out=None, final_out=None, y_dtype=None):
+        self._lib = load_library()
+        self._dims = _scan_dims(x, Bm, chunk)
+        dims = self._dims
+        _validate_scan_inputs(x, dt, A, Bm, Cm, D, initial_states, dims)
+        self._code, y_dtype = _out_code(x, y_dtype)
+        self.y = torch.empty(x.shape, dtype=y_dtype, device=x.device) if out is None else out
+        _require(self.y, "out", x.shape, y_dtype)
+        self.final = None
+        if return_final_states:
+            shape = (dims.batch, dims.nheads, dims.headdim, dims.dstate)
+            self.final = torch.empty(shape, dtype=torch.float32, device=x.device) if final_out is None else final_out
+            _require(self.final, "final_out", shape, torch.float32)
+        need = c_size_t(0)
+        _check(self._lib, self._lib.ssd_workspace_bytes(byref(dims), byref(need)))
+        if workspace is None:
+            workspace = torch.empty(need.value, dtype=torch.uint8, device=x.device)
+        elif (not workspace.is_cuda) or workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+            raise ValueError("SSD workspace must be a contiguous uint8 GPU tensor")
+        self._keep = (x, dt, A, Bm, Cm, D, initial_states, workspace)
+        self._device = x.device
+        self._args = (x.data_ptr(), dt.data_ptr(), A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), _ptr(D),
+                      _ptr(initial_states), self.y.data_ptr(), _ptr(self.final), workspace.data_ptr(),
+                      workspace.numel())
+
+    def __call__(self):
+        rc = self._lib.ssd_chunk_scan_fwd(byref(self._dims), self._code, *self._args,
+                                          torch.cuda.current_stream(self._device).cuda_stream)
+        if rc:
+            _check(self._lib, rc)
+        return self.y, self.final
+
+
+def chunk_scan_is_onepass(batch, seqlen, nheads, headdim, dstate, ngroups, chunk, dtype=torch.bfloat16) -> bool:
+    """Whether ssd_chunk_scan runs this shape as the one-pass kernel (True) or as the staged kernels."""
+    lib = load_library()
+    dims = SsdDims(batch, seqlen, nheads, headdim, dstate, ngroups, chunk)
+    flag = c_int(0)
+    code = SSD_DTYPE_BF16 if dtype == torch.bfloat16 else SSD_DTYPE_F32
+    _check(lib, lib.ssd_chunk_scan_is_onepass(byref(dims), code, byref(flag)))
+    return bool(flag.value)
 
 
 def ssd_chunk_scan_onepass(
