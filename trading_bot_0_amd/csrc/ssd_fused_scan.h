@@ -112,8 +112,12 @@ struct FragBits {  // an operand fragment as four packed pairs
 constexpr float kFastDiagSpan = 120.f;  // log2-decay across a diagonal block up to which E*F is safe
 
 // LDS of one workgroup: B and C tiles, one x tile per wave, (5 + Q/32) float rows and 16 block scalars per wave.
+// Consecutive x tiles start 32 bytes (8 banks) apart modulo the bank width, so the staging writes, which hit
+// the same row and column of all tiles at once, do not collide.
+constexpr int fused_scan_xtile_elems(int Q) { return Q * 32 + 16; }
 constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
-    return (size_t)2 * Q * N * 2 + (size_t)waves * ((size_t)Q * 32 * 2 + (size_t)(5 + Q / 32) * Q * 4 + 64);
+    return (size_t)2 * Q * N * 2 +
+           (size_t)waves * ((size_t)fused_scan_xtile_elems(Q) * 2 + (size_t)(5 + Q / 32) * Q * 4 + 64);
 }
 
 template <typename TO, int NK, int QB, int WAVES, bool EARLY>  // N = 16*NK, Q = 32*QB
@@ -137,13 +141,14 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     __shared__ __attribute__((aligned(16))) unsigned char smem[fused_scan_lds_bytes(N, Q, WAVES)];
     T *Bs = reinterpret_cast<T *>(smem);  // [Q][N]
     T *Cs = Bs + Q * N;                   // [Q][N]
-    T *xs_all = Cs + Q * N;               // [WAVES][Q][32]
+    T *xs_all = Cs + Q * N;               // [WAVES][Q][32] (+16 elements between tiles)
+    constexpr int XS = fused_scan_xtile_elems(Q);
 
     const int tid = threadIdx.x;
     const int lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    T *xs = xs_all + wave * (Q * 32);
-    float *wf = reinterpret_cast<float *>(xs_all + WAVES * Q * 32) + wave * ((5 + QB) * Q + 16);
+    T *xs = xs_all + wave * XS;
+    float *wf = reinterpret_cast<float *>(xs_all + WAVES * XS) + wave * ((5 + QB) * Q + 16);
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
     float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [8..8+QB): log2-decay across block lb
 
@@ -257,7 +262,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
             bw[hf] = BT::off(tw / BPR, (tw % BPR) * 8 + 4 * hf);
 #pragma unroll
             for (int par = 0; par < 2; ++par)
-                xw[par][hf] = ((tw % XPR) / 4) * (Q * 32) + XT::off(tw / XPR + 16 * par, ((tw % XPR) % 4) * 8 + 4 * hf);
+                xw[par][hf] = ((tw % XPR) / 4) * XS + XT::off(tw / XPR + 16 * par, ((tw % XPR) % 4) * 8 + 4 * hf);
         }
 #pragma unroll
         for (int u = 0; u < UBC; ++u) {
