@@ -64,11 +64,16 @@ template <int COLS> struct ChunkTile {  // bf16 [rows][COLS], COLS = 32 or 64
     }
     // this lane's 4 elements tile[k0 + 0..3][c0 + lane%32] (k0 a multiple of 4 that already includes
     // the lane half's K offset): K-consecutive data for operand row/column c0 + lane%32
-    static __device__ inline bf16x4 tr4(const __bf16 *tile, int k0, int c0, int lane) {
+    static __device__ inline int tr_off(int k0, int c0, int lane) {  // element offset this lane hands to the read
         const int q = lane >> 4, a = (lane >> 2) & 3, b = lane & 3;
-        const __bf16 *src = tile + off(k0 + a, c0 + 16 * (q & 1) + 4 * b);
+        return off(k0 + a, c0 + 16 * (q & 1) + 4 * b);
+    }
+    static __device__ inline bf16x4 tr_read(const __bf16 *src) {
         const bf16x4_gcc v = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SSD_LDS_AS bf16x4_gcc *)(src));
         return __builtin_bit_cast(bf16x4, v);
+    }
+    static __device__ inline bf16x4 tr4(const __bf16 *tile, int k0, int c0, int lane) {
+        return tr_read(tile + tr_off(k0, c0, lane));
     }
     static __device__ inline Frag<__bf16> frag(const __bf16 *tile, int k0, int gap, int c0, int lane) {
         Frag<__bf16> fr;
@@ -462,13 +467,33 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         const int lane = opaque_tid() & 63, half = lane >> 5;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) st[nb] = st[nb] * a_end;
+        // Offsets of this lane's transposing reads for K steps 0 and 1.  Both swizzles repeat every 32 rows, so
+        // step i reads at the offset of step i%2 plus (i/2)*32 rows: immediates after unrolling.
+        int xo[2][2], bo[2][2][NB];
+#pragma unroll
+        for (int par = 0; par < 2; ++par) {
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                xo[par][z] = XT::tr_off(16 * par + 8 * half + 4 * z, 0, lane);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) bo[par][z][nb] = BT::tr_off(16 * par + 8 * half + 4 * z, nb * 32, lane);
+            }
+        }
+        auto join = [](const bf16x4 &lo, const bf16x4 &hi) {
+            Frag<T> fr;
+            fr.v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            return fr;
+        };
 #pragma unroll
         for (int ks = 0; ks < Q; ks += 16) {
             const int k0 = ks + 8 * half;
-            const Frag<T> xr = XT::frag(xs, k0, 4, 0, lane);  // x[l = k0..k0+7, p = r]
+            const int par = (ks / 16) & 1, rb = (ks / 32) * 32;
+            // x[l = k0..k0+7, p = r] and B[l = k0..k0+7, n = 32 nb + r]
+            const Frag<T> xr = join(XT::tr_read(xs + xo[par][0] + rb * 32), XT::tr_read(xs + xo[par][1] + rb * 32));
             Frag<T> bf[NB];
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) bf[nb] = BT::frag(Bs, k0, 4, nb * 32, lane);  // B[l = k0..k0+7, n = 32 nb + r]
+            for (int nb = 0; nb < NB; ++nb)
+                bf[nb] = join(BT::tr_read(Bs + bo[par][0][nb] + rb * N), BT::tr_read(Bs + bo[par][1][nb] + rb * N));
             const float4 wa = *reinterpret_cast<const float4 *>(w_s + k0);
             const float4 wb = *reinterpret_cast<const float4 *>(w_s + k0 + 4);
             const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
