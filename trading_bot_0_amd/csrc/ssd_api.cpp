@@ -279,8 +279,8 @@ int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, c
     OPTIONAL_PTR(final_states);
     if (ssd::fused_scan_waves(s, dtype) == 0)
         return fail(SSD_ERR_UNSUPPORTED,
-                    "ssd: the one-pass scan needs bf16 inputs, headdim a multiple of 32, dstate 32 or 64, chunk 64 "
-                    "or 128 and (nheads/ngroups)*(headdim/32) a multiple of 4");
+                    "ssd: the one-pass scan needs bf16 inputs, headdim a multiple of 32, dstate 32 or 64 and "
+                    "(nheads/ngroups)*(headdim/32) a multiple of 4");
     hipError_t e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, y, final_states,
                                           (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");

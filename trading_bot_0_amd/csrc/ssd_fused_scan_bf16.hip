@@ -10,10 +10,9 @@ int fused_scan_waves(const ScanShape &s, int dtype) {
     if (dtype == 0) return 0;                         // float inputs take the staged kernels
     if (s.P % 32 != 0) return 0;
     if (s.N != 32 && s.N != 64) return 0;             // the state block must fit the accumulators
-    if (s.Q != 64 && s.Q != 128) return 0;
     const int units = (s.H / s.G) * (s.P / 32);
     const int waves = (units % 8 == 0) ? 8 : ((units % 4 == 0) ? 4 : 0);
-    if (waves == 0 || fused_scan_lds_bytes(s.N, s.Q, waves) > kLdsLimitBytes) return 0;
+    if (waves == 0 || fused_scan_lds_bytes(s.N, kOnePassTile, waves) > kLdsLimitBytes) return 0;
     return waves;
 }
 
@@ -22,8 +21,11 @@ hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const
                              float *final_states, hipStream_t st) {
     const int waves = fused_scan_waves(s, dtype);
     if (waves == 0) return hipErrorInvalidValue;
-    if (dtype == 2) return launch_fused_scan_y32(s, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
-    return fused_dispatch<__bf16>(s, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
+    ScanShape t = s;  // the kernel's own tiling of time; the caller's chunk length does not enter
+    t.Q = kOnePassTile;
+    t.nc = (s.L + kOnePassTile - 1) / kOnePassTile;
+    if (dtype == 2) return launch_fused_scan_y32(t, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
+    return fused_dispatch<__bf16>(t, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
 }
 
 }  // namespace ssd
