@@ -184,15 +184,15 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 
     // ---- registers holding the next chunk's inputs ----
     // A thread's pieces sit at one fixed 32-bit element offset from a pointer that is uniform per pass.
-    // Offsets and LDS addresses are recomputed from the thread index where they are used (a few
-    // instructions per chunk) instead of being carried through the MFMA phases in registers; the
-    // empty asm keeps the compiler from hoisting them out of the chunk loop again.
-    // The same goes for every LDS address derived from the lane index: each phase starts from its own
-    // opaque copy, so its swizzled offsets live only as long as the phase (hoisted out of the chunk loop
-    // they would occupy a hundred registers through all phases).
-    auto opaque_tid = [&]() {
+    // Tiles of 64 steps leave room for every lane-derived offset and LDS address to stay in registers for
+    // the whole kernel.  Longer tiles do not: there the offsets are recomputed where they are used, from a
+    // copy of the thread index that an empty asm hides from the compiler, so that it cannot hoist them out
+    // of the tile loop again (hoisted, they held about a hundred registers through all phases and forced
+    // spills whose reloads, each an s_waitcnt vmcnt(0), serialised the prefetch).
+    constexpr bool kRecomputeOffsets = QB > 2;
+    auto phase_tid = [&]() {
         int t = tid;
-        asm volatile("" : "+v"(t));
+        if (kRecomputeOffsets) asm volatile("" : "+v"(t));
         return t;
     };
     uint4 bq[UBC], cq[UBC], xq[UX];
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     auto prefetch = [&](int c) {
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
-        const int tv = opaque_tid();
+        const int tv = phase_tid();
         const int bc_row0 = tv / BPR, x_row0 = tv / XPR;
         const unsigned bc_off0 = bc_row0 * s.G * N + (tv % BPR) * 8;
         const unsigned x_off0 = x_row0 * HP + (tv % XPR) * 8;
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         // ---- registers -> LDS tiles ----
         // where the pieces go: the swizzle repeats every 32 rows, so all passes of a thread share the
         // offsets of its first (B, C) or first two (x: passes are 16 rows apart) rows
-        const int tw = opaque_tid();
+        const int tw = phase_tid();
         int bw[2], xw[2][2];
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 
         // ---- phase 1: outputs of this chunk from the state entering it ----
         {
-            const int lane = opaque_tid() & 63;
+            const int lane = phase_tid() & 63;
             const int r = lane & 31, half = lane >> 5;
             Frag<T> Hhi[NK], Hlo[NK];
 #pragma unroll
@@ -455,7 +455,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
                 block(lb, true);
                 // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]
                 {
-                    const int le = opaque_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
+                    const int le = phase_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
                     float o[16];
 #pragma unroll
                     for (int vg = 0; vg < 4; ++vg) {
@@ -470,7 +470,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 
         // ---- phase 2: the state leaving this chunk ----
         if (!EARLY && c + 1 < s.nc) prefetch(c + 1);
-        const int lane = opaque_tid() & 63, half = lane >> 5;
+        const int lane = phase_tid() & 63, half = lane >> 5;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) st[nb] = st[nb] * a_end;
         // Offsets of this lane's transposing reads for K steps 0 and 1.  Both swizzles repeat every 32 rows, so
