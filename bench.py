@@ -16,6 +16,8 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
   stages       the staged kernels issued one by one through their own entry points, each with
                its algorithmic bytes, GB/s and (stages 2, 4) dense MFMA rate; measured in both cases
   stream_step  the single-timestep update at batch 4096: latency and GB/s
+  reference_suite  the reference's historical benchmark cases for this path (batch 4, seq_len 4096,
+               BFloat16), for the SSD op alone, in the reference's result schema
   cpu_baseline the plain-C oracle (sequential recurrence, float32, OpenMP) timed on this
                box's host cores on a bounded batch slice of the same workload
 
@@ -47,6 +49,7 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-stream-step", action="store_true")
+    ap.add_argument("--no-reference-suite", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise kernel over 256 MiB in / 256 MiB out three times, the known-size "
@@ -234,6 +237,35 @@ def main():
         out["stream_step"] = {"batch": sw.batch, "steps": sw.stream_steps, "us_per_step": round(us, 2),
                               "alg_bytes": step_bytes(sw), "GBps": round(gbs, 1),
                               "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
+
+    # ---- the reference's own benchmark cases for this path ------------------------------------
+    # benchmark_results/bench_20260112_070055.json:5-41 lists mamba2_forward_train, mamba2_infer_prefill and
+    # mamba2_infer_step at batch 4, seq_len 4096 (1 for the step), BFloat16, in the schema of
+    # benchmarks/src/results.rs:8-29.  The same cases for the SSD op (the block around it is not part of this
+    # library; head sizes as in the policy shape), same schema; mamba2_fwd_bwd_train needs a backward pass.
+    if not args.no_reference_suite:
+        rw = WORKLOADS["policy_bf16"].with_batch(4)
+        ri = make_inputs(rw, seed=0, device="cuda", seqlen=4096)
+        rf = ssd.PreparedChunkScan(ri["x"], ri["dt"], ri["A"], ri["B"], ri["C"], ri["D"], chunk=rw.chunk)
+        for _ in range(20):
+            rf()
+        t_fwd = wall_time_steps(rf, 200, torch) * 1e3
+        rstate = rf.final.clone()
+        step_args = [ri[k][:, 0].contiguous() for k in ("x", "dt", "B", "C")]
+        ry = torch.empty_like(step_args[0])
+
+        def rstep():
+            ssd.ssd_step(rstate, step_args[0], step_args[1], ri["A"], step_args[2], step_args[3], ri["D"], out=ry)
+
+        for _ in range(20):
+            rstep()
+        t_step = wall_time_steps(rstep, 500, torch) * 1e3
+        cfg = {"batch": 4, "seq_len": 4096, "dtype": "BFloat16"}
+        out["reference_suite"] = [
+            {"name": "mamba2_forward_train", "time_ms": t_fwd, "config": cfg},
+            {"name": "mamba2_infer_prefill", "time_ms": t_fwd, "config": cfg},
+            {"name": "mamba2_infer_step", "time_ms": t_step, "config": {"batch": 4, "seq_len": 1, "dtype": "BFloat16"}},
+        ]
 
     # ---- CPU baseline: the C oracle on a bounded batch slice ---------------------------------
     if not args.no_cpu_baseline:
