@@ -8,11 +8,15 @@
 // score matrix never leaves registers; the A operand xT is read from LDS in the matching K
 // order.  C fragments for the wave's 32 columns stay in registers for both products.
 //
-// Decay factors.  Only the diagonal block (sb == lb) needs a mask and one exp2 per element
-// (mask before exp2: no inf*0).  Below the diagonal the factor separates through the first
-// row m = 32*lb of the column block, exp2(alpha[l]-alpha[s]) = exp2(alpha[l]-alpha[m]) *
-// exp2(alpha[m]-alpha[s]) with both exponents <= 0: one value per lane times a per-row table
-// (dt folded in) that the workgroup builds once in LDS.
+// Decay factors.  The factor separates through the first row m = 32*lb of the column block,
+// exp2(alpha[l]-alpha[s]) dt[s] = E[l] F_lb[s],  E[l] = exp2(alpha[l]-alpha[m]),
+// F_lb[s] = exp2(alpha[m]-alpha[s]) dt[s]: a score element costs one multiply by a per-row table
+// value (the workgroup builds the table once per tile in LDS), and everything summed for a column
+// is scaled by E[l] once at the end.  Below the diagonal both exponents are <= 0.  On the
+// diagonal block (plus the causal mask) the table exponent is >= 0, which is safe as long as the
+// block's total log2-decay stays below 120; a block that decays more takes the exact path, one
+// exp2 of the hi/lo difference per element, after the sum so far has been scaled.  The choice is
+// uniform per wave.
 //
 // In bf16 mode the two operands this kernel manufactures in fp32 -- M and the entering state
 // Hc -- are fed to the MFMA as hi + lo bf16 pairs; x, B and C enter exactly as given.
@@ -49,7 +53,7 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
     using XT = RowMajorTile<Ppad>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *al_s = reinterpret_cast<float *>(smem);  // [3][Q]: alpha hi, alpha lo, dt
-    float *tab = al_s + 3 * Q;                      // [nblk][Q]: exp2(alpha[32k]-alpha[s])*dt[s], s < 32k
+    float *tab = al_s + 3 * Q;                      // [nblk][Q]: F_k[s] = exp2(alpha[32k]-alpha[s])*dt[s], s < 32(k+1)
     T *Bs = reinterpret_cast<T *>(tab + nblk * Q);  // [Q][ldb]
     T *Hs = Bs + Q * ldb;                           // [PARTS][Ppad][ldb]
     T *xs = Hs + PARTS * Ppad * ldb;                // bf16: [Q][Ppad] row-major; float: [Ppad][ldx]
@@ -168,26 +172,29 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
             for (int idx = UH * nthr + tid; idx < htotal; idx += nthr) put_state(idx, hp[idx]);
         }
         block_sync_lds();  // alpha and dt are visible
-        // decay table rows k = 1..nblk-1 (row 0 is never read)
-        if constexpr (nblk > 1) {
+        // decay table: row k holds F_k[s] for the rows at or below column block k
 #pragma unroll
-            for (int i = 0; i < (nblk * Q) / nthr; ++i) {
-                const int idx = i * nthr + tid;
-                const int k = idx / Q, sr = idx % Q;
-                if (k > 0 && sr < 32 * k) {
-                    const float d = alpha_diff(ah_s[32 * k], alo_s[32 * k], ah_s[sr], alo_s[sr]);
-                    tab[idx] = exp2_hw(fminf(d, 0.f)) * dt_s[sr];
-                }
+        for (int i = 0; i < (nblk * Q + nthr - 1) / nthr; ++i) {
+            const int idx = i * nthr + tid;
+            const int k = idx / Q, sr = idx % Q;
+            if (idx < nblk * Q && sr < 32 * (k + 1)) {
+                const float d = alpha_diff(ah_s[32 * k], alo_s[32 * k], ah_s[sr], alo_s[sr]);
+                tab[idx] = exp2_hw(fminf(d, 126.f)) * dt_s[sr];
             }
         }
         if (sched.has_next()) prefetch(sched.next_logical());
         block_sync_lds();
 
         const float al_hi = ah_s[l], al_lo = alo_s[l];
+        const float rf_hi = ah_s[32 * lb], rf_lo = alo_s[32 * lb];   // alpha at the column block's first row
+        const float El = exp2_hw(fminf(alpha_diff(al_hi, al_lo, rf_hi, rf_lo), 0.f));
+        // non-negative floats order like their bit patterns: a scalar compare
+        const float span = fmaxf(alpha_diff(rf_hi, rf_lo, ah_s[32 * lb + 31], alo_s[32 * lb + 31]), 0.f);
+        const bool fast = __builtin_amdgcn_readfirstlane(__float_as_int(span)) <= __float_as_int(120.f);
         f32x16 accY[PB];
-        // state readout, scaled per output column by exp2(alpha[l]) (alpha <= 0)
+        // state readout, brought to the column block's first row (alpha <= 0)
         {
-            const float el = exp2_hw(al_hi + al_lo);
+            const float g0 = exp2_hw(rf_hi + rf_lo);
 #pragma unroll
             for (int pb = 0; pb < PB; ++pb) {
                 f32x16 a = {0};
@@ -197,55 +204,53 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
                     a = mma32(load_frag(hrow + kk * 16), Cf[kk], a);
                     if (PARTS == 2) a = mma32(load_frag(hrow + Ppad * ldb + kk * 16), Cf[kk], a);
                 }
-                accY[pb] = a * el;
+                accY[pb] = a * g0;
             }
         }
         // intra-chunk: s-blocks at or below this wave's column block (causal)
-        const float lane_dec = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah_s[32 * lb], alo_s[32 * lb]), 0.f));
         const float *tab_row = tab + lb * Q;
         for (int sb = 0; sb <= lb; ++sb) {
             f32x16 sc = {0};
             const T *brow = Bs + (sb * 32 + r) * ldb + half * 8;
 #pragma unroll
             for (int kk = 0; kk < NK; ++kk) sc = mma32(load_frag(brow + kk * 16), Cf[kk], sc);
-            Frag<T> mh[2], ml[2];
-            if (sb < lb) {
+            const bool diag = sb == lb;
+            float fv[16];
+            if (!diag || fast) {
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
-                    const int s0 = sb * 32 + 8 * vg + 4 * half;
-                    const float4 t4 = *reinterpret_cast<const float4 *>(tab_row + s0);
-                    const float tv[4] = {t4.x, t4.y, t4.z, t4.w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int v = vg * 4 + i;
-                        T hi, lo;
-                        Split<T>::split(sc[v] * (tv[i] * lane_dec), hi, lo);
-                        mh[v / 8].v[v % 8] = hi;
-                        if (PARTS == 2) ml[v / 8].v[v % 8] = lo;
-                    }
+                    const float4 t4 = *reinterpret_cast<const float4 *>(tab_row + sb * 32 + 8 * vg + 4 * half);
+                    fv[4 * vg] = t4.x; fv[4 * vg + 1] = t4.y; fv[4 * vg + 2] = t4.z; fv[4 * vg + 3] = t4.w;
                 }
             } else {
+                // exact path: scale what has been summed, then full factors (exponents clamped at 0: entries
+                // above the diagonal stay finite and are masked below)
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb) accY[pb] = accY[pb] * El;
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
                     const int s0 = sb * 32 + 8 * vg + 4 * half;
                     const float4 ah4 = *reinterpret_cast<const float4 *>(ah_s + s0);
                     const float4 al4 = *reinterpret_cast<const float4 *>(alo_s + s0);
                     const float4 dt4 = *reinterpret_cast<const float4 *>(dt_s + s0);
-                    const float ahv[4] = {ah4.x, ah4.y, ah4.z, ah4.w};
-                    const float alv[4] = {al4.x, al4.y, al4.z, al4.w};
-                    const float dtv[4] = {dt4.x, dt4.y, dt4.z, dt4.w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int v = vg * 4 + i;
-                        // masked entries get exp2(-inf) = 0: a select on the exponent, no branch
-                        const float arg = fminf(alpha_diff(al_hi, al_lo, ahv[i], alv[i]), 0.f);
-                        const float w = exp2_hw((s0 + i <= l) ? arg : -INFINITY) * dtv[i] * sc[v];
-                        T hi, lo;
-                        Split<T>::split(w, hi, lo);
-                        mh[v / 8].v[v % 8] = hi;
-                        if (PARTS == 2) ml[v / 8].v[v % 8] = lo;
-                    }
+                    fv[4 * vg] = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah4.x, al4.x), 0.f)) * dt4.x;
+                    fv[4 * vg + 1] = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah4.y, al4.y), 0.f)) * dt4.y;
+                    fv[4 * vg + 2] = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah4.z, al4.z), 0.f)) * dt4.z;
+                    fv[4 * vg + 3] = exp2_hw(fminf(alpha_diff(al_hi, al_lo, ah4.w, al4.w), 0.f)) * dt4.w;
                 }
+            }
+            Frag<T> mh[2], ml[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                float sv[8], fj[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int v = 8 * j + i;
+                    // causal mask inside the diagonal block: row 8 (v/4) + 4 half + v%4 <= column r
+                    sv[i] = (!diag || 8 * (v / 4) + 4 * half + (v % 4) <= r) ? sc[v] : 0.f;
+                    fj[i] = fv[v];
+                }
+                ProductFrags<T>::make(sv, fj, mh[j], ml[j]);
             }
 #pragma unroll
             for (int pb = 0; pb < PB; ++pb) {
@@ -261,6 +266,10 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
                     accY[pb] = mma32(xf, mh[j], accY[pb]);
                     if (PARTS == 2) accY[pb] = mma32(xf, ml[j], accY[pb]);
                 }
+            }
+            if (diag && fast) {  // everything summed so far shares the factor E[l]
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb) accY[pb] = accY[pb] * El;
             }
         }
         // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]

@@ -261,6 +261,45 @@ template <> __device__ inline void store_column<float>(float *yrow, float (&o)[1
     }
 }
 
+// hi + lo bf16 pairs of two products a0*f0 and a1*f1 (f = 1 to split plain values): hi is the product
+// rounded to bf16, lo the rounded remainder, which the fused multiply-add gets from the exact product.
+// Four VALU instructions per element: multiply, half a pack, one shift or mask, fma, half a pack.
+__device__ inline void split_pair(float a0, float f0, float a1, float f1, unsigned &hi, unsigned &lo) {
+    hi = pack_bf16x2(a0 * f0, a1 * f1);
+    asm("" : "+v"(hi));  // keep the packed pair as the source of both halves (else the low half is converted twice)
+    const float h0 = __uint_as_float(hi << 16), h1 = __uint_as_float(hi & 0xffff0000u);
+    lo = pack_bf16x2(__builtin_fmaf(a0, f0, -h0), __builtin_fmaf(a1, f1, -h1));
+}
+struct FragBits {  // an operand fragment as four packed pairs
+    unsigned u[4];
+    __device__ inline Frag<__bf16> frag() const {
+        typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+        u32x4 v = {u[0], u[1], u[2], u[3]};
+        Frag<__bf16> f;
+        f.v = __builtin_bit_cast(bf16x8, v);
+        return f;
+    }
+};
+
+// Operand fragments of eight products a[i]*f[i]: a hi + lo pair in bf16 mode, the products themselves in
+// float mode (lo is then unused).
+template <typename T> struct ProductFrags;
+template <> struct ProductFrags<__bf16> {
+    static __device__ inline void make(const float (&a)[8], const float (&f)[8], Frag<__bf16> &hi, Frag<__bf16> &lo) {
+        FragBits fh, fl;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) split_pair(a[2 * k], f[2 * k], a[2 * k + 1], f[2 * k + 1], fh.u[k], fl.u[k]);
+        hi = fh.frag();
+        lo = fl.frag();
+    }
+};
+template <> struct ProductFrags<float> {
+    static __device__ inline void make(const float (&a)[8], const float (&f)[8], Frag<float> &hi, Frag<float> &) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) hi.v[i] = a[i] * f[i];
+    }
+};
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, and
 // on gfx9 loads and stores share one counter, so it drains every outstanding global load -- among
 // them the next tile's prefetch, which must stay in flight across the barrier.  The tile loops

@@ -94,26 +94,6 @@ __device__ inline float readlane_f(float v, int src_lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
 }
 
-// hi + lo bf16 pairs of two products a0*f0 and a1*f1 (f = 1 to split plain values): hi is the product
-// rounded to bf16, lo the rounded remainder, which the fused multiply-add gets from the exact product.
-// Four VALU instructions per element: multiply, half a pack, one shift or mask, fma, half a pack.
-__device__ inline void split_pair(float a0, float f0, float a1, float f1, unsigned &hi, unsigned &lo) {
-    hi = pack_bf16x2(a0 * f0, a1 * f1);
-    asm("" : "+v"(hi));  // keep the packed pair as the source of both halves (else the low half is converted twice)
-    const float h0 = __uint_as_float(hi << 16), h1 = __uint_as_float(hi & 0xffff0000u);
-    lo = pack_bf16x2(__builtin_fmaf(a0, f0, -h0), __builtin_fmaf(a1, f1, -h1));
-}
-struct FragBits {  // an operand fragment as four packed pairs
-    unsigned u[4];
-    __device__ inline Frag<__bf16> frag() const {
-        typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
-        u32x4 v = {u[0], u[1], u[2], u[3]};
-        Frag<__bf16> f;
-        f.v = __builtin_bit_cast(bf16x8, v);
-        return f;
-    }
-};
-
 // Time steps per tile of the one-pass kernel.  The kernel has no workspace whose layout the caller's chunk
 // length would fix, so it tiles time by what runs fastest: with 64 a tile has one s-block below the diagonal
 // per two on it (128: three per two; 32: none, but the per-tile work doubles again); measured 210 us against
