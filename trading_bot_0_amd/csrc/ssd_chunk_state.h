@@ -143,8 +143,12 @@ __global__ __launch_bounds__(64 * PB * ((NK + 1) / 2)) void chunk_state_kernel(
             if (xrows_exact || l < Q) {
                 if constexpr (is_bf16<T>) {
                     Vec16<T> hi, lo;
+                    unsigned hw[4], lw[4];
 #pragma unroll
-                    for (int i = 0; i < VEC; ++i) Split<T>::split(R.wv[u] * (float)R.xv[u].e[i], hi.e[i], lo.e[i]);
+                    for (int i = 0; i < 4; ++i)
+                        split_pair((float)R.xv[u].e[2 * i], R.wv[u], (float)R.xv[u].e[2 * i + 1], R.wv[u], hw[i], lw[i]);
+                    hi.u = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+                    lo.u = make_uint4(lw[0], lw[1], lw[2], lw[3]);
                     const int o = XT::off(l, xch * VEC);
                     *reinterpret_cast<uint4 *>(xs + o) = hi.u;
                     *reinterpret_cast<uint4 *>(xs + Q * Ppad + o) = lo.u;
