@@ -15,7 +15,8 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
                compulsory traffic of the whole op.  Staged forward: the slowest stage.
   stages       the staged kernels issued one by one through their own entry points, each with
                its algorithmic bytes, GB/s and (stages 2, 4) dense MFMA rate; measured in both cases
-  stream_step  the single-timestep update at batch 4096: latency and GB/s
+  stream_step  the single-timestep update at batch 4096: latency and GB/s; stream_steps_one_launch: the same
+               64 steps as one launch of the multi-step kernel
   reference_suite  the reference's historical benchmark cases for this path (batch 4, seq_len 4096,
                BFloat16), for the SSD op alone, in the reference's result schema
   cpu_baseline the plain-C oracle (sequential recurrence, float32, OpenMP) timed on this
@@ -237,6 +238,27 @@ def main():
         out["stream_step"] = {"batch": sw.batch, "steps": sw.stream_steps, "us_per_step": round(us, 2),
                               "alg_bytes": step_bytes(sw), "GBps": round(gbs, 1),
                               "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
+        # the same 64 steps as ONE launch (state in registers between the steps): per-step latency, and the
+        # traffic of the launch = state in and out once plus the 64 steps' inputs and outputs
+        xs64, ds64 = si["x"].contiguous(), si["dt"].contiguous()
+        bs64, cs64 = si["B"].contiguous(), si["C"].contiguous()
+        ys64 = torch.empty_like(xs64)
+        for _ in range(3):
+            ssd.ssd_steps(state, xs64, ds64, si["A"], bs64, cs64, si["D"], out=ys64)
+        reps = 10
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            ssd.ssd_steps(state, xs64, ds64, si["A"], bs64, cs64, si["D"], out=ys64)
+        e1.record()
+        torch.cuda.synchronize()
+        us64 = e0.elapsed_time(e1) * 1e3 / reps
+        bytes64 = 8 * sw.batch * sw.nheads * sw.headdim * sw.dstate + sw.stream_steps * (
+            step_bytes(sw) - 8 * sw.batch * sw.nheads * sw.headdim * sw.dstate)
+        out["stream_steps_one_launch"] = {"batch": sw.batch, "steps": sw.stream_steps,
+                                          "us_per_launch": round(us64, 1),
+                                          "us_per_step": round(us64 / sw.stream_steps, 2), "alg_bytes": bytes64,
+                                          "GBps": round(bytes64 / (us64 * 1e-6) / 1e9, 1)}
 
     # ---- the reference's own benchmark cases for this path ------------------------------------
     # benchmark_results/bench_20260112_070055.json:5-41 lists mamba2_forward_train, mamba2_infer_prefill and

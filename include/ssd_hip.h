@@ -151,6 +151,19 @@ int ssd_step_fwd(const ssd_step_dims *dims, int dtype, float *state, const void 
                  const void *dt, const float *A, const void *Bm, const void *Cm, const float *D,
                  void *y, void *hip_stream);
 
+/* nsteps consecutive recurrent updates in ONE launch, in place on state [B,H,P,N], with per-row resets:
+ * x,y [B,T,H,P]; dt [B,T,H]; Bm,Cm [B,T,G,N] (T = nsteps; the layout of the scan's tensors, so slices of a
+ * sequence can be passed); reset [B,T] bytes or NULL: a non-zero reset[b,t] zeroes batch row b of the state
+ * before step t.  The state stays in registers between the steps, so it crosses HBM once per launch instead
+ * of once per step, and T launches become one.  nsteps = 1 with a mask is the fused "reset some rows, then
+ * step" of a rollout (advance -> reset slots -> forward: trading_bots/src/torch/train/rollout.rs:130-135,
+ * 209-235; trading_bots/src/torch/model/stream/state.rs:10-21 for what a reset is).  headdim 16, 32 or 64;
+ * other head sizes return SSD_ERR_UNSUPPORTED (call ssd_step_fwd per step instead).  Results are those of
+ * ssd_step_fwd applied nsteps times. */
+int ssd_steps_fwd(const ssd_step_dims *dims, int64_t nsteps, int dtype, float *state, const uint8_t *reset,
+                  const void *x, const void *dt, const float *A, const void *Bm, const void *Cm, const float *D,
+                  void *y, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -136,3 +136,83 @@ def test_stream_state_lifecycle():
     st2.init_from_prefix(p2["x"], p2["dt"], dev["A"], p2["B"], p2["C"], dev["D"], chunk=32)
     _, f = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=32)
     assert rel_err(st2.state, np64(f)) < 1e-4
+
+
+# ---- several steps in one launch, with per-row resets ------------------------------------------
+
+def oracle_steps(cpu, reset=None):
+    """The oracle's single step applied T times in float64, zeroing the rows `reset` marks before a step."""
+    x, dt, Bm, Cm = (np64(cpu[k]) for k in ("x", "dt", "B", "C"))
+    A, D = np64(cpu["A"]), np64(cpu["D"])
+    st = np64(cpu["init"]).copy()
+    ys = []
+    for t in range(x.shape[1]):
+        if reset is not None:
+            st[reset[:, t] != 0] = 0.0
+        y, st = orc.ssd_step(st, x[:, t], dt[:, t], A, Bm[:, t], Cm[:, t], D)
+        ys.append(y)
+    return np.stack(ys, 1), st
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(5, 4, 16, 16, 1, 7), (3, 8, 32, 64, 1, 16), (2, 16, 64, 128, 2, 5),
+                                   (6, 6, 32, 32, 3, 1), (4, 8, 16, 128, 1, 9)])
+def test_steps_in_one_launch_match_the_oracle(shape, dtype):
+    from trading_bot_0_amd import ssd_steps
+    Bsz, H, P, N, G, T = shape
+    w = Workload("steps", Bsz, T, H, P, N, G, 32, dtype=dtype, init_std=1.0)
+    cpu = make_inputs(w, seed=21)
+    dev = to_dev(cpu)
+    rng = np.random.default_rng(3)
+    reset = (rng.random((Bsz, T)) < 0.3).astype(np.uint8)
+    reset[0, 0] = 1
+    for mask in (None, reset):
+        yr, sr = oracle_steps(cpu, mask)
+        rm = None if mask is None else torch.from_numpy(mask).cuda()
+        states = []
+
+        def call(yd):
+            states.append(dev["init"].clone())
+            return ssd_steps(states[-1], dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], reset=rm,
+                             y_dtype=yd)
+
+        check_y(call, yr, w.torch_dtype, "steps y")
+        torch.cuda.synchronize()
+        for st in states:
+            assert_close(st, sr, torch.float32, "steps state")
+
+
+def test_steps_equal_repeated_single_steps_and_reset_cleans_a_poisoned_row():
+    from trading_bot_0_amd import ssd_steps
+    w = Workload("eq", 6, 12, 8, 32, 64, 1, 32, dtype="bf16", init_std=0.5)
+    dev = to_dev(make_inputs(w, seed=5))
+    a = SsdStreamState(dev["init"].clone(), True)
+    b = SsdStreamState(dev["init"].clone(), True)
+    reset = torch.zeros((w.batch, w.seqlen), dtype=torch.bool, device="cuda")
+    reset[2, 4] = True
+    reset[5, 0] = True
+    b.state[5].fill_(float("nan"))          # whatever a restarted environment left behind must not survive
+    ys = []
+    for t in range(w.seqlen):
+        rows = reset[:, t]
+        if bool(rows.any()):
+            a.reset_rows(rows)
+        ys.append(a.step(dev["x"][:, t].contiguous(), dev["dt"][:, t].contiguous(), dev["A"],
+                         dev["B"][:, t].contiguous(), dev["C"][:, t].contiguous(), dev["D"], y_dtype=torch.float32))
+    y_one = b.steps(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], reset=reset, y_dtype=torch.float32)
+    torch.cuda.synchronize()
+    y_ref = torch.stack(ys, 1)
+    assert torch.isfinite(y_one).all() and torch.isfinite(b.state).all()
+    assert rel_err(y_one, y_ref.double().cpu().numpy()) <= 1e-5
+    assert rel_err(b.state, a.state.double().cpu().numpy()) <= 1e-5
+
+
+def test_steps_refuses_what_it_cannot_hold_in_registers():
+    from trading_bot_0_amd import SsdError, ssd_steps
+    w = Workload("p48", 2, 3, 2, 48, 16, 2, 32, dtype="f32", init_std=1.0)
+    dev = to_dev(make_inputs(w, seed=1))
+    with pytest.raises(SsdError) as ei:
+        ssd_steps(dev["init"].clone(), dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"])
+    assert ei.value.code == 2
+    with pytest.raises(ValueError):
+        ssd_steps(dev["init"].clone(), dev["x"][:, 0], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"])

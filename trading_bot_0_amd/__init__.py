@@ -11,6 +11,7 @@ from .ssd import (  # noqa: F401
     ssd_chunk_scan,
     ssd_chunk_scan_onepass,
     ssd_step,
+    ssd_steps,
     state_passing,
     workspace_bytes,
 )

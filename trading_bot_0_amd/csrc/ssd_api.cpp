@@ -308,4 +308,33 @@ int ssd_step_fwd(const ssd_step_dims *dims, int dtype, float *state, const void 
     return e == hipSuccess ? SSD_OK : hip_fail(e, "step launch");
 }
 
+int ssd_steps_fwd(const ssd_step_dims *dims, int64_t nsteps, int dtype, float *state, const uint8_t *reset,
+                  const void *x, const void *dt, const float *A, const void *Bm, const void *Cm, const float *D,
+                  void *y, void *hip_stream) {
+    if (dims == nullptr) return fail(SSD_ERR_INVALID, "ssd: dims must not be NULL");
+    if (int rc = check_dtype(dtype)) return rc;
+    if (dims->batch <= 0) return fail(SSD_ERR_INVALID, "ssd: batch must be positive, got %lld", (long long)dims->batch);
+    if (nsteps <= 0 || nsteps > 0x7fffffff)
+        return fail(SSD_ERR_INVALID, "ssd: nsteps must be positive, got %lld", (long long)nsteps);
+    if (int rc = check_state_dims(dims->nheads, dims->headdim, dims->dstate, dims->ngroups)) return rc;
+    if (dims->batch * dims->nheads > 0x7fffffff)
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: batch*nheads exceeds 2^31-1");
+    REQUIRE_PTR(state);
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(dt);
+    REQUIRE_PTR(A);
+    REQUIRE_PTR(Bm);
+    REQUIRE_PTR(Cm);
+    REQUIRE_PTR(y);
+    OPTIONAL_PTR(D);
+    ssd::StepShape s{(int)dims->batch, (int)dims->nheads, (int)dims->headdim, (int)dims->dstate,
+                     (int)dims->ngroups};
+    if (!ssd::steps_supported(s))
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: the multi-step update keeps the state in registers and needs headdim "
+                                         "16, 32 or 64, got %lld", (long long)dims->headdim);
+    hipError_t e = ssd::launch_steps(s, (int)nsteps, dtype, state, reset, x, dt, A, Bm, Cm, D, y,
+                                     (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "multi-step launch");
+}
+
 }  // extern "C"

@@ -48,4 +48,12 @@ hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *
                        const float *A, const void *Bm, const void *Cm, const float *D, void *y,
                        hipStream_t stream);
 
+// nsteps consecutive single-timestep updates in one launch (state in registers), reset [B,nsteps] bytes or NULL:
+// a non-zero entry zeroes that batch row before the step.  Tensors as for the scan: x,y [B,T,H,P], dt [B,T,H],
+// Bm,Cm [B,T,G,N].  steps_supported: headdim 16, 32 or 64.
+bool steps_supported(const StepShape &s);
+hipError_t launch_steps(const StepShape &s, int nsteps, int dtype, float *state, const unsigned char *reset,
+                        const void *x, const void *dt, const float *A, const void *Bm, const void *Cm,
+                        const float *D, void *y, hipStream_t stream);
+
 }  // namespace ssd

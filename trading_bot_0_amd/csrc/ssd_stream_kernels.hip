@@ -186,6 +186,82 @@ __global__ __launch_bounds__(256) void step_kernel(float *__restrict__ state, co
 }
 
 // ------------------------------------------------------------------------------------------
+// T consecutive single-timestep updates in one launch, with per-row resets.  One wave per (b,h)
+// keeps its [P,N] state in registers for all T steps (PASSES float4 per lane), so the state is
+// read and written once per launch instead of once per step; the next step's x, dt, B, C are
+// requested before the current step's arithmetic.  reset[b,t] != 0 zeroes batch row b before
+// step t.  Inputs and y have the layout of the scan's tensors: [B,T,...].
+// ------------------------------------------------------------------------------------------
+template <typename T, typename TO, int NL, int PASSES>
+__global__ __launch_bounds__(256) void steps_kernel(float *__restrict__ state, const unsigned char *__restrict__ reset,
+                                                    const T *__restrict__ x, const T *__restrict__ dt,
+                                                    const float *__restrict__ A, const T *__restrict__ Bm,
+                                                    const T *__restrict__ Cm, const float *__restrict__ D,
+                                                    TO *__restrict__ y, StepShape s, int nsteps) {
+    constexpr int N = NL * 4;
+    constexpr int RPP = 64 / NL;  // rows per pass
+    const int lane = threadIdx.x & 63;
+    const long long bh = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (bh >= (long long)s.B * s.H) return;
+    const int b = (int)(bh / s.H), h = (int)(bh % s.H);
+    const int g = h / (s.H / s.G);
+    const int nl = lane % NL, rl = lane / NL;
+    const float a_h = A[h];
+    const float dh = D ? D[h] : 0.f;
+    float4 *sp = reinterpret_cast<float4 *>(state) + (size_t)bh * s.P * NL;
+    float4 hv[PASSES];
+#pragma unroll
+    for (int u = 0; u < PASSES; ++u) hv[u] = sp[(size_t)(u * RPP + rl) * NL + nl];
+
+    struct StepIn {
+        float dtv, bv[4], cv[4], xv[PASSES];
+        bool clear;
+    };
+    auto fetch = [&](int t, StepIn &in) {
+        const size_t bt = (size_t)b * nsteps + t;
+        in.dtv = (float)dt[bt * s.H + h];
+        in.clear = reset != nullptr && reset[bt] != 0;
+        const T *bp = Bm + (bt * s.G + g) * N + nl * 4, *cp = Cm + (bt * s.G + g) * N + nl * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            in.bv[i] = (float)bp[i];
+            in.cv[i] = (float)cp[i];
+        }
+        const T *xp = x + (bt * s.H + h) * s.P + rl;
+#pragma unroll
+        for (int u = 0; u < PASSES; ++u) in.xv[u] = (float)xp[u * RPP];
+    };
+    StepIn cur, nxt;
+    fetch(0, cur);
+    for (int t = 0; t < nsteps; ++t) {
+        if (t + 1 < nsteps) fetch(t + 1, nxt);
+        const float decay = expf(cur.dtv * a_h);
+        if (cur.clear) {  // a reset row restarts from zero, whatever the state held (uniform per wave)
+#pragma unroll
+            for (int u = 0; u < PASSES; ++u) hv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        TO *yp = y + (((size_t)b * nsteps + t) * s.H + h) * s.P + rl;
+#pragma unroll
+        for (int u = 0; u < PASSES; ++u) {
+            const float xd = cur.xv[u] * cur.dtv;
+            float4 v = hv[u];
+            v.x = decay * v.x + xd * cur.bv[0];
+            v.y = decay * v.y + xd * cur.bv[1];
+            v.z = decay * v.z + xd * cur.bv[2];
+            v.w = decay * v.w + xd * cur.bv[3];
+            hv[u] = v;
+            float part = v.x * cur.cv[0] + v.y * cur.cv[1] + v.z * cur.cv[2] + v.w * cur.cv[3];
+#pragma unroll
+            for (int m = NL / 2; m >= 1; m >>= 1) part += __shfl_xor(part, m, 64);
+            if (nl == 0) yp[u * RPP] = (TO)(part + dh * cur.xv[u]);
+        }
+        if (t + 1 < nsteps) cur = nxt;
+    }
+#pragma unroll
+    for (int u = 0; u < PASSES; ++u) sp[(size_t)(u * RPP + rl) * NL + nl] = hv[u];
+}
+
+// ------------------------------------------------------------------------------------------
 // Launchers
 // ------------------------------------------------------------------------------------------
 template <typename T>
@@ -243,6 +319,50 @@ hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *
         case 0: return step_dispatch<float, float>(s, state, x, dt, A, Bm, Cm, D, y, st);
         case 1: return step_dispatch<__bf16, __bf16>(s, state, x, dt, A, Bm, Cm, D, y, st);
         default: return step_dispatch<__bf16, float>(s, state, x, dt, A, Bm, Cm, D, y, st);
+    }
+}
+
+template <typename T, typename TO, int NL>
+static hipError_t steps_dispatch_p(const StepShape &s, int nsteps, float *state, const unsigned char *reset,
+                                   const T *x, const T *dt, const float *A, const T *Bm, const T *Cm,
+                                   const float *D, TO *y, hipStream_t st) {
+    const long long pairs = (long long)s.B * s.H;
+    const dim3 grid((unsigned)((pairs + 3) / 4)), block(256);
+    constexpr int RPP = 64 / NL;
+    switch (s.P) {
+        case 16: steps_kernel<T, TO, NL, 16 / RPP><<<grid, block, 0, st>>>(state, reset, x, dt, A, Bm, Cm, D, y, s, nsteps); break;
+        case 32: steps_kernel<T, TO, NL, 32 / RPP><<<grid, block, 0, st>>>(state, reset, x, dt, A, Bm, Cm, D, y, s, nsteps); break;
+        case 64: steps_kernel<T, TO, NL, 64 / RPP><<<grid, block, 0, st>>>(state, reset, x, dt, A, Bm, Cm, D, y, s, nsteps); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+template <typename T, typename TO>
+static hipError_t steps_dispatch(const StepShape &s, int nsteps, float *state, const unsigned char *reset,
+                                 const void *x, const void *dt, const float *A, const void *Bm, const void *Cm,
+                                 const float *D, void *y, hipStream_t st) {
+    const T *xx = static_cast<const T *>(x), *dd = static_cast<const T *>(dt);
+    const T *bb = static_cast<const T *>(Bm), *cc = static_cast<const T *>(Cm);
+    TO *yy = static_cast<TO *>(y);
+    switch (s.N) {
+        case 16: return steps_dispatch_p<T, TO, 4>(s, nsteps, state, reset, xx, dd, A, bb, cc, D, yy, st);
+        case 32: return steps_dispatch_p<T, TO, 8>(s, nsteps, state, reset, xx, dd, A, bb, cc, D, yy, st);
+        case 64: return steps_dispatch_p<T, TO, 16>(s, nsteps, state, reset, xx, dd, A, bb, cc, D, yy, st);
+        case 128: return steps_dispatch_p<T, TO, 32>(s, nsteps, state, reset, xx, dd, A, bb, cc, D, yy, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+bool steps_supported(const StepShape &s) { return s.P == 16 || s.P == 32 || s.P == 64; }
+
+hipError_t launch_steps(const StepShape &s, int nsteps, int dtype, float *state, const unsigned char *reset,
+                        const void *x, const void *dt, const float *A, const void *Bm, const void *Cm,
+                        const float *D, void *y, hipStream_t st) {
+    switch (dtype) {
+        case 0: return steps_dispatch<float, float>(s, nsteps, state, reset, x, dt, A, Bm, Cm, D, y, st);
+        case 1: return steps_dispatch<__bf16, __bf16>(s, nsteps, state, reset, x, dt, A, Bm, Cm, D, y, st);
+        default: return steps_dispatch<__bf16, float>(s, nsteps, state, reset, x, dt, A, Bm, Cm, D, y, st);
     }
 }
 

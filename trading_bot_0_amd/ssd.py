@@ -39,6 +39,7 @@ EXPORTED_SYMBOLS = (
     "ssd_chunk_scan_is_onepass",
     "ssd_chunk_scan_stage_fwd",
     "ssd_step_fwd",
+    "ssd_steps_fwd",
 )
 
 
@@ -94,6 +95,7 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_chunk_scan_is_onepass.argtypes = [POINTER(SsdDims), c_int, POINTER(c_int)]
         lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
+        lib.ssd_steps_fwd.argtypes = [POINTER(SsdStepDims), c_int64, c_int, P, P, P, P, P, P, P, P, P, P]
         for name in EXPORTED_SYMBOLS[2:]:
             getattr(lib, name).restype = c_int
         _lib = lib
@@ -450,4 +452,55 @@ def ssd_step(
     _check(lib, lib.ssd_step_fwd(byref(dims), code, state.data_ptr(), x.data_ptr(), dt.data_ptr(),
                                  A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), _ptr(D), y.data_ptr(),
                                  _stream_ptr(x)))
+    return y
+
+
+def ssd_steps(
+    state: torch.Tensor,
+    x: torch.Tensor,
+    dt: torch.Tensor,
+    A: torch.Tensor,
+    Bm: torch.Tensor,
+    Cm: torch.Tensor,
+    D: Optional[torch.Tensor] = None,
+    reset: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+    y_dtype: Optional[torch.dtype] = None,
+) -> torch.Tensor:
+    """T consecutive recurrent updates in one launch.  `state` [B,H,P,N] fp32 is advanced in place
+    by T steps; x [B,T,H,P], dt [B,T,H], Bm/Cm [B,T,G,N]; returns y [B,T,H,P].  `reset` [B,T] uint8
+    or bool: a non-zero entry zeroes that batch row of the state before the step (a rollout's
+    "reset some environments, then step")."""
+    lib = load_library()
+    if state.dim() != 4:
+        raise ValueError(f"SSD state must be rank-4 [batch, nheads, headdim, dstate], got {tuple(state.shape)}")
+    if x.dim() != 4:
+        raise ValueError(f"SSD steps x must be rank-4 [batch, nsteps, nheads, headdim], got {tuple(x.shape)}")
+    if Bm.dim() != 4:
+        raise ValueError(f"SSD steps B must be rank-4 [batch, nsteps, ngroups, dstate], got {tuple(Bm.shape)}")
+    Bsz, H, P, N = state.shape
+    T, G = x.shape[1], Bm.shape[2]
+    if T < 1:
+        raise ValueError("SSD steps needs at least one step")
+    dtype = x.dtype
+    _dtype_code(x)
+    _require(state, "state", (Bsz, H, P, N), torch.float32)
+    _require(x, "x", (Bsz, T, H, P), dtype)
+    _require(dt, "dt", (Bsz, T, H), dtype)
+    _require(A, "A", (H,), torch.float32)
+    _require(Bm, "B", (Bsz, T, G, N), dtype)
+    _require(Cm, "C", (Bsz, T, G, N), dtype)
+    if D is not None:
+        _require(D, "D", (H,), torch.float32)
+    if reset is not None:
+        if reset.dtype == torch.bool:
+            reset = reset.view(torch.uint8)
+        _require(reset, "reset", (Bsz, T), torch.uint8)
+    code, y_dtype = _out_code(x, y_dtype)
+    y = torch.empty((Bsz, T, H, P), dtype=y_dtype, device=x.device) if out is None else out
+    _require(y, "out", (Bsz, T, H, P), y_dtype)
+    dims = SsdStepDims(Bsz, H, P, N, G)
+    _check(lib, lib.ssd_steps_fwd(byref(dims), T, code, state.data_ptr(), _ptr(reset), x.data_ptr(), dt.data_ptr(),
+                                  A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), _ptr(D), y.data_ptr(),
+                                  _stream_ptr(x)))
     return y

@@ -73,3 +73,16 @@ class SsdStreamState:
         y = ssd.ssd_step(self.state, x, dt, A, Bm, Cm, D, out=out, y_dtype=y_dtype)
         self.initialized = True
         return y
+
+    def steps(self, x, dt, A, Bm, Cm, D=None, reset: Optional[torch.Tensor] = None,
+              out: Optional[torch.Tensor] = None, y_dtype=None) -> torch.Tensor:
+        """Advance every stream by T timesteps in one launch, the state staying on chip between them.
+        x [B,T,H,P], dt [B,T,H], Bm/Cm [B,T,G,N]; `reset` [B,T] (bool or uint8) zeroes a stream right
+        before the marked step, which is the rollout's advance -> reset slots -> forward
+        (trading_bots/src/torch/train/rollout.rs:130-135,209-235) without a separate pass over the
+        state.  Returns y [B,T,H,P]."""
+        if x.shape[0] != self.batch:
+            raise ValueError(f"stream state batch size mismatch: state has {self.batch}, input has {x.shape[0]}")
+        y = ssd.ssd_steps(self.state, x, dt, A, Bm, Cm, D, reset=reset, out=out, y_dtype=y_dtype)
+        self.initialized = True
+        return y
