@@ -120,3 +120,32 @@ def test_unsupported_shapes_are_refused():
         with pytest.raises(SsdError) as ei:
             run(dev, w.chunk)
         assert ei.value.code == 2, w.name
+
+
+def test_one_pass_kernel_on_a_side_stream_and_inside_a_captured_graph():
+    """Same contract as the staged kernels: nothing allocated, nothing synchronised, so the launch can be
+    captured (the reference captures its update, trading_bots/src/torch/train/update.rs:206-330).  Replays
+    are interleaved with eager work and each is checked."""
+    w = Workload("graph", 4, 320, 8, 32, 64, 1, 128, init_std=0.2)
+    dev = to_dev(make_inputs(w, seed=8))
+    y_ref, f_ref = run(dev, 128)
+    out, fin = torch.empty_like(dev["x"]), torch.empty(4, 8, 32, 64, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(dev, 128, out=out, final_out=fin)
+    side.synchronize()
+    assert torch.equal(out, y_ref) and torch.equal(fin, f_ref)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ssd_chunk_scan_onepass(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=128,
+                               initial_states=dev["init"], out=out, final_out=fin)
+    x_keep = dev["x"].clone()
+    for i in range(4):
+        out.fill_(float("nan"))
+        fin.fill_(float("nan"))
+        dev["x"].copy_(x_keep * 0.5 if i % 2 else x_keep)     # change the captured inputs in place
+        graph.replay()
+        torch.cuda.synchronize()
+        y_e, f_e = run(dev, 128)
+        assert torch.equal(out, y_e) and torch.equal(fin, f_e), f"replay {i}"
