@@ -114,15 +114,27 @@ int ssd_chunk_state_passing_fwd(const ssd_dims *dims, int dtype, const void *x, 
 
 /* The whole forward in one kernel and one pass over the inputs (bf16 inputs only): a wave keeps the running
  * state of 32 head-dim columns of one (batch, head) in registers while it walks the chunks, so no workspace
- * is needed and nothing but x, dt, B, C is read and y, final_states written.  Same arguments and results as
- * ssd_chunk_scan_fwd.  Parallel over (batch, head) sequences only; ssd_chunk_scan_fwd takes this path by
- * itself when there are enough of them.  SSD_ERR_UNSUPPORTED unless dtype is bf16 (1 or 2), headdim is a
+ * is needed and nothing but x, dt, B, C is read and y, final_states written.  Same arguments (with the
+ * optional reset mask of ssd_chunk_scan_reset_fwd) and results as ssd_chunk_scan_fwd.  Parallel over
+ * (batch, head) sequences only; ssd_chunk_scan_fwd takes this path by itself when there are enough of them.  SSD_ERR_UNSUPPORTED unless dtype is bf16 (1 or 2), headdim is a
  * multiple of 32, dstate is 32 or 64 and (nheads/ngroups)*(headdim/32) is a multiple of 4.  dims->chunk must
  * be a valid chunk length but does not enter: with no workspace layout to honour, the kernel tiles time by
  * its own block of 64 steps (results agree with every chunk length to rounding).  Replaces the same slot as ssd_chunk_scan_fwd (model/trading_model.rs:589-606). */
 int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
                                const void *Bm, const void *Cm, const float *D, const float *initial_states,
-                               void *y, float *final_states, void *hip_stream);
+                               const uint8_t *reset, void *y, float *final_states, void *hip_stream);
+
+/* ssd_chunk_scan_fwd with restarts inside the sequences: reset [B,L] bytes or NULL; a non-zero reset[b,t]
+ * sets the state of batch row b to zero before timestep t, i.e. y[b,t..] and the final state see nothing
+ * from before t (an episode boundary inside a replayed window: the reset slots of
+ * trading_bots/src/torch/train/rollout.rs:130-135 landing inside the chunks that
+ * trading_bots/src/torch/model/stream/replay.rs:83-114 replays).  reset[b,0] != 0 discards
+ * initial_states[b].  Implemented as a drop of the cumulative log-decay at t, so it costs nothing beyond
+ * reading the mask.  ssd_chunk_scan_fwd is this function with reset = NULL. */
+int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
+                             const void *Bm, const void *Cm, const float *D, const float *initial_states,
+                             const uint8_t *reset, void *y, float *final_states, void *workspace,
+                             size_t workspace_bytes, void *hip_stream);
 
 /* *is_onepass = 1 if ssd_chunk_scan_fwd runs these dims as the one-pass kernel (its workspace is then not
  * touched), 0 if as the staged kernels.  A plan query like ssd_workspace_bytes; no reference counterpart. */

@@ -48,8 +48,9 @@ def _group_of_head(H: int, G: int) -> np.ndarray:
     return np.arange(H) // (H // G)
 
 
-def ssd_sequential(x, dt, A, Bm, Cm, D=None, init=None, dtype=np.float64):
-    """Definitional recurrence, one timestep at a time.  Ground truth for everything."""
+def ssd_sequential(x, dt, A, Bm, Cm, D=None, init=None, dtype=np.float64, reset=None):
+    """Definitional recurrence, one timestep at a time.  Ground truth for everything.
+    reset [B,L] (optional): a non-zero entry sets that batch row's state to zero before the timestep."""
     x = np.asarray(x, dtype)
     dt = np.asarray(dt, dtype)
     A = np.asarray(A, dtype)
@@ -61,6 +62,8 @@ def ssd_sequential(x, dt, A, Bm, Cm, D=None, init=None, dtype=np.float64):
     h = np.zeros((Bsz, H, P, N), dtype) if init is None else np.array(init, dtype)
     y = np.empty((Bsz, L, H, P), dtype)
     for t in range(L):
+        if reset is not None:
+            h[np.asarray(reset)[:, t] != 0] = 0
         a = np.exp(dt[:, t, :] * A[None, :])                      # [B,H]
         Bt = Bm[:, t, gh, :]                                      # [B,H,N]
         Ct = Cm[:, t, gh, :]

@@ -261,3 +261,27 @@ def test_c_oracle_matches_numpy_oracle():
     y1n, s1n = orc.ssd_step(init, x[:, 0], dt[:, 0], A, Bm[:, 0], Cm[:, 0], D)
     np.testing.assert_allclose(y1, y1n, rtol=1e-12)
     np.testing.assert_allclose(s1, s1n, rtol=1e-12)
+
+
+def test_reset_is_a_fresh_sequence_from_that_timestep():
+    """ssd_sequential(reset=...) against the reset-free function: a row with resets at t1 < t2 is the
+    concatenation of three independent scans, the later two from a zero state; a reset at t = 0 discards
+    the initial state; rows without resets are untouched."""
+    x, dt, A, Bm, Cm, D, init = rand_inputs(Bsz=3, L=40)
+    reset = np.zeros((3, 40), np.uint8)
+    reset[1, [13, 29]] = 1
+    reset[2, 0] = 1
+    y, f = orc.ssd_sequential(x, dt, A, Bm, Cm, D, init, reset=reset)
+    y0, f0 = orc.ssd_sequential(x[:1], dt[:1], A, Bm[:1], Cm[:1], D, init[:1])
+    np.testing.assert_array_equal(y[:1], y0)
+    np.testing.assert_array_equal(f[:1], f0)
+    parts, st = [], init[1:2]
+    for a, b in ((0, 13), (13, 29), (29, 40)):
+        yp, fp = orc.ssd_sequential(x[1:2, a:b], dt[1:2, a:b], A, Bm[1:2, a:b], Cm[1:2, a:b], D, st)
+        parts.append(yp)
+        st = None
+    np.testing.assert_allclose(y[1:2], np.concatenate(parts, 1), rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(f[1:2], fp, rtol=1e-12, atol=1e-13)
+    y2, f2 = orc.ssd_sequential(x[2:], dt[2:], A, Bm[2:], Cm[2:], D, None)
+    np.testing.assert_allclose(y[2:], y2, rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(f[2:], f2, rtol=1e-12, atol=1e-13)

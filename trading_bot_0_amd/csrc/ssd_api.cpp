@@ -148,7 +148,7 @@ int ssd_chunk_cumsum_fwd(const ssd_dims *dims, int dtype, const void *dt, const 
     REQUIRE_PTR(dt);
     REQUIRE_PTR(A);
     REQUIRE_PTR(dtcs);
-    hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dtcs, (hipStream_t)hip_stream);
+    hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, nullptr, dtcs, (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "chunk_cumsum launch");
 }
 
@@ -214,6 +214,14 @@ int ssd_chunk_scan_stage_fwd(const ssd_dims *dims, int dtype, const void *x, con
 int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
                        const void *Bm, const void *Cm, const float *D, const float *initial_states, void *y,
                        float *final_states, void *workspace, size_t workspace_bytes, void *hip_stream) {
+    return ssd_chunk_scan_reset_fwd(dims, dtype, x, dt, A, Bm, Cm, D, initial_states, nullptr, y, final_states,
+                                    workspace, workspace_bytes, hip_stream);
+}
+
+int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
+                             const void *Bm, const void *Cm, const float *D, const float *initial_states,
+                             const uint8_t *reset, void *y, float *final_states, void *workspace,
+                             size_t workspace_bytes, void *hip_stream) {
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
     REQUIRE_PTR(x);
@@ -235,10 +243,10 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
     hipStream_t st = (hipStream_t)hip_stream;
     hipError_t e;
     if (takes_one_pass(s, dtype)) {
-        e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, y, final_states, st);
+        e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states, st);
         return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
     }
-    e = ssd::launch_chunk_cumsum(s, dtype, dt, A, dtcs, st);
+    e = ssd::launch_chunk_cumsum(s, dtype, dt, A, reset, dtcs, st);
     if (e != hipSuccess) return hip_fail(e, "chunk_cumsum launch");
     if ((int64_t)s.B * s.H >= kFusedStatePassingMinSequences) {
         // enough (b,h) sequences to fill the chip: stages 2 and 3 in one pass, states carried on chip
@@ -265,7 +273,7 @@ int ssd_chunk_scan_is_onepass(const ssd_dims *dims, int dtype, int *is_onepass) 
 
 int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
                                const void *Bm, const void *Cm, const float *D, const float *initial_states,
-                               void *y, float *final_states, void *hip_stream) {
+                               const uint8_t *reset, void *y, float *final_states, void *hip_stream) {
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
     REQUIRE_PTR(x);
@@ -281,7 +289,7 @@ int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, c
         return fail(SSD_ERR_UNSUPPORTED,
                     "ssd: the one-pass scan needs bf16 inputs, headdim a multiple of 32, dstate 32 or 64 and "
                     "(nheads/ngroups)*(headdim/32) a multiple of 4");
-    hipError_t e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, y, final_states,
+    hipError_t e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states,
                                           (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
 }

@@ -186,6 +186,14 @@ template <int COLS> struct RowMajorTile {
     }
 };
 
+// A reset before step t (the state restarts from zero there) is a drop of the cumulative log2-decay by
+// kResetLog2 at t: every decay factor that spans the reset becomes exp2(-16384 or less) = 0 and everything
+// on one side of it is unchanged, since only differences of alpha are ever used.  In the natural-log units
+// of the float64 scan that is kResetDrop per reset.  (Up to 256 resets per chunk keep |alpha| below 2^22,
+// where the hi + lo float pair still resolves differences to 1e-8.)
+constexpr double kResetLog2 = 16384.0;
+constexpr double kResetDrop = kResetLog2 / 1.4426950408889634;
+
 // ------------------------------------------------------------------------------------------
 // Wavefront inclusive scan in float64 (DPP data movement)
 // ------------------------------------------------------------------------------------------

@@ -115,7 +115,8 @@ template <typename TO, int NK, int QB, int WAVES, bool EARLY>  // N = 16*NK, Q =
 __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_kernel(
     const __bf16 *__restrict__ x, const __bf16 *__restrict__ dt, const float *__restrict__ A,
     const __bf16 *__restrict__ Bm, const __bf16 *__restrict__ Cm, const float *__restrict__ D,
-    const float *init, TO *__restrict__ y, float *final_states, ScanShape s) {
+    const float *init, const unsigned char *__restrict__ reset, TO *__restrict__ y, float *final_states,
+    ScanShape s) {
     using T = __bf16;
     constexpr int N = 16 * NK, NB = NK / 2, Q = 32 * QB, nthr = 64 * WAVES;
     constexpr int EPL = Q >= 64 ? Q / 64 : 1;  // chunk positions per lane in the scan
@@ -158,6 +159,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     const T *Bb = Bm + ((size_t)b * s.L * s.G + g) * N;
     const T *Cb = Cm + ((size_t)b * s.L * s.G + g) * N;
     const T *dtb = dt + (size_t)b * s.L * s.H + h;
+    const unsigned char *rsb = reset ? reset + (size_t)b * s.L : nullptr;  // state restarts, see kResetLog2
     TO *yb = y + (size_t)b * s.L * HP + h * s.P + pb * 32;
     const float dh = D ? D[h] : 0.f;
     const double a_h = (double)A[h];
@@ -177,6 +179,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     };
     uint4 bq[UBC], cq[UBC], xq[UX];
     unsigned short dq[EPL];
+    unsigned char rq[EPL];
     auto prefetch = [&](int c) {
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
@@ -206,6 +209,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
                 dq[e] = (Q >= 64 || (tv & 63) < Q) ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e)
+                rq[e] = (rsb != nullptr && (Q >= 64 || (tv & 63) < Q)) ? rsb[t0 + (tv & 63) * EPL + e] : (unsigned char)0;
         } else {  // ragged last chunk: rows past the sequence read as zero (dt = 0 makes them no-ops)
 #pragma unroll
             for (int u = 0; u < UBC; ++u) {
@@ -218,6 +224,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
                 dq[e] = ((tv & 63) * EPL + e < rows) ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e)
+                rq[e] = (rsb != nullptr && (tv & 63) * EPL + e < rows) ? rsb[t0 + (tv & 63) * EPL + e] : (unsigned char)0;
         }
     };
 
@@ -279,7 +288,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
                 dtv[e] = (float)__builtin_bit_cast(__bf16, dq[e]);
-                run += (double)dtv[e] * a_h;
+                run += (double)dtv[e] * a_h - (rq[e] ? kResetDrop : 0.0);
                 cs[e] = run;
             }
             const double excl = wave_inclusive_scan(run) - run;
@@ -513,35 +522,34 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 // ------------------------------------------------------------------------------------------
 template <typename TO, int NK, int QB, int WAVES>
 static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
-                               const void *Cm, const float *D, const float *init, void *y, float *final_states,
-                               hipStream_t st) {
-#ifndef SSD_ONEPASS_EARLY
-#define SSD_ONEPASS_EARLY false
-#endif
-    constexpr bool EARLY = SSD_ONEPASS_EARLY;
+                               const void *Cm, const float *D, const float *init, const unsigned char *reset, void *y,
+                               float *final_states, hipStream_t st) {
+    // requesting the next tile's inputs at the top of the tile instead of after phase 1 measured the same
+    // (217.6 us against 218.8 us) for 26 more live registers
+    constexpr bool EARLY = false;
     const int units = (s.H / s.G) * (s.P / 32);
     const int grid = s.B * s.G * (units / WAVES);
     fused_scan_kernel<TO, NK, QB, WAVES, EARLY><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
         static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
-        static_cast<const __bf16 *>(Cm), D, init, static_cast<TO *>(y), final_states, s);
+        static_cast<const __bf16 *>(Cm), D, init, reset, static_cast<TO *>(y), final_states, s);
     return hipGetLastError();
 }
 
 template <typename TO, int NK, int QB>
 static hipError_t fused_dispatch_w(const ScanShape &s, int waves, const void *x, const void *dt, const float *A,
-                                   const void *Bm, const void *Cm, const float *D, const float *init, void *y,
-                                   float *final_states, hipStream_t st) {
-    return waves == 8 ? fused_launch<TO, NK, QB, 8>(s, x, dt, A, Bm, Cm, D, init, y, final_states, st)
-                      : fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, y, final_states, st);
+                                   const void *Bm, const void *Cm, const float *D, const float *init,
+                                   const unsigned char *reset, void *y, float *final_states, hipStream_t st) {
+    return waves == 8 ? fused_launch<TO, NK, QB, 8>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st)
+                      : fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
 }
 
 template <typename TO>
 hipError_t fused_dispatch(const ScanShape &s, int waves, const void *x, const void *dt, const float *A,
-                          const void *Bm, const void *Cm, const float *D, const float *init, void *y,
-                          float *final_states, hipStream_t st) {
+                          const void *Bm, const void *Cm, const float *D, const float *init,
+                          const unsigned char *reset, void *y, float *final_states, hipStream_t st) {
 #define SSD_FUSED_CASE(NKv, QBv) \
     if (s.N == 16 * NKv && s.Q == 32 * QBv) \
-        return fused_dispatch_w<TO, NKv, QBv>(s, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
+        return fused_dispatch_w<TO, NKv, QBv>(s, waves, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
     SSD_FUSED_CASE(2, kOnePassTile / 32)
     SSD_FUSED_CASE(4, kOnePassTile / 32)
 #undef SSD_FUSED_CASE

@@ -4,7 +4,8 @@
 namespace ssd {
 
 hipError_t launch_fused_scan_y32(const ScanShape &, int, const void *, const void *, const float *, const void *,
-                                 const void *, const float *, const float *, void *, float *, hipStream_t);
+                                 const void *, const float *, const float *, const unsigned char *, void *, float *,
+                                 hipStream_t);
 
 int fused_scan_waves(const ScanShape &s, int dtype) {
     if (dtype == 0) return 0;                         // float inputs take the staged kernels
@@ -17,15 +18,15 @@ int fused_scan_waves(const ScanShape &s, int dtype) {
 }
 
 hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const void *dt, const float *A,
-                             const void *Bm, const void *Cm, const float *D, const float *init, void *y,
-                             float *final_states, hipStream_t st) {
+                             const void *Bm, const void *Cm, const float *D, const float *init,
+                             const unsigned char *reset, void *y, float *final_states, hipStream_t st) {
     const int waves = fused_scan_waves(s, dtype);
     if (waves == 0) return hipErrorInvalidValue;
     ScanShape t = s;  // the kernel's own tiling of time; the caller's chunk length does not enter
     t.Q = kOnePassTile;
     t.nc = (s.L + kOnePassTile - 1) / kOnePassTile;
-    if (dtype == 2) return launch_fused_scan_y32(t, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
-    return fused_dispatch<__bf16>(t, waves, x, dt, A, Bm, Cm, D, init, y, final_states, st);
+    if (dtype == 2) return launch_fused_scan_y32(t, waves, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
+    return fused_dispatch<__bf16>(t, waves, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
 }
 
 }  // namespace ssd

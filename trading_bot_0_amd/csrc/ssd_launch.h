@@ -24,8 +24,9 @@ size_t chunk_scan_lds_bytes(const ScanShape &s, int elem_bytes);
 // dtype: 0 = float32, 1 = bf16, 2 = bf16 inputs with float32 y (stage 4 only; stages 1-2 treat it as 1).
 // dtcs is the stage-1 output [B,H,nc,4,Q] float32: log2(e) * cumulative dt*A as a hi/lo pair, dt, and
 // the stage-2 weight exp2(alpha[Q-1] - alpha[l]) * dt[l].
+// reset: [B,L] bytes or NULL; a non-zero entry restarts the state from zero before that timestep
 hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A,
-                               float *dtcs, hipStream_t stream);
+                               const unsigned char *reset, float *dtcs, hipStream_t stream);
 hipError_t launch_chunk_state(const ScanShape &s, int dtype, const void *x, const void *Bm,
                               const float *dtcs, float *states, hipStream_t stream);
 // stages 2+3 in one pass: writes the state entering each chunk into `prev` and the final state
@@ -42,8 +43,8 @@ hipError_t launch_chunk_scan(const ScanShape &s, int dtype, const void *x, const
 // fused_scan_waves is 0 when the shape cannot run there, else the waves per workgroup it would use.
 int fused_scan_waves(const ScanShape &s, int dtype);
 hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const void *dt, const float *A,
-                             const void *Bm, const void *Cm, const float *D, const float *init, void *y,
-                             float *final_states, hipStream_t stream);
+                             const void *Bm, const void *Cm, const float *D, const float *init,
+                             const unsigned char *reset, void *y, float *final_states, hipStream_t stream);
 hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *x, const void *dt,
                        const float *A, const void *Bm, const void *Cm, const float *D, void *y,
                        hipStream_t stream);

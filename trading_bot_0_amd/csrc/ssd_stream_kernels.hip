@@ -22,10 +22,12 @@ namespace ssd {
 template <typename T, int EPL>  // EPL = elements per lane = max(Q/64, 1)
 __global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__ dt,
                                                            const float *__restrict__ A,
+                                                           const unsigned char *__restrict__ reset,
                                                            float *__restrict__ dtcs, ScanShape s) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *tile = reinterpret_cast<float *>(smem);  // [H][Q+1]
     const int ldt = s.Q + 1;
+    float *drop = tile + s.H * ldt;                 // [Q]: kResetDrop where the state restarts, else 0
     const int b = blockIdx.x / s.nc, c = blockIdx.x % s.nc;
     const int t0 = c * s.Q;
     for (int idx = threadIdx.x; idx < s.Q * s.H; idx += blockDim.x) {
@@ -34,6 +36,8 @@ __global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__
         const float v = (t < s.L) ? (float)dt[((size_t)b * s.L + t) * s.H + h] : 0.f;
         tile[h * ldt + l] = v;
     }
+    for (int l = threadIdx.x; l < s.Q; l += blockDim.x)
+        drop[l] = (reset != nullptr && t0 + l < s.L && reset[(size_t)b * s.L + t0 + l] != 0) ? (float)kResetDrop : 0.f;
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     constexpr double kLog2e = 1.4426950408889634;
@@ -46,7 +50,7 @@ __global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
             dtv[e] = (l0 + e < s.Q) ? tile[h * ldt + l0 + e] : 0.f;
-            run += (double)dtv[e] * a;
+            run += (double)dtv[e] * a - (double)((l0 + e < s.Q) ? drop[l0 + e] : 0.f);
             cs[e] = run;
         }
         const double incl = wave_inclusive_scan(run);
@@ -265,24 +269,24 @@ __global__ __launch_bounds__(256) void steps_kernel(float *__restrict__ state, c
 // Launchers
 // ------------------------------------------------------------------------------------------
 template <typename T>
-static hipError_t cumsum_dispatch(const ScanShape &s, const void *dt, const float *A, float *dtcs,
-                                  hipStream_t st) {
+static hipError_t cumsum_dispatch(const ScanShape &s, const void *dt, const float *A, const unsigned char *reset,
+                                  float *dtcs, hipStream_t st) {
     const dim3 grid(s.B * s.nc), block(256);
-    const size_t lds = (size_t)s.H * (s.Q + 1) * sizeof(float);
+    const size_t lds = ((size_t)s.H * (s.Q + 1) + s.Q) * sizeof(float);
     const T *d = static_cast<const T *>(dt);
     if (s.Q <= 64) {
-        chunk_cumsum_kernel<T, 1><<<grid, block, lds, st>>>(d, A, dtcs, s);
+        chunk_cumsum_kernel<T, 1><<<grid, block, lds, st>>>(d, A, reset, dtcs, s);
     } else if (s.Q == 128) {
-        chunk_cumsum_kernel<T, 2><<<grid, block, lds, st>>>(d, A, dtcs, s);
+        chunk_cumsum_kernel<T, 2><<<grid, block, lds, st>>>(d, A, reset, dtcs, s);
     } else {
-        chunk_cumsum_kernel<T, 4><<<grid, block, lds, st>>>(d, A, dtcs, s);
+        chunk_cumsum_kernel<T, 4><<<grid, block, lds, st>>>(d, A, reset, dtcs, s);
     }
     return hipGetLastError();
 }
 
-hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A, float *dtcs,
-                               hipStream_t st) {
-    return dtype ? cumsum_dispatch<__bf16>(s, dt, A, dtcs, st) : cumsum_dispatch<float>(s, dt, A, dtcs, st);
+hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A,
+                               const unsigned char *reset, float *dtcs, hipStream_t st) {
+    return dtype ? cumsum_dispatch<__bf16>(s, dt, A, reset, dtcs, st) : cumsum_dispatch<float>(s, dt, A, reset, dtcs, st);
 }
 
 hipError_t launch_state_passing(const ScanShape &s, const float *states, const float *dtcs, const float *init,

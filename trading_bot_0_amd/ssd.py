@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "ssd_get_and_reset_last_err",
     "ssd_workspace_bytes",
     "ssd_chunk_scan_fwd",
+    "ssd_chunk_scan_reset_fwd",
     "ssd_chunk_cumsum_fwd",
     "ssd_chunk_state_fwd",
     "ssd_state_passing_fwd",
@@ -91,7 +92,8 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_chunk_state_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P]
         lib.ssd_state_passing_fwd.argtypes = [POINTER(SsdDims), P, P, P, P, P, P]
         lib.ssd_chunk_state_passing_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P]
-        lib.ssd_chunk_scan_onepass_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P]
+        lib.ssd_chunk_scan_onepass_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
+        lib.ssd_chunk_scan_reset_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, P, c_size_t, P]
         lib.ssd_chunk_scan_is_onepass.argtypes = [POINTER(SsdDims), c_int, POINTER(c_int)]
         lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
@@ -158,6 +160,16 @@ def _require(t: torch.Tensor, name: str, shape, dtype) -> None:
         raise ValueError(f"SSD {name} must be contiguous")
 
 
+def _reset_mask(reset, dims: "SsdDims"):
+    """[B,L] uint8 (bool accepted) or None."""
+    if reset is None:
+        return None
+    if reset.dtype == torch.bool:
+        reset = reset.view(torch.uint8)
+    _require(reset, "reset", (dims.batch, dims.seqlen), torch.uint8)
+    return reset
+
+
 def _scan_dims(x, Bm, chunk) -> SsdDims:
     if x.dim() != 4:
         raise ValueError(f"SSD x must be rank-4 [batch, seqlen, nheads, headdim], got {tuple(x.shape)}")
@@ -214,8 +226,11 @@ def ssd_chunk_scan(
     out: Optional[torch.Tensor] = None,
     final_out: Optional[torch.Tensor] = None,
     y_dtype: Optional[torch.dtype] = None,
+    reset: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """SSD chunk-scan forward.  Returns (y [B,L,H,P] in x's dtype, final_states [B,H,P,N] fp32).
+    `reset` [B,L] (uint8 or bool): a non-zero entry restarts that batch row's state from zero before the
+    timestep (episode boundaries inside a window).
 
     `workspace` (uint8, >= workspace_bytes(...)), `out` and `final_out` let a caller that runs
     under stream capture or in a tight loop avoid any allocation.  `y_dtype=torch.float32` with
@@ -237,9 +252,11 @@ def ssd_chunk_scan(
         workspace = torch.empty(need.value, dtype=torch.uint8, device=x.device)
     elif (not workspace.is_cuda) or workspace.dtype != torch.uint8 or not workspace.is_contiguous():
         raise ValueError("SSD workspace must be a contiguous uint8 GPU tensor")
-    rc = lib.ssd_chunk_scan_fwd(byref(dims), code, x.data_ptr(), dt.data_ptr(), A.data_ptr(),
-                                Bm.data_ptr(), Cm.data_ptr(), _ptr(D), _ptr(initial_states), y.data_ptr(),
-                                _ptr(final), workspace.data_ptr(), workspace.numel(), _stream_ptr(x))
+    reset = _reset_mask(reset, dims)
+    rc = lib.ssd_chunk_scan_reset_fwd(byref(dims), code, x.data_ptr(), dt.data_ptr(), A.data_ptr(),
+                                      Bm.data_ptr(), Cm.data_ptr(), _ptr(D), _ptr(initial_states), _ptr(reset),
+                                      y.data_ptr(), _ptr(final), workspace.data_ptr(), workspace.numel(),
+                                      _stream_ptr(x))
     _check(lib, rc)
     return y, final
 
@@ -252,7 +269,7 @@ class PreparedChunkScan:
     per call it costs one foreign call, where ssd_chunk_scan spends tens of microseconds in Python."""
 
     def __init__(self, x, dt, A, Bm, Cm, D=None, chunk=128, initial_states=None, return_final_states=True,
-                 workspace=None, out=None, final_out=None, y_dtype=None):
+                 workspace=None, out=None, final_out=None, y_dtype=None, reset=None):
         self._lib = load_library()
         self._dims = _scan_dims(x, Bm, chunk)
         dims = self._dims
@@ -271,15 +288,16 @@ class PreparedChunkScan:
             workspace = torch.empty(need.value, dtype=torch.uint8, device=x.device)
         elif (not workspace.is_cuda) or workspace.dtype != torch.uint8 or not workspace.is_contiguous():
             raise ValueError("SSD workspace must be a contiguous uint8 GPU tensor")
-        self._keep = (x, dt, A, Bm, Cm, D, initial_states, workspace)
+        reset = _reset_mask(reset, dims)
+        self._keep = (x, dt, A, Bm, Cm, D, initial_states, workspace, reset)
         self._device = x.device
         self._args = (x.data_ptr(), dt.data_ptr(), A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), _ptr(D),
-                      _ptr(initial_states), self.y.data_ptr(), _ptr(self.final), workspace.data_ptr(),
+                      _ptr(initial_states), _ptr(reset), self.y.data_ptr(), _ptr(self.final), workspace.data_ptr(),
                       workspace.numel())
 
     def __call__(self):
-        rc = self._lib.ssd_chunk_scan_fwd(byref(self._dims), self._code, *self._args,
-                                          torch.cuda.current_stream(self._device).cuda_stream)
+        rc = self._lib.ssd_chunk_scan_reset_fwd(byref(self._dims), self._code, *self._args,
+                                                torch.cuda.current_stream(self._device).cuda_stream)
         if rc:
             _check(self._lib, rc)
         return self.y, self.final
@@ -308,6 +326,7 @@ def ssd_chunk_scan_onepass(
     out: Optional[torch.Tensor] = None,
     final_out: Optional[torch.Tensor] = None,
     y_dtype: Optional[torch.dtype] = None,
+    reset: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """The forward as one kernel and one pass over the inputs (bf16 only, no workspace); same results
     as ssd_chunk_scan, which takes this path by itself when the batch is large enough.  Raises
@@ -323,8 +342,9 @@ def ssd_chunk_scan_onepass(
         shape = (dims.batch, dims.nheads, dims.headdim, dims.dstate)
         final = torch.empty(shape, dtype=torch.float32, device=x.device) if final_out is None else final_out
         _require(final, "final_out", shape, torch.float32)
+    reset = _reset_mask(reset, dims)
     rc = lib.ssd_chunk_scan_onepass_fwd(byref(dims), code, x.data_ptr(), dt.data_ptr(), A.data_ptr(),
-                                        Bm.data_ptr(), Cm.data_ptr(), _ptr(D), _ptr(initial_states),
+                                        Bm.data_ptr(), Cm.data_ptr(), _ptr(D), _ptr(initial_states), _ptr(reset),
                                         y.data_ptr(), _ptr(final), _stream_ptr(x))
     _check(lib, rc)
     return y, final
