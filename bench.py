@@ -38,6 +38,10 @@ import sys
 import time
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE
+# on this very command (profiles/chunk_scan_forward_policy_bf16.md: 200 800 + 278 500 KiB, copy-kernel
+# calibration factor 1.00); counters cannot be read from inside this script, so the figure is carried here
+MEASURED_TRAFFIC_BYTES = {("policy_bf16", 256, "onepass_scan"): 490.8e6}
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
@@ -189,7 +193,8 @@ def main():
                         "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "dense_TFLOPs": round(tf, 1),
                         "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)}
         roofline = {"kernel": "onepass_scan", "bound": "hbm", "achieved": onepass_info["GBps"],
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": onepass_info["hbm_frac"], "traffic": None}
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": onepass_info["hbm_frac"],
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, w.batch, "onepass_scan"))}
     else:
         dom = max(stages, key=lambda k: stages[k]["ms"])
         roofline = {"kernel": dom, "bound": "hbm", "achieved": stages[dom]["GBps"], "peak": HBM_PEAK_GBS,
