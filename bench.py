@@ -19,6 +19,8 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
                64 steps as one launch of the multi-step kernel
   reference_suite  the reference's historical benchmark cases for this path (batch 4, seq_len 4096,
                BFloat16), for the SSD op alone, in the reference's result schema
+  mamba2_block the block around the scan at the policy shape (d_model = nheads*headdim): whole block, and the
+               library's pre-scan and post-scan kernels alone with their GB/s
   cpu_baseline the plain-C oracle (sequential recurrence, float32, OpenMP) timed on this
                box's host cores on a bounded batch slice of the same workload
 
@@ -55,6 +57,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-stream-step", action="store_true")
     ap.add_argument("--no-reference-suite", action="store_true")
+    ap.add_argument("--no-block", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise kernel over 256 MiB in / 256 MiB out three times, the known-size "
@@ -293,6 +296,40 @@ def main():
             {"name": "mamba2_infer_prefill", "time_ms": t_fwd, "config": cfg},
             {"name": "mamba2_infer_step", "time_ms": t_step, "config": {"batch": 4, "seq_len": 1, "dtype": "BFloat16"}},
         ]
+
+    # ---- the Mamba-2 block around the scan (projections by torch's GEMM, the rest in the library) ----
+    if not args.no_block:
+        from trading_bot_0_amd import Mamba2Block, block_post, block_pre
+        bw = WORKLOADS["policy_bf16"]
+        blk = Mamba2Block(d_model=bw.nheads * bw.headdim, nheads=bw.nheads, headdim=bw.headdim, dstate=bw.dstate,
+                          ngroups=bw.ngroups, chunk=bw.chunk)
+        u = torch.randn(bw.batch, bw.seqlen, blk.d_model, device="cuda").to(torch.bfloat16)
+        zx = torch.matmul(u, blk.in_proj.to(u.dtype).t()).contiguous()
+        xs_, bs_, cs_, ds_ = block_pre(zx, blk.conv_w, blk.conv_b, blk.dt_bias, blk.H, blk.P, blk.N, blk.G)
+        ys_, _ = ssd.ssd_chunk_scan(xs_, ds_, blk.A, bs_, cs_, blk.D, chunk=bw.chunk, return_final_states=False)
+
+        def timed(fn, n=20):
+            for _ in range(3):
+                fn()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            a.record()
+            for _ in range(n):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / n
+
+        e = 2
+        pre_bytes = e * bw.batch * bw.seqlen * (2 * (blk.conv_dim + blk.H))          # reads x|B|C|dt, writes them
+        post_bytes = e * bw.batch * bw.seqlen * 3 * blk.d_inner                     # reads y and z, writes out
+        t_pre = timed(lambda: block_pre(zx, blk.conv_w, blk.conv_b, blk.dt_bias, blk.H, blk.P, blk.N, blk.G))
+        t_post = timed(lambda: block_post(ys_, zx, blk.norm_w, blk.H, blk.P, blk.N, blk.G))
+        t_block = timed(lambda: blk.forward(u), n=10)
+        out["mamba2_block"] = {"d_model": blk.d_model, "ms": round(t_block, 4),
+                               "pre_ms": round(t_pre, 4), "pre_GBps": round(pre_bytes / t_pre / 1e6, 1),
+                               "post_ms": round(t_post, 4), "post_GBps": round(post_bytes / t_post / 1e6, 1)}
+        del u, zx, xs_, bs_, cs_, ds_, ys_, blk
 
     # ---- CPU baseline: the C oracle on a bounded batch slice ---------------------------------
     if not args.no_cpu_baseline:

@@ -176,6 +176,33 @@ int ssd_steps_fwd(const ssd_step_dims *dims, int64_t nsteps, int dtype, float *s
                   const void *x, const void *dt, const float *A, const void *Bm, const void *Cm, const float *D,
                   void *y, void *hip_stream);
 
+/* ---- The memory-bound stages of a Mamba-2 block around the scan ("next" after the scan itself) ----------
+ * The layer that would take GqaBlock's place in patch_trunk (trading_bots/src/torch/model/trading_model.rs:
+ * 589-606, trading_bots/src/torch/model/blocks/gqa.rs:82-109; the reference already mixes with a causal
+ * depthwise filter, gqa.rs:172-178): in-projection -> [pre] -> SSD scan -> [post] -> out-projection.  The two
+ * projections are plain GEMMs and stay with the caller's BLAS; pre and post are these two kernels.
+ * zxbcdt [B,L,E] is the in-projection's output, E = 2*H*P + 2*G*N + H channels per timestep laid out as
+ * [ z | x | B | C | dt_raw ]; activations are float32 (dtype 0) or bf16 (dtype 1; dtype 2 = bf16 with the
+ * scan's float32 y as the input of post); parameters are float32. */
+typedef struct {
+    int64_t batch, seqlen, nheads, headdim, dstate, ngroups, d_conv;
+} ssd_block_dims;
+
+/* x [B,L,H,P], Bm, Cm [B,L,G,N] = silu(causal depthwise conv1d of width d_conv (2..4) over the x | B | C
+ * channels + conv_b) and dt [B,L,H] = softplus(dt_raw + dt_bias): exactly the tensors ssd_chunk_scan_fwd takes.
+ * conv_w [H*P + 2*G*N, d_conv] (tap d_conv-1 multiplies the current timestep), conv_b [H*P + 2*G*N].
+ * conv_state_in [B, d_conv-1, H*P + 2*G*N] (activation dtype) holds the x | B | C inputs of the d_conv-1
+ * timesteps before the first one (NULL = zeros); conv_state_out (nullable) receives those of the last d_conv-1
+ * timesteps: the conv's streaming state, carried next to the SSM state (cf. StreamState,
+ * trading_bots/src/torch/model/trading_model.rs:56-75).  The two may alias only for seqlen 1. */
+int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt, const float *conv_w,
+                      const float *conv_b, const float *dt_bias, const void *conv_state_in, void *conv_state_out,
+                      void *x, void *Bm, void *Cm, void *dt, void *hip_stream);
+
+/* out [B,L,H*P] = rmsnorm(y * silu(z)) * norm_w over the H*P channels of a timestep (z from zxbcdt). */
+int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,
+                       const float *norm_w, float eps, void *out, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,135 @@
+"""The Mamba-2 block stages around the scan through the C ABI (pre: conv + SiLU + softplus; post: gated
+RMSNorm) against the numpy oracle, and the assembled block (torch GEMMs + library kernels) against the
+oracle's block, batched and streamed."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mamba2_block_oracle as blk
+from trading_bot_0_amd import Mamba2Block, SsdError, block_post, block_pre
+
+from _util import np64, rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
+
+
+def params(H, P, N, G, K, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    C = H * P + 2 * G * N
+    return dict(conv_w=torch.randn(C, K, generator=g).cuda() / 2, conv_b=torch.randn(C, generator=g).cuda() / 4,
+                dt_bias=torch.randn(H, generator=g).cuda(), norm_w=torch.randn(H * P, generator=g).cuda())
+
+
+def close(out, ref, dtype, what):
+    """float32: max|err| / rms <= 2e-5.  bf16: these stages are elementwise and store bf16, so every element
+    must be within two bf16 ulps (2^-7 relative) of the float64 result, plus a floor of 1e-3 rms for values
+    that cancel to nearly zero."""
+    o = out.detach().float().cpu().numpy().astype(np.float64).reshape(ref.shape)
+    assert np.isfinite(o).all(), what
+    if dtype == torch.float32:
+        e = rel_err(out, ref)
+        assert e <= TOL[dtype], f"{what}: {e:.3e}"
+        return e
+    rms = np.sqrt(np.mean(ref * ref))
+    bad = np.abs(o - ref) > 2.0 ** -7 * np.abs(ref) + 1e-3 * rms
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements off by more than two bf16 ulps"
+    return 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 8, 32, 64, 1, 4), (3, 7, 8, 16, 16, 2, 3), (1, 130, 16, 64, 128, 2, 2),
+                                   (4, 1, 8, 32, 64, 1, 4), (2, 2, 8, 32, 32, 4, 4)])
+def test_pre_scan_stage(shape, dtype):
+    Bsz, L, H, P, N, G, K = shape
+    p = params(H, P, N, G, K)
+    E = 2 * H * P + 2 * G * N + H
+    g = torch.Generator().manual_seed(1)
+    z = torch.randn(Bsz, L, E, generator=g).to(dtype).cuda()
+    st = (torch.randn(Bsz, K - 1, H * P + 2 * G * N, generator=g)).to(dtype).cuda()
+    for state in (None, st):
+        got = block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=state, return_conv_state=True)
+        ref = blk.block_pre(np64(z), np64(p["conv_w"]), np64(p["conv_b"]), np64(p["dt_bias"]), H, P, N, G,
+                            None if state is None else np64(state))
+        for name, a, b in zip(("x", "B", "C", "dt"), got[:4], ref[:4]):
+            close(a, b, dtype, f"pre {name}")
+        assert torch.equal(got[4].float().cpu(), torch.from_numpy(ref[4]).float()), "conv state is a copy of inputs"
+        # without asking for the state the outputs are the same
+        again = block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=state)
+        assert all(torch.equal(a, b) for a, b in zip(again, got[:4]))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 8, 32, 64, 1), (3, 7, 8, 16, 16, 2), (1, 33, 16, 64, 128, 2), (2, 5, 32, 64, 16, 1)])
+def test_post_scan_stage(shape, dtype):
+    Bsz, L, H, P, N, G = shape
+    p = params(H, P, N, G, 4)
+    g = torch.Generator().manual_seed(2)
+    z = torch.randn(Bsz, L, 2 * H * P + 2 * G * N + H, generator=g).to(dtype).cuda()
+    y = (torch.randn(Bsz, L, H, P, generator=g) * 3).to(dtype).cuda()
+    ref = blk.block_post(np64(y), np64(z), np64(p["norm_w"]), 1e-5)
+    close(block_post(y, z, p["norm_w"], H, P, N, G), ref, dtype, "post")
+    if dtype == torch.bfloat16:      # the scan's float32 y as input
+        y32 = y.float() + 1e-3
+        close(block_post(y32, z, p["norm_w"], H, P, N, G), blk.block_post(np64(y32), np64(z), np64(p["norm_w"]), 1e-5),
+              dtype, "post from float32 y")
+
+
+def oracle_params(b):
+    return dict(in_proj=np64(b.in_proj), conv_w=np64(b.conv_w), conv_b=np64(b.conv_b), dt_bias=np64(b.dt_bias),
+                A=np64(b.A), D=np64(b.D), norm_w=np64(b.norm_w), out_proj=np64(b.out_proj), H=b.H, P=b.P, N=b.N, G=b.G,
+                eps=b.eps)
+
+
+def test_block_forward_float32_matches_the_oracle_block():
+    b = Mamba2Block(d_model=64, nheads=8, headdim=32, dstate=64, ngroups=1, seed=3)
+    u = torch.randn(2, 200, 64, generator=torch.Generator().manual_seed(4)).cuda()
+    out = b.forward(u)
+    ref, _, _ = blk.block_forward(np64(u), oracle_params(b))
+    assert rel_err(out, ref) <= 1e-3          # float32 GEMMs (hipBLASLt) on top of the 1e-4 scan
+
+
+def test_block_forward_bf16_is_close_to_the_oracle_block():
+    b = Mamba2Block(d_model=64, nheads=8, headdim=32, dstate=64, ngroups=1, seed=3)
+    u = torch.randn(2, 200, 64, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).cuda()
+    out = b.forward(u)
+    ref, _, _ = blk.block_forward(np64(u), oracle_params(b))
+    # every bf16 tensor between the stages (projection output, x, B, C, dt, y, normed y) is rounded once: 2^-9
+    # each, about five of them in a chain
+    assert out.dtype == torch.bfloat16 and rel_err(out, ref) <= 1e-1
+    corr = np.corrcoef(out.float().cpu().numpy().ravel(), ref.ravel())[0, 1]
+    assert corr > 0.9995
+
+
+def test_block_streams_prefix_then_steps_equals_the_window():
+    b = Mamba2Block(d_model=64, nheads=8, headdim=32, dstate=64, ngroups=1, seed=5)
+    u = torch.randn(3, 96, 64, generator=torch.Generator().manual_seed(6)).cuda()
+    full = b.forward(u)
+    st = b.new_state(3, dtype=torch.float32)
+    outs = [b.forward(u[:, :70].contiguous(), state=st)]
+    for t in range(70, 96):
+        outs.append(b.step(u[:, t].contiguous(), st).unsqueeze(1))
+    got = torch.cat(outs, 1)
+    torch.cuda.synchronize()
+    assert rel_err(got, np64(full)) <= 1e-3
+    ref, conv, ssm = blk.block_forward(np64(u), oracle_params(b))
+    assert rel_err(st.ssm.state, ssm) <= 1e-3 and rel_err(st.conv, conv) <= 1e-6
+    # a restarted stream forgets: zero both states of row 1 and compare with a fresh stream on the same input
+    st.reset_rows(torch.tensor([1], device="cuda"))
+    fresh = b.new_state(3, dtype=torch.float32)
+    o1 = b.step(u[:, 0].contiguous(), st)
+    o2 = b.step(u[:, 0].contiguous(), fresh)
+    assert torch.equal(o1[1], o2[1])
+
+
+def test_block_stage_errors():
+    p = params(8, 32, 64, 1, 4)
+    z = torch.randn(2, 4, 2 * 256 + 128 + 8).cuda()
+    with pytest.raises(ValueError, match="channels"):
+        block_pre(z[:, :, :-8].contiguous(), p["conv_w"], p["conv_b"], p["dt_bias"], 8, 32, 64, 1)
+    with pytest.raises(SsdError) as ei:        # width-5 conv is not built
+        block_pre(z, torch.randn(256 + 128, 5).cuda(), p["conv_b"], p["dt_bias"], 8, 32, 64, 1)
+    assert ei.value.code == 2
+    with pytest.raises(ValueError, match="conv_state"):
+        block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], 8, 32, 64, 1, conv_state=torch.zeros(2, 2, 384).cuda())

@@ -1,0 +1,191 @@
+"""A Mamba-2 block around the SSD scan: in-projection -> causal depthwise conv + SiLU on (x, B, C), softplus on
+dt -> SSD scan -> gated RMSNorm -> out-projection.  It is the layer that would sit where the reference's
+encoder block sits in `patch_trunk` (`trading_bots/src/torch/model/trading_model.rs:589-606`,
+`trading_bots/src/torch/model/blocks/gqa.rs:82-109`), with the conv's streaming state carried next to the SSM
+state the way the reference's `StreamState` carries its encoder memory (`trading_model.rs:56-75`).
+
+The two projections are torch matmuls (plain GEMMs); everything between them runs in libssd_hip: the pre-scan
+and post-scan kernels bound here and the scan / step of `ssd.py`.
+"""
+from __future__ import annotations
+
+import math
+from ctypes import POINTER, Structure, byref, c_float, c_int, c_int64, c_void_p
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import ssd
+from .stream_state import SsdStreamState
+
+
+class SsdBlockDims(Structure):
+    _fields_ = [(n, c_int64) for n in ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "d_conv")]
+
+
+_bound = False
+
+
+def _lib():
+    global _bound
+    lib = ssd.load_library()
+    if not _bound:
+        P = c_void_p
+        lib.ssd_block_pre_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
+        lib.ssd_block_post_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, P]
+        lib.ssd_block_pre_fwd.restype = c_int
+        lib.ssd_block_post_fwd.restype = c_int
+        _bound = True
+    return lib
+
+
+def in_proj_width(nheads, headdim, dstate, ngroups) -> int:
+    return 2 * nheads * headdim + 2 * ngroups * dstate + nheads
+
+
+def block_pre(zxbcdt, conv_w, conv_b, dt_bias, nheads, headdim, dstate, ngroups, conv_state=None,
+              return_conv_state=False):
+    """zxbcdt [B,L,E] -> (x [B,L,H,P], Bm, Cm [B,L,G,N], dt [B,L,H][, conv state [B,d_conv-1,C]])."""
+    lib = _lib()
+    if zxbcdt.dim() != 3:
+        raise ValueError(f"block input must be rank-3 [batch, seqlen, channels], got {tuple(zxbcdt.shape)}")
+    Bsz, L, E = zxbcdt.shape
+    H, P, N, G = nheads, headdim, dstate, ngroups
+    C = H * P + 2 * G * N
+    if E != in_proj_width(H, P, N, G):
+        raise ValueError(f"block input must have {in_proj_width(H, P, N, G)} channels, got {E}")
+    dtype = zxbcdt.dtype
+    code = ssd._dtype_code(zxbcdt)
+    ssd._require(zxbcdt, "zxbcdt", (Bsz, L, E), dtype)
+    if conv_w.dim() != 2 or conv_w.shape[0] != C:
+        raise ValueError(f"conv_w must be [{C}, d_conv], got {tuple(conv_w.shape)}")
+    d_conv = conv_w.shape[1]
+    ssd._require(conv_w, "conv_w", (C, d_conv), torch.float32)
+    ssd._require(conv_b, "conv_b", (C,), torch.float32)
+    ssd._require(dt_bias, "dt_bias", (H,), torch.float32)
+    if conv_state is not None:
+        ssd._require(conv_state, "conv_state", (Bsz, d_conv - 1, C), dtype)
+    dev = zxbcdt.device
+    x = torch.empty((Bsz, L, H, P), dtype=dtype, device=dev)
+    Bm = torch.empty((Bsz, L, G, N), dtype=dtype, device=dev)
+    Cm = torch.empty((Bsz, L, G, N), dtype=dtype, device=dev)
+    dt = torch.empty((Bsz, L, H), dtype=dtype, device=dev)
+    new_state = torch.empty((Bsz, d_conv - 1, C), dtype=dtype, device=dev) if return_conv_state else None
+    dims = SsdBlockDims(Bsz, L, H, P, N, G, d_conv)
+    ssd._check(lib, lib.ssd_block_pre_fwd(byref(dims), code, zxbcdt.data_ptr(), conv_w.data_ptr(), conv_b.data_ptr(),
+                                          dt_bias.data_ptr(), ssd._ptr(conv_state), ssd._ptr(new_state), x.data_ptr(),
+                                          Bm.data_ptr(), Cm.data_ptr(), dt.data_ptr(), ssd._stream_ptr(zxbcdt)))
+    return (x, Bm, Cm, dt, new_state) if return_conv_state else (x, Bm, Cm, dt)
+
+
+def block_post(y, zxbcdt, norm_w, nheads, headdim, dstate, ngroups, eps=1e-5):
+    """out [B,L,H*P] = rmsnorm(y * silu(z)) * norm_w; y [B,L,H,P] in the activation dtype or float32."""
+    lib = _lib()
+    Bsz, L, E = zxbcdt.shape
+    H, P, N, G = nheads, headdim, dstate, ngroups
+    dtype = zxbcdt.dtype
+    code = ssd._dtype_code(zxbcdt)
+    if y.dtype != dtype:
+        if not (dtype == torch.bfloat16 and y.dtype == torch.float32):
+            raise ValueError(f"block y must be {dtype} (or float32 with bf16 activations), got {y.dtype}")
+        code = ssd.SSD_DTYPE_BF16_Y32
+    ssd._require(zxbcdt, "zxbcdt", (Bsz, L, in_proj_width(H, P, N, G)), dtype)
+    ssd._require(y, "y", (Bsz, L, H, P), y.dtype)
+    ssd._require(norm_w, "norm_w", (H * P,), torch.float32)
+    out = torch.empty((Bsz, L, H * P), dtype=dtype, device=zxbcdt.device)
+    dims = SsdBlockDims(Bsz, L, H, P, N, G, 4)
+    ssd._check(lib, lib.ssd_block_post_fwd(byref(dims), code, y.data_ptr(), zxbcdt.data_ptr(), norm_w.data_ptr(),
+                                           c_float(eps), out.data_ptr(), ssd._stream_ptr(zxbcdt)))
+    return out
+
+
+@dataclass
+class Mamba2StreamState:
+    """Streaming memory of one block: the conv's last d_conv-1 inputs and the SSM state."""
+    conv: torch.Tensor          # [B, d_conv-1, H*P + 2*G*N], activation dtype
+    ssm: SsdStreamState         # [B, H, P, N] float32
+
+    def reset(self) -> None:
+        self.conv.zero_()
+        self.ssm.reset()
+
+    def reset_rows(self, rows: torch.Tensor) -> None:
+        if rows.dtype == torch.bool:
+            self.conv.mul_((~rows).to(self.conv.dtype).view(-1, 1, 1))
+        else:
+            self.conv.index_fill_(0, rows, 0.0)
+        self.ssm.reset_rows(rows)
+
+
+class Mamba2Block:
+    """Parameters and forward of one block.  Parameters are float32 masters; the projections run in the
+    activation dtype of the input (bf16 on the GPU, as the reference policy runs,
+    `trading_bots/src/torch/model/trading_model.rs:140-146`)."""
+
+    def __init__(self, d_model, nheads, headdim, dstate, ngroups=1, d_conv=4, chunk=128, eps=1e-5, device="cuda",
+                 seed=0):
+        self.d_model, self.H, self.P, self.N, self.G = d_model, nheads, headdim, dstate, ngroups
+        self.d_conv, self.chunk, self.eps = d_conv, chunk, eps
+        self.d_inner = nheads * headdim
+        self.conv_dim = self.d_inner + 2 * ngroups * dstate
+        E = in_proj_width(nheads, headdim, dstate, ngroups)
+        g = torch.Generator(device="cpu")
+        g.manual_seed(seed)
+
+        def rnd(*shape, scale=1.0):
+            return (torch.randn(*shape, generator=g) * scale).to(device)
+
+        self.in_proj = rnd(E, d_model, scale=1.0 / math.sqrt(d_model))
+        self.conv_w = rnd(self.conv_dim, d_conv, scale=1.0 / math.sqrt(d_conv))
+        self.conv_b = rnd(self.conv_dim, scale=0.1)
+        # dt after softplus spread over [1e-3, 1e-1] (log-uniform), as Mamba-2 initialises it
+        dt0 = torch.exp(torch.rand(nheads, generator=g) * (math.log(0.1) - math.log(1e-3)) + math.log(1e-3))
+        self.dt_bias = (dt0 + torch.log(-torch.expm1(-dt0))).to(device)
+        self.A_log = torch.log(torch.rand(nheads, generator=g) * 15.0 + 1.0).to(device)
+        self.D = torch.ones(nheads, device=device)
+        self.norm_w = torch.ones(self.d_inner, device=device)
+        self.out_proj = rnd(d_model, self.d_inner, scale=1.0 / math.sqrt(self.d_inner))
+
+    @property
+    def A(self) -> torch.Tensor:
+        return -torch.exp(self.A_log)
+
+    def new_state(self, batch, dtype=torch.bfloat16) -> Mamba2StreamState:
+        conv = torch.zeros((batch, self.d_conv - 1, self.conv_dim), dtype=dtype, device=self.in_proj.device)
+        return Mamba2StreamState(conv, SsdStreamState.build(batch, self.H, self.P, self.N, device=self.in_proj.device))
+
+    def forward(self, u: torch.Tensor, state: Optional[Mamba2StreamState] = None,
+                reset: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """u [B,L,d_model] -> [B,L,d_model].  With `state`, continues from it and leaves it at the end of the
+        window (a prefix scan; then `step` per bar)."""
+        if u.dim() != 3 or u.shape[2] != self.d_model:
+            raise ValueError(f"block input must be [batch, seqlen, {self.d_model}], got {tuple(u.shape)}")
+        if reset is not None and state is not None:
+            raise ValueError("restarts inside the window and a carried conv state cannot be combined")
+        dt_ = u.dtype
+        zxbcdt = torch.matmul(u, self.in_proj.to(dt_).t()).contiguous()
+        if state is None:
+            x, Bm, Cm, dt = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G)
+            y, _ = ssd.ssd_chunk_scan(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk, return_final_states=False,
+                                      reset=reset)
+        else:
+            x, Bm, Cm, dt, conv = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N,
+                                            self.G, conv_state=state.conv, return_conv_state=True)
+            state.conv = conv
+            y = state.ssm.init_from_prefix(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk)
+        yn = block_post(y, zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
+        return torch.matmul(yn, self.out_proj.to(dt_).t())
+
+    def step(self, u_t: torch.Tensor, state: Mamba2StreamState) -> torch.Tensor:
+        """One timestep for every stream: u_t [B,d_model] -> [B,d_model]; advances `state` in place."""
+        if u_t.dim() != 2 or u_t.shape[1] != self.d_model:
+            raise ValueError(f"block step input must be [batch, {self.d_model}], got {tuple(u_t.shape)}")
+        dt_ = u_t.dtype
+        zxbcdt = torch.matmul(u_t, self.in_proj.to(dt_).t()).unsqueeze(1).contiguous()
+        x, Bm, Cm, dt, conv = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N,
+                                        self.G, conv_state=state.conv, return_conv_state=True)
+        state.conv = conv
+        y = state.ssm.step(x[:, 0], dt[:, 0], self.A, Bm[:, 0], Cm[:, 0], self.D)
+        yn = block_post(y.unsqueeze(1), zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
+        return torch.matmul(yn[:, 0], self.out_proj.to(dt_).t())

@@ -345,4 +345,61 @@ int ssd_steps_fwd(const ssd_step_dims *dims, int64_t nsteps, int dtype, float *s
     return e == hipSuccess ? SSD_OK : hip_fail(e, "multi-step launch");
 }
 
+static int make_block_shape(const ssd_block_dims *d, int dtype, ssd::BlockShape *out) {
+    if (d == nullptr) return fail(SSD_ERR_INVALID, "ssd: dims must not be NULL");
+    if (int rc = check_dtype(dtype)) return rc;
+    if (d->batch <= 0 || d->seqlen <= 0)
+        return fail(SSD_ERR_INVALID, "ssd: batch and seqlen must be positive, got %lld %lld", (long long)d->batch,
+                    (long long)d->seqlen);
+    if (int rc = check_state_dims(d->nheads, d->headdim, d->dstate, d->ngroups)) return rc;
+    const int64_t E = 2 * d->nheads * d->headdim + 2 * d->ngroups * d->dstate + d->nheads;
+    if (d->batch * d->seqlen > 0x7fffffff || d->batch * d->seqlen * E / 8 > 0x7fffffffffLL)
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: batch*seqlen exceeds 2^31-1");
+    if (E % (dtype == SSD_DTYPE_F32 ? 4 : 8) != 0)
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: the %lld channels of a timestep must be a whole number of 16-byte "
+                                         "pieces (nheads a multiple of %d)", (long long)E, dtype == SSD_DTYPE_F32 ? 4 : 8);
+    ssd::BlockShape s{(int)d->batch, (int)d->seqlen, (int)d->nheads, (int)d->headdim, (int)d->dstate,
+                      (int)d->ngroups, (int)d->d_conv};
+    if (!ssd::block_supported(s))
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: block stages need d_conv 2..4 (got %lld) and nheads*headdim <= 2048",
+                    (long long)d->d_conv);
+    *out = s;
+    return SSD_OK;
+}
+
+int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt, const float *conv_w,
+                      const float *conv_b, const float *dt_bias, const void *conv_state_in, void *conv_state_out,
+                      void *x, void *Bm, void *Cm, void *dt, void *hip_stream) {
+    ssd::BlockShape s;
+    if (int rc = make_block_shape(dims, dtype, &s)) return rc;
+    REQUIRE_PTR(zxbcdt);
+    REQUIRE_PTR(conv_w);
+    REQUIRE_PTR(conv_b);
+    REQUIRE_PTR(dt_bias);
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(Bm);
+    REQUIRE_PTR(Cm);
+    REQUIRE_PTR(dt);
+    OPTIONAL_PTR(conv_state_in);
+    OPTIONAL_PTR(conv_state_out);
+    if (conv_state_in != nullptr && conv_state_in == conv_state_out && s.L > 1)
+        return fail(SSD_ERR_INVALID, "ssd: conv_state_in and conv_state_out may alias only for seqlen 1");
+    hipError_t e = ssd::launch_block_pre(s, dtype == SSD_DTYPE_F32 ? 0 : 1, zxbcdt, conv_w, conv_b, dt_bias,
+                                         conv_state_in, conv_state_out, x, Bm, Cm, dt, (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "block pre-scan launch");
+}
+
+int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,
+                       const float *norm_w, float eps, void *out, void *hip_stream) {
+    ssd::BlockShape s;
+    if (int rc = make_block_shape(dims, dtype, &s)) return rc;
+    REQUIRE_PTR(y);
+    REQUIRE_PTR(zxbcdt);
+    REQUIRE_PTR(norm_w);
+    REQUIRE_PTR(out);
+    if (!(eps > 0.f)) return fail(SSD_ERR_INVALID, "ssd: eps must be positive");
+    hipError_t e = ssd::launch_block_post(s, dtype, y, zxbcdt, norm_w, eps, out, (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "block post-scan launch");
+}
+
 }  // extern "C"

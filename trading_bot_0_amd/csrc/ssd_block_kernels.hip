@@ -1,0 +1,255 @@
+// The two memory-bound stages of a Mamba-2 block around the SSD scan (gfx950):
+//   pre   causal depthwise conv1d (width d_conv) + bias + SiLU over the x, B, C channels of the
+//         in-projection's output, split into the tensors the scan takes, and dt = softplus(dt_raw + dt_bias)
+//   post  gated RMSNorm: out = rmsnorm(y * silu(z)) * weight
+// The projections on either side are plain GEMMs and stay with the caller's BLAS.
+//
+// Input layout (per timestep, E = 2*H*P + 2*G*N + H channels): [ z | x | B | C | dt_raw ].
+#include "ssd_device.h"
+
+namespace ssd {
+
+__device__ inline float silu(float v) { return v * __builtin_amdgcn_rcpf(1.f + __expf(-v)); }
+__device__ inline float softplus(float v) { return v > 20.f ? v : log1pf(__expf(v)); }
+
+template <typename T> struct Pack8;  // eight consecutive channels
+template <> struct Pack8<__bf16> {
+    uint4 u;
+    __device__ inline float get(int i) const {
+        const unsigned w = (&u.x)[i >> 1];
+        return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+    }
+    static __device__ inline Pack8 load(const __bf16 *p) { return Pack8{*reinterpret_cast<const uint4 *>(p)}; }
+    static __device__ inline void store(__bf16 *p, const float (&v)[8]) {
+        uint4 o;
+        o.x = pack_bf16x2(v[0], v[1]);
+        o.y = pack_bf16x2(v[2], v[3]);
+        o.z = pack_bf16x2(v[4], v[5]);
+        o.w = pack_bf16x2(v[6], v[7]);
+        *reinterpret_cast<uint4 *>(p) = o;
+    }
+};
+template <> struct Pack8<float> {
+    float4 a, b;
+    __device__ inline float get(int i) const { return i < 4 ? (&a.x)[i] : (&b.x)[i - 4]; }
+    static __device__ inline Pack8 load(const float *p) {
+        return Pack8{*reinterpret_cast<const float4 *>(p), *reinterpret_cast<const float4 *>(p + 4)};
+    }
+    static __device__ inline void store(float *p, const float (&v)[8]) {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+};
+
+// One thread per (run of kPreSteps timesteps, 8 channels of x | B | C): the filter taps of its channels are
+// loaded once and the d_conv-1 previous input rows slide through registers, so every input row is read once
+// per run.  The dt channels are done by the threads after those, one (timestep, 8 heads) each, so that no
+// wave mixes the two code paths.  History
+// before t = 0 comes from state_in [B, d_conv-1, C] (the last d_conv-1 input rows of the previous call) or is
+// zero; state_out receives the last d_conv-1 input rows.
+constexpr int kPreSteps = 8;
+
+template <typename T, int DCONV>
+__global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zxbcdt, const float *__restrict__ conv_w,
+                                                        const float *__restrict__ conv_b, const float *__restrict__ dt_bias,
+                                                        const T *__restrict__ state_in, T *__restrict__ state_out,
+                                                        T *__restrict__ x, T *__restrict__ Bm, T *__restrict__ Cm,
+                                                        T *__restrict__ dt, BlockShape s) {
+    const int DI = s.H * s.P, GN = s.G * s.N, C = DI + 2 * GN, E = 2 * DI + 2 * GN + s.H;
+    const int CP = C / 8, HP8 = (s.H + 7) / 8;
+    const int runs = (s.L + kPreSteps - 1) / kPreSteps;
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long conv_total = (long long)s.B * runs * CP;
+    if (gid >= conv_total) {
+        // the threads after the conv threads: dt = softplus(dt_raw + dt_bias), one (timestep, 8 heads) each
+        const long long d = gid - conv_total;
+        if (d >= (long long)s.B * s.L * HP8) return;
+        const int h0 = (int)(d % HP8) * 8;
+        const long long bt = d / HP8;
+        const T *src = zxbcdt + (size_t)bt * E + 2 * DI + 2 * GN;
+        for (int h = h0; h < min(h0 + 8, s.H); ++h) dt[(size_t)bt * s.H + h] = (T)softplus((float)src[h] + dt_bias[h]);
+        return;
+    }
+    const int piece = (int)(gid % CP);
+    const long long br = gid / CP;
+    const int t0 = (int)(br % runs) * kPreSteps, b = (int)(br / runs);
+    const int t1 = min(t0 + kPreSteps, s.L);
+    const T *row0 = zxbcdt + ((size_t)b * s.L) * E;  // this batch row's first timestep
+    const int c0 = piece * 8;  // channel within [x | B | C]
+    float w[8][DCONV], bias[8];
+    {   // the taps of 8 consecutive channels are 8*DCONV consecutive floats
+        float wf[8 * DCONV];
+#pragma unroll
+        for (int q = 0; q < 2 * DCONV; ++q) {
+            const float4 v = *reinterpret_cast<const float4 *>(conv_w + (size_t)c0 * DCONV + 4 * q);
+            wf[4 * q] = v.x; wf[4 * q + 1] = v.y; wf[4 * q + 2] = v.z; wf[4 * q + 3] = v.w;
+        }
+        const float4 b0 = *reinterpret_cast<const float4 *>(conv_b + c0), b1 = *reinterpret_cast<const float4 *>(conv_b + c0 + 4);
+        bias[0] = b0.x; bias[1] = b0.y; bias[2] = b0.z; bias[3] = b0.w;
+        bias[4] = b1.x; bias[5] = b1.y; bias[6] = b1.z; bias[7] = b1.w;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int k = 0; k < DCONV; ++k) w[i][k] = wf[i * DCONV + k];
+        }
+    }
+    // win[k] = input row t - (DCONV-1) + k for the current t; the last slot is loaded per timestep
+    float win[DCONV][8];
+#pragma unroll
+    for (int k = 0; k < DCONV - 1; ++k) {
+        const int ts = t0 - (DCONV - 1) + k;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) win[k][i] = 0.f;
+        if (ts >= 0) {
+            const Pack8<T> v = Pack8<T>::load(row0 + (size_t)ts * E + DI + c0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) win[k][i] = v.get(i);
+        } else if (state_in != nullptr) {
+            const Pack8<T> v = Pack8<T>::load(state_in + ((size_t)b * (DCONV - 1) + (DCONV - 1 + ts)) * C + c0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) win[k][i] = v.get(i);
+        }
+    }
+    T *dst;
+    int dst_stride;
+    if (c0 < DI) {
+        dst = x + ((size_t)b * s.L) * DI + c0;
+        dst_stride = DI;
+    } else if (c0 < DI + GN) {
+        dst = Bm + ((size_t)b * s.L) * GN + (c0 - DI);
+        dst_stride = GN;
+    } else {
+        dst = Cm + ((size_t)b * s.L) * GN + (c0 - DI - GN);
+        dst_stride = GN;
+    }
+    for (int t = t0; t < t1; ++t) {
+        const Pack8<T> v = Pack8<T>::load(row0 + (size_t)t * E + DI + c0);
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            win[DCONV - 1][i] = v.get(i);
+            float a = bias[i];
+#pragma unroll
+            for (int k = 0; k < DCONV; ++k) a += w[i][k] * win[k][i];
+            acc[i] = silu(a);
+        }
+        Pack8<T>::store(dst + (size_t)t * dst_stride, acc);
+        // streaming state: the last d_conv-1 input rows
+        if (state_out != nullptr && t >= s.L - (DCONV - 1))
+            Pack8<T>::store(state_out + ((size_t)b * (DCONV - 1) + (t - (s.L - (DCONV - 1)))) * C + c0, win[DCONV - 1]);
+#pragma unroll
+        for (int k = 0; k < DCONV - 1; ++k) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) win[k][i] = win[k + 1][i];
+        }
+    }
+    if (state_out != nullptr && s.L < DCONV - 1 && t0 == 0) {
+        // fewer new rows than the state holds: rows 0 .. d_conv-2-L of the new state are the old state's tail
+        for (int j = 0; j < (DCONV - 1) - s.L; ++j) {
+            float o[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = 0.f;
+            if (state_in != nullptr) {
+                const Pack8<T> v = Pack8<T>::load(state_in + ((size_t)b * (DCONV - 1) + j + s.L) * C + c0);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o[i] = v.get(i);
+            }
+            Pack8<T>::store(state_out + ((size_t)b * (DCONV - 1) + j) * C + c0, o);
+        }
+    }
+}
+
+// One wave per (b, t): out = rmsnorm(y * silu(z)) * weight over the H*P channels.
+template <typename T, typename TY>
+__global__ __launch_bounds__(256) void block_post_kernel(const TY *__restrict__ y, const T *__restrict__ zxbcdt,
+                                                         const float *__restrict__ norm_w, float eps,
+                                                         T *__restrict__ out, BlockShape s) {
+    const int DI = s.H * s.P, E = 2 * DI + 2 * s.G * s.N + s.H;
+    const int lane = threadIdx.x & 63;
+    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= (long long)s.B * s.L) return;
+    const TY *yr = y + (size_t)row * DI;
+    const T *zr = zxbcdt + (size_t)row * E;
+    constexpr int MAXP = 4;  // pieces of 8 channels per lane kept in registers: covers H*P <= 2048
+    float v[MAXP][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < MAXP; ++u) {
+        const int c0 = (u * 64 + lane) * 8;
+        if (c0 < DI) {
+            const Pack8<TY> yv = Pack8<TY>::load(yr + c0);
+            const Pack8<T> zv = Pack8<T>::load(zr + c0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                v[u][i] = yv.get(i) * silu(zv.get(i));
+                ss += v[u][i] * v[u][i];
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
+    const float scale = rsqrtf(ss / (float)DI + eps);
+#pragma unroll
+    for (int u = 0; u < MAXP; ++u) {
+        const int c0 = (u * 64 + lane) * 8;
+        if (c0 < DI) {
+            float o[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = v[u][i] * scale * norm_w[c0 + i];
+            Pack8<T>::store(out + (size_t)row * DI + c0, o);
+        }
+    }
+}
+
+bool block_supported(const BlockShape &s) {
+    return (s.d_conv >= 2 && s.d_conv <= 4) && (s.H * s.P) % 8 == 0 && (s.G * s.N) % 8 == 0 && s.H * s.P <= 2048;
+}
+
+template <typename T>
+static hipError_t pre_dispatch(const BlockShape &s, const void *zxbcdt, const float *conv_w, const float *conv_b,
+                               const float *dt_bias, const void *state_in, void *state_out, void *x, void *Bm,
+                               void *Cm, void *dt, hipStream_t st) {
+    const long long total = (long long)s.B * ((s.L + kPreSteps - 1) / kPreSteps) * ((s.H * s.P + 2 * s.G * s.N) / 8) +
+                            (long long)s.B * s.L * ((s.H + 7) / 8);
+    const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    const T *in = static_cast<const T *>(zxbcdt), *si = static_cast<const T *>(state_in);
+    T *so = static_cast<T *>(state_out), *xx = static_cast<T *>(x), *bb = static_cast<T *>(Bm), *cc = static_cast<T *>(Cm),
+      *dd = static_cast<T *>(dt);
+    switch (s.d_conv) {
+        case 2: block_pre_kernel<T, 2><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, xx, bb, cc, dd, s); break;
+        case 3: block_pre_kernel<T, 3><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, xx, bb, cc, dd, s); break;
+        case 4: block_pre_kernel<T, 4><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, xx, bb, cc, dd, s); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w,
+                            const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
+                            void *x, void *Bm, void *Cm, void *dt, hipStream_t st) {
+    return dtype ? pre_dispatch<__bf16>(s, zxbcdt, conv_w, conv_b, dt_bias, state_in, state_out, x, Bm, Cm, dt, st)
+                 : pre_dispatch<float>(s, zxbcdt, conv_w, conv_b, dt_bias, state_in, state_out, x, Bm, Cm, dt, st);
+}
+
+hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                             float eps, void *out, hipStream_t st) {
+    const long long rows = (long long)s.B * s.L;
+    const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    switch (dtype) {
+        case 0:
+            block_post_kernel<float, float><<<grid, block, 0, st>>>(static_cast<const float *>(y), static_cast<const float *>(zxbcdt),
+                                                                    norm_w, eps, static_cast<float *>(out), s);
+            break;
+        case 1:
+            block_post_kernel<__bf16, __bf16><<<grid, block, 0, st>>>(static_cast<const __bf16 *>(y), static_cast<const __bf16 *>(zxbcdt),
+                                                                      norm_w, eps, static_cast<__bf16 *>(out), s);
+            break;
+        default:  // bf16 activations with the scan's float32 y
+            block_post_kernel<__bf16, float><<<grid, block, 0, st>>>(static_cast<const float *>(y), static_cast<const __bf16 *>(zxbcdt),
+                                                                     norm_w, eps, static_cast<__bf16 *>(out), s);
+            break;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace ssd

@@ -15,6 +15,10 @@ struct StepShape {
     int B, H, P, N, G;
 };
 
+struct BlockShape {  // a Mamba-2 block around the scan: conv width d_conv over the x | B | C channels
+    int B, L, H, P, N, G, d_conv;
+};
+
 constexpr size_t kLdsLimitBytes = 160 * 1024;  // LDS per workgroup on gfx950
 
 // Dynamic LDS the stage-2 / stage-4 workgroup needs (elem_bytes = 2 for bf16, 4 for float).
@@ -56,5 +60,16 @@ bool steps_supported(const StepShape &s);
 hipError_t launch_steps(const StepShape &s, int nsteps, int dtype, float *state, const unsigned char *reset,
                         const void *x, const void *dt, const float *A, const void *Bm, const void *Cm,
                         const float *D, void *y, hipStream_t stream);
+
+// The memory-bound stages of a Mamba-2 block around the scan.  zxbcdt [B,L,E], E = 2*H*P + 2*G*N + H, laid out
+// per timestep as [ z | x | B | C | dt_raw ].  pre: conv1d + bias + SiLU over x|B|C into the scan's tensors and
+// dt = softplus(dt_raw + dt_bias); conv state [B, d_conv-1, H*P + 2*G*N] in the activation dtype (both optional).
+// post: out [B,L,H*P] = rmsnorm(y * silu(z)) * norm_w.  dtype 2 = bf16 activations with float32 y.
+bool block_supported(const BlockShape &s);
+hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w,
+                            const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
+                            void *x, void *Bm, void *Cm, void *dt, hipStream_t stream);
+hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                             float eps, void *out, hipStream_t stream);
 
 }  // namespace ssd

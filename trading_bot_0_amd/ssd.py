@@ -41,6 +41,8 @@ EXPORTED_SYMBOLS = (
     "ssd_chunk_scan_stage_fwd",
     "ssd_step_fwd",
     "ssd_steps_fwd",
+    "ssd_block_pre_fwd",
+    "ssd_block_post_fwd",
 )
 
 
@@ -99,7 +101,7 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
         lib.ssd_steps_fwd.argtypes = [POINTER(SsdStepDims), c_int64, c_int, P, P, P, P, P, P, P, P, P, P]
         for name in EXPORTED_SYMBOLS[2:]:
-            getattr(lib, name).restype = c_int
+            getattr(lib, name).restype = c_int   # (argument types of the block stages: block.py)
         _lib = lib
         return lib
 
