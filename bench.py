@@ -177,6 +177,28 @@ def main():
             tf = sf[name] / (ms * 1e-3) / 1e12
             stages[name]["dense_TFLOPs"] = round(tf, 1)
             stages[name]["mfma_frac"] = round(tf / MFMA_BF16_PEAK_TFLOPS, 4)
+    # stages 2 and 3 as kernels of their own (the whole-forward entry point fuses them for large batches):
+    # state passing alone is the pure-bandwidth recurrence over the chunk states
+    separate = {}
+    if len(stage_fns) == 3:
+        pair = [("chunk_state", k2), ("state_passing", k3)]
+        n_sep = max(10, args.steps // 5)
+        for _, fn in pair:
+            assert fn() == 0, ssd.last_error(lib)
+        se = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(n_sep)]
+        torch.cuda.synchronize()
+        for i in range(n_sep):
+            se[i][0].record()
+            k2()
+            se[i][1].record()
+            k3()
+            se[i][2].record()
+        torch.cuda.synchronize()
+        for j, (name, _) in enumerate(pair):
+            ms = sum(se[i][j].elapsed_time(se[i][j + 1]) for i in range(n_sep)) / n_sep
+            gbs = sb[name] / (ms * 1e-3) / 1e9
+            separate[name] = {"ms": round(ms, 5), "alg_bytes": sb[name], "GBps": round(gbs, 1),
+                              "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
     onepass = ssd.chunk_scan_is_onepass(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk,
                                         w.torch_dtype)
     if onepass:
@@ -215,6 +237,7 @@ def main():
         "forward_hbm_frac": round(algorithmic_bytes_fwd(w) / sec / 1e9 / HBM_PEAK_GBS, 4),
         "forward_path": "onepass" if onepass else "staged",
         "roofline": roofline, "stages": stages,
+        "stages_alone": separate,
         "stages_ms_sum": round(sum(s["ms"] for s in stages.values()), 5),
     }
     if onepass:

@@ -270,13 +270,21 @@ template <> __device__ inline void store_column<float>(float *yrow, float (&o)[1
 }
 
 // hi + lo bf16 pairs of two products a0*f0 and a1*f1 (f = 1 to split plain values): hi is the product
-// rounded to bf16, lo the rounded remainder, which the fused multiply-add gets from the exact product.
-// Four VALU instructions per element: multiply, half a pack, one shift or mask, fma, half a pack.
+// rounded to bf16, lo the rounded remainder m - hi, which is exact in float before its own rounding.
+// The remainder takes one v_dot2c_f32_bf16 per element, m + (-1)*half + 0*other half, which reads the half
+// straight out of the packed pair.  Three VALU instructions per element: multiply, half a pack, dot2c, half
+// a pack.  The selectors are kept out of the compiler's sight: it would encode the pair (-1, 0) as the
+// inline constant -1.0, which the instruction reads as the pair (0, -1).
 __device__ inline void split_pair(float a0, float f0, float a1, float f1, unsigned &hi, unsigned &lo) {
-    hi = pack_bf16x2(a0 * f0, a1 * f1);
-    asm("" : "+v"(hi));  // keep the packed pair as the source of both halves (else the low half is converted twice)
-    const float h0 = __uint_as_float(hi << 16), h1 = __uint_as_float(hi & 0xffff0000u);
-    lo = pack_bf16x2(__builtin_fmaf(a0, f0, -h0), __builtin_fmaf(a1, f1, -h1));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    unsigned first = 0x0000bf80u, second = 0xbf800000u;
+    asm("" : "+s"(first));
+    asm("" : "+s"(second));
+    const float m0 = a0 * f0, m1 = a1 * f1;
+    hi = pack_bf16x2(m0, m1);
+    const bf16x2 h = __builtin_bit_cast(bf16x2, hi);
+    lo = pack_bf16x2(__builtin_amdgcn_fdot2_f32_bf16(h, __builtin_bit_cast(bf16x2, first), m0, false),
+                     __builtin_amdgcn_fdot2_f32_bf16(h, __builtin_bit_cast(bf16x2, second), m1, false));
 }
 struct FragBits {  // an operand fragment as four packed pairs
     unsigned u[4];
