@@ -19,6 +19,8 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
                64 steps as one launch of the multi-step kernel
   reference_suite  the reference's historical benchmark cases for this path (batch 4, seq_len 4096,
                BFloat16), for the SSD op alone, in the reference's result schema
+  backward     the backward pass of the scan at the same shape: time per call, and its compulsory traffic
+               (x, dt, B, C, dy read; dx, ddt, dB, dC written) against the HBM peak
   mamba2_block the block around the scan at the policy shape (d_model = nheads*headdim): whole block, and the
                library's pre-scan and post-scan kernels alone with their GB/s
   cpu_baseline the plain-C oracle (sequential recurrence, float32, OpenMP) timed on this
@@ -58,6 +60,7 @@ def parse_args():
     ap.add_argument("--no-stream-step", action="store_true")
     ap.add_argument("--no-reference-suite", action="store_true")
     ap.add_argument("--no-block", action="store_true")
+    ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise kernel over 256 MiB in / 256 MiB out three times, the known-size "
@@ -243,6 +246,27 @@ def main():
     if onepass:
         out["onepass_scan"] = onepass_info
 
+    # ---- the backward pass at the benchmark shape ------------------------------------------------------
+    if not args.no_backward:
+        dyb = torch.randn_like(x)
+        wsb = torch.empty(ssd.backward_workspace_bytes(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk,
+                                                        w.torch_dtype), dtype=torch.uint8, device="cuda")
+
+        def bwd_call():
+            ssd.ssd_chunk_scan_backward(x, dt, A, Bm, Cm, D, dyb, chunk=w.chunk, initial_states=init, workspace=wsb)
+
+        for _ in range(3):
+            bwd_call()
+        t_bwd = wall_time_steps(bwd_call, 20, torch)
+        e = 2 if w.dtype == "bf16" else 4
+        BL = w.batch * w.seqlen
+        bwd_bytes = e * BL * (3 * w.nheads * w.headdim + 2 * w.nheads + 4 * w.ngroups * w.dstate)
+        out["backward"] = {"ms": round(t_bwd * 1e3, 4), "alg_bytes": bwd_bytes,
+                           "GBps": round(bwd_bytes / t_bwd / 1e9, 1),
+                           "hbm_frac": round(bwd_bytes / t_bwd / 1e9 / HBM_PEAK_GBS, 4),
+                           "workspace_bytes": wsb.numel(), "units_per_s": round(BL / t_bwd, 1)}
+        del dyb, wsb
+
     # ---- streaming step at batch 4096 ---------------------------------------------------------
     if not args.no_stream_step:
         sw = WORKLOADS["streamed_bf16"]
@@ -295,7 +319,8 @@ def main():
     # benchmark_results/bench_20260112_070055.json:5-41 lists mamba2_forward_train, mamba2_infer_prefill and
     # mamba2_infer_step at batch 4, seq_len 4096 (1 for the step), BFloat16, in the schema of
     # benchmarks/src/results.rs:8-29.  The same cases for the SSD op (the block around it is not part of this
-    # library; head sizes as in the policy shape), same schema; mamba2_fwd_bwd_train needs a backward pass.
+    # library; head sizes as in the policy shape), same schema; mamba2_fwd_bwd_train is the forward followed by
+    # the backward pass.
     if not args.no_reference_suite:
         rw = WORKLOADS["policy_bf16"].with_batch(4)
         ri = make_inputs(rw, seed=0, device="cuda", seqlen=4096)
@@ -314,7 +339,22 @@ def main():
             rstep()
         t_step = wall_time_steps(rstep, 500, torch) * 1e3
         cfg = {"batch": 4, "seq_len": 4096, "dtype": "BFloat16"}
-        out["reference_suite"] = [
+        suite_bwd = []
+        if not args.no_backward:
+            rdy = torch.randn_like(ri["x"])
+            rws = torch.empty(ssd.backward_workspace_bytes(4, 4096, rw.nheads, rw.headdim, rw.dstate, rw.ngroups, rw.chunk),
+                              dtype=torch.uint8, device="cuda")
+
+            def fwd_bwd():
+                rf()
+                ssd.ssd_chunk_scan_backward(ri["x"], ri["dt"], ri["A"], ri["B"], ri["C"], ri["D"], rdy, chunk=rw.chunk,
+                                            workspace=rws)
+
+            for _ in range(5):
+                fwd_bwd()
+            suite_bwd = [{"name": "mamba2_fwd_bwd_train", "time_ms": wall_time_steps(fwd_bwd, 50, torch) * 1e3, "config": cfg}]
+            del rdy, rws
+        out["reference_suite"] = suite_bwd + [
             {"name": "mamba2_forward_train", "time_ms": t_fwd, "config": cfg},
             {"name": "mamba2_infer_prefill", "time_ms": t_fwd, "config": cfg},
             {"name": "mamba2_infer_step", "time_ms": t_step, "config": {"batch": 4, "seq_len": 1, "dtype": "BFloat16"}},

@@ -1,0 +1,167 @@
+"""Backward pass of the scan through the C ABI against the float64 sequential adjoint
+(oracle/ssd_backward_oracle.py, itself pinned by central differences of the forward oracle).
+
+Parity rules, with tol = 1e-4 in float32 mode and 2e-2 in bf16 mode: max|out - ref| <= tol * rms(ref) for dx,
+ddt, dB, dC and dinitial_states; the gradients stored in bf16 (dx, ddt, dB, dC) are allowed, on top of that, the
+one rounding of the exact value that the output format itself costs (2^-8 |ref| per element), for the reason
+given in _util.py for the forward's bf16 y.  dA and dD are sums over batch and time of terms of both signs
+that largely cancel (with random dy, |dA| is some 1 % of the sum of the |terms|), so their error is measured on
+the scale such a sum's rounding lives on: |out - ref| <= tol * (rms(ref) + 2-norm of the summed terms)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ssd_backward_oracle as bwd
+from oracle import ssd_oracle as orc
+from trading_bot_0_amd import SsdError, ssd_chunk_scan, ssd_chunk_scan_backward
+from trading_bot_0_amd.synthetic import Workload, make_inputs
+
+from _util import TOL, np64, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def check(out, ref, dtype, what, terms_norm=0.0):
+    o = out.detach().float().cpu().numpy().astype(np.float64)
+    rms = np.sqrt((ref ** 2).mean())
+    allowed = TOL[dtype] * (rms + terms_norm)
+    if out.dtype == torch.bfloat16:
+        allowed = allowed + 2.0 ** -8 * np.abs(ref)
+    worst = (np.abs(o - ref) / allowed).max()
+    assert np.isfinite(worst) and worst <= 1.0, f"{what}: error is {worst:.3g} x the allowance (rms {rms:.3g})"
+
+
+def run_case(w, seed, with_D=True, with_init=True, with_dfinal=True, chunk=None):
+    cpu = make_inputs(w, seed=seed)
+    if not with_init:
+        cpu["init"] = None
+    dev = to_dev(cpu)
+    g = torch.Generator().manual_seed(seed + 100)
+    dy = torch.randn(cpu["x"].shape, generator=g).to(w.torch_dtype)
+    dfin = torch.randn(w.batch, w.nheads, w.headdim, w.dstate, generator=g) if with_dfinal else None
+    D = cpu["D"] if with_D else None
+    ref = bwd.ssd_backward_sequential(np64(cpu["x"]), np64(cpu["dt"]), np64(cpu["A"]), np64(cpu["B"]), np64(cpu["C"]),
+                                      np64(D), np64(cpu["init"]), np64(dy), np64(dfin))
+    Dd = dev["D"] if with_D else None
+    q = chunk or w.chunk
+    got = ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], Dd, dy.cuda(), chunk=q,
+                                  initial_states=dev["init"], dfinal_states=None if dfin is None else dfin.cuda(),
+                                  need_dinitial_states=True)
+    torch.cuda.synchronize()
+    for k_out, k_ref in (("dx", "dx"), ("ddt", "ddt"), ("dB", "dB"), ("dC", "dC"), ("dinitial_states", "dinit")):
+        check(got[k_out], ref[k_ref], w.torch_dtype, f"{w.name} {k_out}")
+    check(got["dA"], ref["dA"], w.torch_dtype, f"{w.name} dA", ref["dA_scale"])
+    if with_D:
+        check(got["dD"], ref["dD"], w.torch_dtype, f"{w.name} dD", ref["dD_scale"])
+    else:
+        assert got["dD"] is None
+    return got, ref
+
+
+SHAPES = [
+    Workload("bwd_policy_like", 2, 300, 8, 32, 64, 1, 128, init_std=0.5),
+    Workload("bwd_groups", 3, 77, 4, 16, 16, 2, 64, init_std=0.5),
+    Workload("bwd_per_head_bc", 2, 256, 4, 64, 32, 4, 32, init_std=0.5),
+    Workload("bwd_tiny_state", 2, 130, 2, 16, 64, 1, 64, init_std=0.5),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("w", SHAPES, ids=lambda w: w.name)
+def test_gradients_match_the_adjoint(w, dtype):
+    run_case(w.with_dtype(dtype), seed=21)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("with_D,with_init,with_dfinal", [(False, False, False), (True, False, True), (False, True, False)])
+def test_optional_operands(dtype, with_D, with_init, with_dfinal):
+    w = Workload("bwd_optional", 2, 200, 8, 32, 64, 1, 64, dtype=dtype, init_std=0.5)
+    run_case(w, seed=5, with_D=with_D, with_init=with_init, with_dfinal=with_dfinal)
+
+
+@pytest.mark.parametrize("chunk", [32, 64, 128, 256])
+def test_chunk_size_does_not_change_the_gradients(chunk):
+    w = Workload("bwd_chunks", 2, 300, 8, 32, 64, 1, 128, dtype="f32", init_std=0.5)
+    run_case(w, seed=8, chunk=chunk)
+
+
+def test_plumbing_workload_gradients():
+    from trading_bot_0_amd.synthetic import WORKLOADS
+    run_case(WORKLOADS["plumbing_f32"], seed=0, with_init=False)
+
+
+def test_strong_decay_and_heavy_tails():
+    w = Workload("bwd_decay_extreme", 2, 384, 8, 32, 64, 1, 128, dtype="f32", a_log_range=(0.01, 64.0),
+                 dt_law="mixture", x_law="student-t3")
+    run_case(w, seed=3, with_init=False)
+    run_case(w.with_dtype("bf16"), seed=3, with_init=False)
+
+
+def test_directional_derivative_of_the_gpu_forward():
+    """Independent of the oracle: the float32 GPU forward's change along a random direction equals the
+    gradient's projection on it (central difference, step chosen for float32)."""
+    w = Workload("bwd_fd", 2, 96, 4, 32, 64, 1, 32, dtype="f32", init_std=0.5)
+    cpu = make_inputs(w, seed=2)
+    dev = to_dev(cpu)
+    g = torch.Generator().manual_seed(9)
+    dy = torch.randn(cpu["x"].shape, generator=g).cuda()
+    got = ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], dy, chunk=w.chunk,
+                                  initial_states=dev["init"], need_dinitial_states=True)
+
+    def loss(**kw):
+        a = dict(x=dev["x"], dt=dev["dt"], A=dev["A"], B=dev["B"], C=dev["C"], D=dev["D"], init=dev["init"])
+        a.update(kw)
+        y, _ = ssd_chunk_scan(a["x"], a["dt"], a["A"], a["B"], a["C"], a["D"], chunk=w.chunk, initial_states=a["init"])
+        return (y.double() * dy.double()).sum().item()
+
+    for name, key, grad in (("x", "x", "dx"), ("B", "B", "dB"), ("C", "C", "dC"), ("dt", "dt", "ddt"), ("init", "init", "dinitial_states")):
+        v = torch.randn(dev[key].shape, generator=g).cuda()
+        if name == "dt":
+            v = v * dev["dt"] * 0.5          # keep dt positive
+        eps = 1e-2
+        num = (loss(**{key: dev[key] + eps * v}) - loss(**{key: dev[key] - eps * v})) / (2 * eps)
+        ana = (got[grad].double() * v.double()).sum().item()
+        assert abs(num - ana) <= 2e-3 * max(1.0, abs(ana)), (name, num, ana)
+
+
+def test_unsupported_shapes_are_refused():
+    w = Workload("bwd_big_state", 1, 64, 2, 32, 128, 1, 64, dtype="bf16")
+    dev = to_dev(make_inputs(w, seed=0))
+    with pytest.raises(SsdError) as e:
+        ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], torch.zeros_like(dev["x"]), chunk=64)
+    assert "dstate <= 64" in str(e.value)
+    w = Workload("bwd_ok", 1, 64, 2, 32, 64, 1, 64, dtype="bf16")
+    dev = to_dev(make_inputs(w, seed=0))
+    with pytest.raises(ValueError):
+        ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], torch.zeros_like(dev["x"]), chunk=64,
+                                dfinal_states=torch.zeros(1, 2, 32, 32, device="cuda"))
+
+
+def test_full_size_policy_shape_against_batch_rows():
+    """The benchmark shape (B=256, L=2048, bf16): the gradients of two batch rows against the oracle, and the
+    per-head sums (dA, dD) against the same sums taken from a float64 run of those rows scaled up is not
+    possible, so they are checked for the additivity the sum has: the full batch equals the two halves added."""
+    from trading_bot_0_amd.synthetic import WORKLOADS
+    w = WORKLOADS["policy_bf16"]
+    dev = make_inputs(w, seed=0, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(4)
+    dy = torch.randn(dev["x"].shape, generator=g, device="cuda").to(torch.bfloat16)
+    full = ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], dy, chunk=w.chunk,
+                                   need_dinitial_states=True)
+    rows = [0, w.batch - 1]
+    sub = lambda t: t[rows].contiguous()
+    ref = bwd.ssd_backward_sequential(np64(sub(dev["x"])), np64(sub(dev["dt"])), np64(dev["A"]), np64(sub(dev["B"])),
+                                      np64(sub(dev["C"])), np64(dev["D"]), None, np64(sub(dy)), None)
+    for k_out, k_ref in (("dx", "dx"), ("ddt", "ddt"), ("dB", "dB"), ("dC", "dC"), ("dinitial_states", "dinit")):
+        check(full[k_out][rows], ref[k_ref], torch.bfloat16, f"policy {k_out}")
+    half = w.batch // 2
+    parts = []
+    for sl in (slice(0, half), slice(half, w.batch)):
+        c = lambda t: t[sl].contiguous()
+        parts.append(ssd_chunk_scan_backward(c(dev["x"]), c(dev["dt"]), dev["A"], c(dev["B"]), c(dev["C"]), dev["D"], c(dy),
+                                             chunk=w.chunk))
+    for k in ("dA", "dD"):
+        both = parts[0][k].double() + parts[1][k].double()
+        scale = full[k].double().abs().max().item()
+        assert (full[k].double() - both).abs().max().item() <= 1e-5 * scale, k
+    assert torch.equal(full["dx"][:half], parts[0]["dx"]) and torch.equal(full["dB"][half:], parts[1]["dB"])

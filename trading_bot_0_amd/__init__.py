@@ -9,6 +9,7 @@ from .ssd import (  # noqa: F401
     chunk_state_passing,
     load_library,
     ssd_chunk_scan,
+    ssd_chunk_scan_backward,
     ssd_chunk_scan_onepass,
     ssd_step,
     ssd_steps,

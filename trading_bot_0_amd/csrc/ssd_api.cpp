@@ -119,6 +119,91 @@ int hip_fail(hipError_t e, const char *what) {
     return fail(SSD_ERR_RUNTIME, "ssd: %s failed: %s", what, hipGetErrorString(e));
 }
 
+// Stages 1-4 one after the other.  mode as for launch_chunk_cumsum (0 = the forward's decays and weights).
+int run_staged(const ssd::ScanShape &s, int dtype, const void *x, const void *dt, const float *A, const void *Bm,
+               const void *Cm, const float *D, const float *initial_states, const uint8_t *reset, int mode, void *y,
+               float *final_states, float *dtcs, float *states, hipStream_t st, int dt_len = 0) {
+    hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, reset, dtcs, st, mode, dt_len);
+    if (e != hipSuccess) return hip_fail(e, "chunk_cumsum launch");
+    if ((int64_t)s.B * s.H >= kFusedStatePassingMinSequences) {
+        // enough (b,h) sequences to fill the chip: stages 2 and 3 in one pass, states carried on chip
+        e = ssd::launch_chunk_state_scan(s, dtype, x, Bm, dtcs, initial_states, states, final_states, st);
+        if (e != hipSuccess) return hip_fail(e, "chunk_state_passing launch");
+    } else {
+        e = ssd::launch_chunk_state(s, dtype, x, Bm, dtcs, states, st);
+        if (e != hipSuccess) return hip_fail(e, "chunk_state launch");
+        e = ssd::launch_state_passing(s, states, dtcs, initial_states, states, final_states, st);  // in place
+        if (e != hipSuccess) return hip_fail(e, "state_passing launch");
+    }
+    e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dtcs, states, D, y, st);
+    if (e != hipSuccess) return hip_fail(e, "chunk_scan launch");
+    return SSD_OK;
+}
+
+// Workspace of the backward pass: the scan workspace (its three scans have the same number of chunks, heads and
+// state elements; the two transposed scans keep their chunk states for the anchors, so there is a second state
+// array), the gathered operands (reversed ones padded to whole chunks) and the scans' float outputs.
+struct BwdWorkspace {
+    size_t scan_off, states2, dy_rev, x_rev, c_rev_g, b_rev_g, c_rev_h, b_fwd_h, r_rev, yb_rev, yc, gfin, gfin_t, ffin_t,
+        init_t, dfin_t, e1, dd, u, anchor, da_part, total;
+};
+
+BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
+    BwdWorkspace w;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = off;
+        off += align_up(bytes, 256);
+        return at;
+    };
+    const size_t BL = (size_t)s.B * s.L, BLp = (size_t)s.B * s.nc * s.Q;  // true and padded rows
+    const size_t HP = (size_t)s.H * s.P, HN = (size_t)s.H * s.N, GN = (size_t)s.G * s.N;
+    const size_t st = (size_t)s.B * s.H * s.P * s.N * sizeof(float);
+    w.scan_off = take(carve(s).total);
+    w.states2 = take((size_t)s.nc * st);
+    w.dy_rev = take(BLp * HP * elem_bytes);
+    w.x_rev = take(BLp * HP * elem_bytes);
+    w.c_rev_g = take(BLp * GN * elem_bytes);
+    w.b_rev_g = take(BLp * GN * elem_bytes);
+    w.c_rev_h = take(BLp * HN * elem_bytes);
+    w.b_fwd_h = take(BL * HN * elem_bytes);
+    w.r_rev = take(BLp * HP * sizeof(float));
+    w.yb_rev = take(BLp * HN * sizeof(float));
+    w.yc = take(BL * HN * sizeof(float));
+    w.gfin = take(st);
+    w.gfin_t = take(st);
+    w.ffin_t = take(st);
+    w.init_t = take(st);
+    w.dfin_t = take(st);
+    w.e1 = take(BL * s.H * sizeof(float));
+    w.dd = take(BL * s.H * sizeof(float));
+    w.u = take(BL * s.H * sizeof(float));
+    w.anchor = take((size_t)s.B * (s.nc + 1) * s.H * sizeof(double));
+    w.da_part = take((size_t)s.B * s.H * sizeof(double));
+    w.total = off;
+    return w;
+}
+
+constexpr int64_t kBackwardChunk = 64;
+
+// The backward pass runs the forward's stage kernels on the transposed state ([N,P] per head, B and C per head),
+// so the transposed shape must be one they take as well.
+int make_bwd_shapes(const ssd_dims *dims, int dtype, ssd::ScanShape *s, ssd::ScanShape *sT) {
+    if (dtype != SSD_DTYPE_F32 && dtype != SSD_DTYPE_BF16)
+        return fail(SSD_ERR_INVALID, "ssd: the backward pass takes dtype 0 (float32) or 1 (bfloat16), got %d", dtype);
+    // The pass tiles time by at most kBackwardChunk steps whatever chunk the caller names (it owns its workspace
+    // layout): the decay gradient sums rounding errors over a chunk, see ssd_backward_kernels.hip.
+    ssd_dims own = *dims;
+    if (own.chunk > kBackwardChunk) own.chunk = kBackwardChunk;
+    if (int rc = make_shape(&own, dtype, s)) return rc;
+    if (dims->dstate > 64 || dims->headdim < 16 || (dims->headdim & (dims->headdim - 1)) != 0)
+        return fail(SSD_ERR_UNSUPPORTED,
+                    "ssd: the backward pass needs dstate <= 64 and headdim 16, 32 or 64, got %lld and %lld",
+                    (long long)dims->dstate, (long long)dims->headdim);
+    const ssd_dims t = {dims->batch, dims->seqlen, dims->nheads, dims->dstate, dims->headdim, dims->nheads, own.chunk};
+    return make_shape(&t, dtype, sT);
+}
+
 }  // namespace
 
 extern "C" {
@@ -246,20 +331,112 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
         e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states, st);
         return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
     }
-    e = ssd::launch_chunk_cumsum(s, dtype, dt, A, reset, dtcs, st);
-    if (e != hipSuccess) return hip_fail(e, "chunk_cumsum launch");
-    if ((int64_t)s.B * s.H >= kFusedStatePassingMinSequences) {
-        // enough (b,h) sequences to fill the chip: stages 2 and 3 in one pass, states carried on chip
-        e = ssd::launch_chunk_state_scan(s, dtype, x, Bm, dtcs, initial_states, states, final_states, st);
-        if (e != hipSuccess) return hip_fail(e, "chunk_state_passing launch");
-    } else {
-        e = ssd::launch_chunk_state(s, dtype, x, Bm, dtcs, states, st);
-        if (e != hipSuccess) return hip_fail(e, "chunk_state launch");
-        e = ssd::launch_state_passing(s, states, dtcs, initial_states, states, final_states, st);  // in place
-        if (e != hipSuccess) return hip_fail(e, "state_passing launch");
+    return run_staged(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, 0, y, final_states, dtcs, states, st);
+}
+
+int ssd_chunk_scan_bwd_workspace_bytes(const ssd_dims *dims, int dtype, size_t *out_bytes) {
+    if (out_bytes == nullptr) return fail(SSD_ERR_INVALID, "ssd: out_bytes must not be NULL");
+    ssd::ScanShape s, sT;
+    if (int rc = make_bwd_shapes(dims, dtype, &s, &sT)) return rc;
+    *out_bytes = carve_bwd(s, dtype == SSD_DTYPE_F32 ? 4 : 2).total;
+    return SSD_OK;
+}
+
+int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A, const void *Bm,
+                       const void *Cm, const float *D, const float *initial_states, const void *dy,
+                       const float *dfinal_states, void *dx, void *ddt, float *dA, void *dB, void *dC, float *dD,
+                       float *dinitial_states, void *workspace, size_t workspace_bytes, void *hip_stream) {
+    ssd::ScanShape s, sT;
+    if (int rc = make_bwd_shapes(dims, dtype, &s, &sT)) return rc;
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(dt);
+    REQUIRE_PTR(A);
+    REQUIRE_PTR(Bm);
+    REQUIRE_PTR(Cm);
+    REQUIRE_PTR(dy);
+    REQUIRE_PTR(dx);
+    REQUIRE_PTR(ddt);
+    REQUIRE_PTR(dA);
+    REQUIRE_PTR(dB);
+    REQUIRE_PTR(dC);
+    REQUIRE_PTR(workspace);
+    OPTIONAL_PTR(D);
+    OPTIONAL_PTR(initial_states);
+    OPTIONAL_PTR(dfinal_states);
+    OPTIONAL_PTR(dD);
+    OPTIONAL_PTR(dinitial_states);
+    if (dD != nullptr && D == nullptr) return fail(SSD_ERR_INVALID, "ssd: dD asked for without D");
+    const int eb = dtype == SSD_DTYPE_F32 ? 4 : 2;
+    const BwdWorkspace w = carve_bwd(s, eb);
+    if (workspace_bytes < w.total)
+        return fail(SSD_ERR_WORKSPACE, "ssd: backward workspace has %zu bytes, %zu needed", workspace_bytes, w.total);
+    char *base = static_cast<char *>(workspace);
+    auto at = [&](size_t off) { return static_cast<void *>(base + off); };
+    auto atf = [&](size_t off) { return reinterpret_cast<float *>(base + off); };
+    const Workspace sw = carve(s);
+    float *dtcs = atf(w.scan_off + sw.dtcs_off), *states = atf(w.scan_off + sw.st_off);
+    hipStream_t st = (hipStream_t)hip_stream;
+    const int inner = dtype == SSD_DTYPE_F32 ? SSD_DTYPE_F32 : SSD_DTYPE_BF16_Y32;  // the scans write float y
+    const int el = dtype == SSD_DTYPE_F32 ? 0 : 1;
+    const int rep = s.H / s.G;
+    hipError_t e;
+#define BWD_LAUNCH(call, what)                      \
+    do {                                            \
+        e = (call);                                 \
+        if (e != hipSuccess) return hip_fail(e, what); \
+    } while (0)
+    // The reversed sequences are padded in front to whole chunks (Lp rows), so that chunk k of a reversed scan
+    // begins where chunk nc - k of the forward ends.
+    const int Lp = s.nc * s.Q;
+    ssd::ScanShape sR = s, sTR = sT;
+    sR.L = Lp;
+    sTR.L = Lp;
+    float *states2 = atf(w.states2);
+    // operands: time-reversed dy, x, C, B; C (reversed) and B (forward) once per head for the transposed scans
+    BWD_LAUNCH(ssd::launch_gather_rows(el, dy, at(w.dy_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather dy");
+    BWD_LAUNCH(ssd::launch_gather_rows(el, x, at(w.x_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather x");
+    BWD_LAUNCH(ssd::launch_gather_rows(el, Cm, at(w.c_rev_g), s.B, s.L, Lp, s.G, s.N, 1, true, st), "gather C");
+    BWD_LAUNCH(ssd::launch_gather_rows(el, Bm, at(w.b_rev_g), s.B, s.L, Lp, s.G, s.N, 1, true, st), "gather B");
+    BWD_LAUNCH(ssd::launch_gather_rows(el, Cm, at(w.c_rev_h), s.B, s.L, Lp, s.G, s.N, rep, true, st), "gather C per head");
+    const void *b_heads = Bm;
+    if (rep > 1) {
+        BWD_LAUNCH(ssd::launch_gather_rows(el, Bm, at(w.b_fwd_h), s.B, s.L, s.L, s.G, s.N, rep, false, st),
+                   "gather B per head");
+        b_heads = at(w.b_fwd_h);
     }
-    e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dtcs, states, D, y, st);
-    if (e != hipSuccess) return hip_fail(e, "chunk_scan launch");
+    const float *init_t = nullptr, *dfin_t = nullptr;
+    if (initial_states != nullptr) {
+        BWD_LAUNCH(ssd::launch_transpose_state(initial_states, atf(w.init_t), (long long)s.B * s.H, s.P, s.N, st), "transpose");
+        init_t = atf(w.init_t);
+    }
+    if (dfinal_states != nullptr) {
+        BWD_LAUNCH(ssd::launch_transpose_state(dfinal_states, atf(w.dfin_t), (long long)s.B * s.H, s.P, s.N, st), "transpose");
+        dfin_t = atf(w.dfin_t);
+    }
+    // r = g B: the adjoint recurrence, reversed in time; its last state is g_0
+    if (int rc = run_staged(sR, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states, nullptr, 1,
+                            at(w.r_rev), atf(w.gfin), dtcs, states, st, s.L))
+        return rc;
+    // yB = x . g: the same recurrence with the state transposed; its chunk states stay in `states`
+    if (int rc = run_staged(sTR, inner, at(w.c_rev_h), dt, A, at(w.dy_rev), at(w.x_rev), nullptr, dfin_t, nullptr, 1,
+                            at(w.yb_rev), atf(w.gfin_t), dtcs, states, st, s.L))
+        return rc;
+    // yC = dy . h: the forward recurrence with the state transposed; its chunk states go to `states2`
+    if (int rc = run_staged(sT, inner, b_heads, dt, A, x, dy, nullptr, init_t, nullptr, 0, at(w.yc), atf(w.ffin_t), dtcs,
+                            states2, st))
+        return rc;
+    BWD_LAUNCH(ssd::launch_bwd_rows(s, Lp, el, x, dy, dt, Cm, D, atf(w.r_rev), atf(w.yc), dx, atf(w.e1), atf(w.dd), atf(w.u), st),
+               "backward rows");
+    BWD_LAUNCH(ssd::launch_bwd_group_sums(s, Lp, el, dt, atf(w.yb_rev), atf(w.yc), dB, dC, st), "backward group sums");
+    double *anchor = reinterpret_cast<double *>(base + w.anchor);
+    BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, anchor, st),
+               "backward anchors");
+    double *da_part = reinterpret_cast<double *>(base + w.da_part);
+    BWD_LAUNCH(ssd::launch_bwd_ddt(s, el, dt, A, atf(w.e1), atf(w.u), anchor, ddt, da_part, st), "backward ddt");
+    BWD_LAUNCH(ssd::launch_bwd_head_sums(s, da_part, atf(w.dd), dA, dD, st), "backward head sums");
+    if (dinitial_states != nullptr)
+        BWD_LAUNCH(ssd::launch_bwd_dinit(s, el, dt, A, atf(w.gfin), dinitial_states, st), "backward dinit");
+#undef BWD_LAUNCH
     return SSD_OK;
 }
 

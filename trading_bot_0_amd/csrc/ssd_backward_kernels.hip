@@ -1,0 +1,397 @@
+// Backward pass of the SSD scan: the memory-bound kernels around three role-swapped runs of the forward.
+//
+// With g_t = dLoss/dh_t, the adjoint recurrence g_t = dy_t (x) C_t + a_{t+1} g_{t+1} is the forward recurrence
+// run backwards in time with (x, B, C) <- (dy, C, B), unit input weights and the decays shifted by one step.
+// The three heavy products of the backward pass are readouts of such recurrences:
+//   r_t  = g_t B_t                (x <- dy, B <- C, C <- B; reversed time)            dx  = D dy + dt r
+//   yB_t = x_t . g_t              (transposed state: x <- C, B <- dy, C <- x; reversed) dB = sum_heads dt yB
+//   yC_t = dy_t . h_t             (transposed state: x <- B, B <- x, C <- dy; forward)  dC = sum_heads yC
+// and run on the forward's own stage kernels.  What is left is here: gathering the operands (time reversal,
+// one copy of a group's B or C per head), the per-timestep products, the sums over the heads of a group, and
+//   ddt_t = x_t . r_t + A q_t,   q_t = a_t <g_t, h_{t-1}>,   dA = sum dt q,   dD = sum dy . x,   dinit = a_0 g_0.
+// q obeys q_t = u_t + q_{t+1} with u_t = C_t . yC_t - dt_t x_t . r_t (because a_t <g_t, h_{t-1}> =
+// <g_t, h_t> - dt_t <g_t, x_t (x) B_t> and <g_t, h_t> = dy_t . (h_t C_t) + a_{t+1} <g_{t+1}, h_t>), but the u
+// are each of the size of q and only their sum telescopes, so summing them over a whole sequence would add up
+// their rounding errors (q is small against u where the decay is strong).  q is therefore anchored at the first
+// step of every chunk, where it is the inner product of the two transposed scans' chunk states (forward state
+// entering the chunk, adjoint state entering it), and at the end of the sequence (<dfinal, final>); the u are
+// summed inside a chunk only, and the pass uses chunks of at most 64 steps.  For the two sets of chunk states to
+// meet at the same timesteps the reversed sequences are padded in front with no-op steps to whole chunks.
+#include "ssd_device.h"
+#include "ssd_launch.h"
+
+namespace ssd {
+
+namespace {
+
+template <typename T> struct Row8;  // eight consecutive elements as floats
+template <> struct Row8<__bf16> {
+    float v[8];
+    static __device__ inline Row8 load(const __bf16 *p) {
+        const bf16x8 q = *reinterpret_cast<const bf16x8 *>(p);
+        Row8 r;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r.v[i] = (float)q[i];
+        return r;
+    }
+    __device__ inline void store(__bf16 *p) const {
+        bf16x8 q;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = (__bf16)v[i];
+        *reinterpret_cast<bf16x8 *>(p) = q;
+    }
+};
+template <> struct Row8<float> {
+    float v[8];
+    static __device__ inline Row8 load(const float *p) {
+        const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + 4);
+        Row8 r;
+        r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w;
+        r.v[4] = b.x; r.v[5] = b.y; r.v[6] = b.z; r.v[7] = b.w;
+        return r;
+    }
+    __device__ inline void store(float *p) const {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+};
+
+// dst[b, t', (g*rep + k)*W + w] = src[b, t, g*W + w] for k < rep, with t = Ldst-1-t' if reverse else t';
+// zero where t >= Lsrc.  One thread per 8 elements of dst (W is a multiple of 8), moved as raw bits.
+template <typename T>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const T *__restrict__ src, T *__restrict__ dst, int Lsrc,
+                                                          int L, int groups, int W, int rep, int reverse,
+                                                          long long total) {
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const int w8 = W / 8, per_row = groups * rep * w8;
+    const int j = (int)(gid % per_row);
+    const long long bt = gid / per_row;
+    const int tp = (int)(bt % L);
+    const long long b = bt / L;
+    const int w = (j % w8) * 8, g = (j / w8) / rep;
+    const int t = reverse ? L - 1 - tp : tp;
+    typedef __attribute__((ext_vector_type(sizeof(T) * 2))) unsigned piece;  // 8 elements
+    piece v = {};
+    if (t < Lsrc) v = *reinterpret_cast<const piece *>(src + ((size_t)(b * Lsrc + t) * groups + g) * W + w);
+    *reinterpret_cast<piece *>(dst + (size_t)bt * groups * rep * W + (size_t)j * 8) = v;
+}
+
+// [.., P, N] -> [.., N, P] for every (b,h): the state of the transposed recurrences
+__global__ __launch_bounds__(256) void transpose_state_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                              int P, int N, long long total) {
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const int pn = P * N;
+    const long long bh = gid / pn;
+    const int i = (int)(gid % pn), n = i / P, p = i % P;  // dst index (n, p)
+    dst[gid] = src[bh * pn + (size_t)p * N + n];
+}
+
+// One thread per (b, t, h): dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1.
+// r_rev is the reversed scan's float output (time reversed), yC the forward-time transposed scan's.
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                                                       const T *__restrict__ dt, const T *__restrict__ Cm,
+                                                       const float *__restrict__ D, const float *__restrict__ r_rev,
+                                                       const float *__restrict__ yC, T *__restrict__ dx,
+                                                       float *__restrict__ e1, float *__restrict__ dd,
+                                                       float *__restrict__ u, ScanShape s, int Lrev, long long total) {
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const int h = (int)(gid % s.H);
+    const long long bt = gid / s.H;
+    const int t = (int)(bt % s.L);
+    const long long b = bt / s.L;
+    const int g = h / (s.H / s.G);
+    const float dtv = (float)dt[gid], dh = D ? D[h] : 0.f;
+    const size_t row = (size_t)gid * s.P, rrow = ((size_t)(b * Lrev + (Lrev - 1 - t)) * s.H + h) * s.P;
+    float se1 = 0.f, sdd = 0.f;
+    for (int p = 0; p < s.P; p += 8) {
+        const Row8<T> xv = Row8<T>::load(x + row + p), dv = Row8<T>::load(dy + row + p);
+        const Row8<float> rv = Row8<float>::load(r_rev + rrow + p);
+        Row8<T> o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            o.v[i] = dh * dv.v[i] + dtv * rv.v[i];
+            se1 += xv.v[i] * rv.v[i];
+            sdd += dv.v[i] * xv.v[i];
+        }
+        o.store(dx + row + p);
+    }
+    float sc = 0.f;
+    const T *crow = Cm + ((size_t)bt * s.G + g) * s.N;
+    const float *yrow = yC + (size_t)gid * s.N;
+    for (int n = 0; n < s.N; n += 8) {
+        const Row8<T> cv = Row8<T>::load(crow + n);
+        const Row8<float> yv = Row8<float>::load(yrow + n);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sc += cv.v[i] * yv.v[i];
+    }
+    e1[gid] = se1;
+    dd[gid] = sdd;
+    u[gid] = sc - dtv * se1;
+}
+
+// One thread per (b, t, g, 8 state columns): dB = sum over the group's heads of dt yB, dC = the same of yC.
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_group_sums_kernel(const T *__restrict__ dt, const float *__restrict__ yB_rev,
+                                                             const float *__restrict__ yC, T *__restrict__ dB,
+                                                             T *__restrict__ dC, ScanShape s, int Lrev, long long total) {
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const int n8 = s.N / 8, hpg = s.H / s.G;
+    const int n = (int)(gid % n8) * 8;
+    const long long btg = gid / n8;
+    const int g = (int)(btg % s.G);
+    const long long bt = btg / s.G;
+    const int t = (int)(bt % s.L);
+    const long long b = bt / s.L;
+    Row8<T> ob, oc;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ob.v[i] = oc.v[i] = 0.f;
+    for (int k = 0; k < hpg; ++k) {
+        const int h = g * hpg + k;
+        const float dtv = (float)dt[(size_t)bt * s.H + h];
+        const Row8<float> vb = Row8<float>::load(yB_rev + ((size_t)(b * Lrev + (Lrev - 1 - t)) * s.H + h) * s.N + n);
+        const Row8<float> vc = Row8<float>::load(yC + ((size_t)bt * s.H + h) * s.N + n);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            ob.v[i] += dtv * vb.v[i];
+            oc.v[i] += vc.v[i];
+        }
+    }
+    ob.store(dB + (size_t)btg * s.N + n);
+    oc.store(dC + (size_t)btg * s.N + n);
+}
+
+// One wave per (b, c, h), c = 0 .. nc: anchor[b,c,h] = q at the first step of chunk c = exp(dt A) <adjoint state
+// entering chunk c, forward state entering chunk c>, dt the first step's of the chunk.  The reversed scan's chunk
+// nc - c begins where forward chunk c does; for c = 0 that is past its last chunk, i.e. its final state, and the
+// forward state is the initial one.  c = nc is the end of the sequence: q_L = <dfinal, final> (no decay).
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_anchor_kernel(const T *__restrict__ dt, const float *__restrict__ A,
+                                                         const float *__restrict__ fwd_prev, const float *__restrict__ rev_prev,
+                                                         const float *__restrict__ rev_final, const float *__restrict__ init_t,
+                                                         const float *__restrict__ fwd_final, const float *__restrict__ dfin_t,
+                                                         double *__restrict__ anchor, ScanShape s) {
+    const int lane = threadIdx.x & 63;
+    const long long id = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (id >= (long long)s.B * (s.nc + 1) * s.H) return;
+    const int h = (int)(id % s.H);
+    const int c = (int)((id / s.H) % (s.nc + 1));
+    const long long b = id / ((long long)s.H * (s.nc + 1));
+    const int pn = s.P * s.N;
+    const size_t bh = ((size_t)b * s.H + h) * pn;
+    const float *f, *g;
+    if (c == 0) {
+        f = init_t ? init_t + bh : nullptr;
+        g = rev_final + bh;
+    } else if (c == s.nc) {
+        f = dfin_t ? fwd_final + bh : nullptr;
+        g = dfin_t ? dfin_t + bh : nullptr;
+    } else {
+        f = fwd_prev + (((size_t)b * s.nc + c) * s.H + h) * pn;
+        g = rev_prev + (((size_t)b * s.nc + (s.nc - c)) * s.H + h) * pn;
+    }
+    double part = 0.0;
+    if (f != nullptr)
+        for (int i = lane * 4; i < pn; i += 256) {
+            const float4 fv = *reinterpret_cast<const float4 *>(f + i), gv = *reinterpret_cast<const float4 *>(g + i);
+            part += (double)fv.x * gv.x + (double)fv.y * gv.y + (double)fv.z * gv.z + (double)fv.w * gv.w;
+        }
+    const double incl = wave_inclusive_scan(part);
+    if (lane == 63) {
+        const double a = c == s.nc ? 1.0 : exp((double)(float)dt[((size_t)b * s.L + (size_t)c * s.Q) * s.H + h] * (double)A[h]);
+        anchor[id] = a * incl;
+    }
+}
+
+// One wave per (b, h), one pass of the wave per chunk (chunks of at most 64 steps).  q is known at both ends of a
+// chunk (the anchors) and obeys q_t - q_{t+1} = u_t in between; the computed u do not sum exactly to the
+// difference of the anchors, and the mismatch is spread evenly over the chunk's steps:
+// q_t = anchor_c - sum_{v < t in the chunk} u_v - mismatch * (steps before t) / (steps of the chunk).
+// ddt_t = e1_t + A q_t and this sequence's part of dA = sum dt_t q_t.  Sums in float64.
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, const float *__restrict__ A,
+                                                      const float *__restrict__ e1, const float *__restrict__ u,
+                                                      const double *__restrict__ anchor, T *__restrict__ ddt,
+                                                      double *__restrict__ dA_part, ScanShape s) {
+    const int lane = threadIdx.x & 63;
+    const long long bh = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (bh >= (long long)s.B * s.H) return;
+    const int h = (int)(bh % s.H);
+    const long long b = bh / s.H;
+    auto last_lane = [](double v) {
+        return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), 63),
+                                __builtin_amdgcn_readlane(__double2loint(v), 63));
+    };
+    const double a = (double)A[h];
+    double da = 0.0;
+    for (int c = 0; c < s.nc; ++c) {
+        const double q0 = anchor[((size_t)b * (s.nc + 1) + c) * s.H + h];
+        const double q1 = anchor[((size_t)b * (s.nc + 1) + c + 1) * s.H + h];
+        const int t0 = c * s.Q, len = min(s.Q, s.L - t0);
+        const bool ok = lane < len;
+        const size_t at = ((size_t)b * s.L + t0 + (ok ? lane : 0)) * s.H + h;
+        const double uv = ok ? (double)u[at] : 0.0;
+        const double incl = wave_inclusive_scan(uv);
+        const double mismatch = q0 - last_lane(incl) - q1;
+        if (ok) {
+            const double q = q0 - (incl - uv) - mismatch * (double)lane / (double)len;
+            ddt[at] = (T)(float)((double)e1[at] + a * q);
+            da += (double)(float)dt[at] * q;
+        }
+    }
+    const double tot = last_lane(wave_inclusive_scan(da));
+    if (lane == 0) dA_part[bh] = tot;
+}
+
+// One workgroup per head: dA[h] = sum_b dA_part[b,h]; dD[h] = sum_{b,t} dd[b,t,h] (float64 sums).
+__global__ __launch_bounds__(256) void bwd_head_sums_kernel(const double *__restrict__ dA_part, const float *__restrict__ dd,
+                                                            float *__restrict__ dA, float *__restrict__ dD, ScanShape s) {
+    __shared__ double red[2][256];
+    const int h = blockIdx.x;
+    double sa = 0.0, sd = 0.0;
+    for (long long i = threadIdx.x; i < s.B; i += blockDim.x) sa += dA_part[i * s.H + h];
+    if (dD != nullptr)
+        for (long long i = threadIdx.x; i < (long long)s.B * s.L; i += blockDim.x) sd += (double)dd[i * s.H + h];
+    red[0][threadIdx.x] = sa;
+    red[1][threadIdx.x] = sd;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) {
+            red[0][threadIdx.x] += red[0][threadIdx.x + w];
+            red[1][threadIdx.x] += red[1][threadIdx.x + w];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        dA[h] = (float)red[0][0];
+        if (dD != nullptr) dD[h] = (float)red[1][0];
+    }
+}
+
+// dinit = exp(dt_0 A) g_0, g_0 = the reversed scan's final state
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_dinit_kernel(const T *__restrict__ dt, const float *__restrict__ A,
+                                                        const float *__restrict__ gfin, float *__restrict__ dinit,
+                                                        ScanShape s, long long total) {
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const long long bh = gid / (s.P * s.N);
+    const int h = (int)(bh % s.H);
+    const long long b = bh / s.H;
+    const float a0 = __expf((float)dt[(size_t)b * s.L * s.H + h] * A[h]);
+    dinit[gid] = a0 * gfin[gid];
+}
+
+inline unsigned blocks_for(long long total) { return (unsigned)((total + 255) / 256); }
+
+template <typename T>
+hipError_t gather_t(const void *src, void *dst, int B, int Lsrc, int L, int groups, int W, int rep, bool reverse,
+                    hipStream_t st) {
+    const long long total = (long long)B * L * groups * rep * (W / 8);
+    gather_rows_kernel<T><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(static_cast<const T *>(src), static_cast<T *>(dst), Lsrc,
+                                                                         L, groups, W, rep, reverse ? 1 : 0, total);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t rows_t(const ScanShape &s, int Lrev, const void *x, const void *dy, const void *dt, const void *Cm, const float *D,
+                  const float *r_rev, const float *yC, void *dx, float *e1, float *dd, float *u, hipStream_t st) {
+    const long long total = (long long)s.B * s.L * s.H;
+    bwd_rows_kernel<T><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(
+        static_cast<const T *>(x), static_cast<const T *>(dy), static_cast<const T *>(dt), static_cast<const T *>(Cm), D,
+        r_rev, yC, static_cast<T *>(dx), e1, dd, u, s, Lrev, total);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t group_sums_t(const ScanShape &s, int Lrev, const void *dt, const float *yB_rev, const float *yC, void *dB, void *dC,
+                        hipStream_t st) {
+    const long long total = (long long)s.B * s.L * s.G * (s.N / 8);
+    bwd_group_sums_kernel<T><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(static_cast<const T *>(dt), yB_rev, yC,
+                                                                            static_cast<T *>(dB), static_cast<T *>(dC), s, Lrev, total);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t anchors_t(const ScanShape &s, const void *dt, const float *A, const float *fwd_prev, const float *rev_prev,
+                     const float *rev_final, const float *init_t, const float *fwd_final, const float *dfin_t,
+                     double *anchor, hipStream_t st) {
+    const long long waves = (long long)s.B * (s.nc + 1) * s.H;
+    bwd_anchor_kernel<T><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st>>>(
+        static_cast<const T *>(dt), A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, anchor, s);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float *e1, const float *u, const double *anchor,
+                 void *ddt, double *dA_part, hipStream_t st) {
+    if (s.Q > 64) return hipErrorInvalidValue;  // one pass of the wave per chunk
+    const long long waves = (long long)s.B * s.H;
+    bwd_ddt_kernel<T><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, e1, u, anchor,
+                                                                              static_cast<T *>(ddt), dA_part, s);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t dinit_t(const ScanShape &s, const void *dt, const float *A, const float *gfin, float *dinit, hipStream_t st) {
+    const long long total = (long long)s.B * s.H * s.P * s.N;
+    bwd_dinit_kernel<T><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, gfin, dinit, s, total);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_gather_rows(int dtype, const void *src, void *dst, int B, int Lsrc, int Ldst, int groups, int W,
+                              int rep, bool reverse, hipStream_t st) {
+    return dtype ? gather_t<__bf16>(src, dst, B, Lsrc, Ldst, groups, W, rep, reverse, st)
+                 : gather_t<float>(src, dst, B, Lsrc, Ldst, groups, W, rep, reverse, st);
+}
+
+hipError_t launch_transpose_state(const float *src, float *dst, long long BH, int P, int N, hipStream_t st) {
+    const long long total = BH * P * N;
+    transpose_state_kernel<<<dim3(blocks_for(total)), dim3(256), 0, st>>>(src, dst, P, N, total);
+    return hipGetLastError();
+}
+
+hipError_t launch_bwd_rows(const ScanShape &s, int Lrev, int dtype, const void *x, const void *dy, const void *dt,
+                           const void *Cm, const float *D, const float *r_rev, const float *yC, void *dx, float *e1,
+                           float *dd, float *u, hipStream_t st) {
+    return dtype ? rows_t<__bf16>(s, Lrev, x, dy, dt, Cm, D, r_rev, yC, dx, e1, dd, u, st)
+                 : rows_t<float>(s, Lrev, x, dy, dt, Cm, D, r_rev, yC, dx, e1, dd, u, st);
+}
+
+hipError_t launch_bwd_group_sums(const ScanShape &s, int Lrev, int dtype, const void *dt, const float *yB_rev,
+                                 const float *yC, void *dB, void *dC, hipStream_t st) {
+    return dtype ? group_sums_t<__bf16>(s, Lrev, dt, yB_rev, yC, dB, dC, st)
+                 : group_sums_t<float>(s, Lrev, dt, yB_rev, yC, dB, dC, st);
+}
+
+hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, const float *A, const float *fwd_prev,
+                              const float *rev_prev, const float *rev_final, const float *init_t, const float *fwd_final,
+                              const float *dfin_t, double *anchor, hipStream_t st) {
+    return dtype ? anchors_t<__bf16>(s, dt, A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, anchor, st)
+                 : anchors_t<float>(s, dt, A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, anchor, st);
+}
+
+hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
+                          const double *anchor, void *ddt, double *dA_part, hipStream_t st) {
+    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, anchor, ddt, dA_part, st)
+                 : ddt_t<float>(s, dt, A, e1, u, anchor, ddt, dA_part, st);
+}
+
+hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const float *dd, float *dA, float *dD,
+                                hipStream_t st) {
+    bwd_head_sums_kernel<<<dim3(s.H), dim3(256), 0, st>>>(dA_part, dd, dA, dD, s);
+    return hipGetLastError();
+}
+
+hipError_t launch_bwd_dinit(const ScanShape &s, int dtype, const void *dt, const float *A, const float *gfin,
+                            float *dinit, hipStream_t st) {
+    return dtype ? dinit_t<__bf16>(s, dt, A, gfin, dinit, st) : dinit_t<float>(s, dt, A, gfin, dinit, st);
+}
+
+}  // namespace ssd

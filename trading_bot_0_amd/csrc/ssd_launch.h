@@ -29,8 +29,13 @@ size_t chunk_scan_lds_bytes(const ScanShape &s, int elem_bytes);
 // dtcs is the stage-1 output [B,H,nc,4,Q] float32: log2(e) * cumulative dt*A as a hi/lo pair, dt, and
 // the stage-2 weight exp2(alpha[Q-1] - alpha[l]) * dt[l].
 // reset: [B,L] bytes or NULL; a non-zero entry restarts the state from zero before that timestep
+// mode 0: decays exp(dt_t A) and input weights dt_t (the forward).  mode 1: the time-reversed adjoint
+// recurrence of the backward pass: step t decays by exp(dt_{L-t} A) and every step weighs one; dt then has
+// dt_len <= L rows per batch row (0 = L) and steps whose L-t falls outside 1..dt_len-1 do not decay, so a
+// reversed sequence can carry L - dt_len leading no-op steps that pad it to whole chunks.
 hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A,
-                               const unsigned char *reset, float *dtcs, hipStream_t stream);
+                               const unsigned char *reset, float *dtcs, hipStream_t stream, int mode = 0,
+                               int dt_len = 0);
 hipError_t launch_chunk_state(const ScanShape &s, int dtype, const void *x, const void *Bm,
                               const float *dtcs, float *states, hipStream_t stream);
 // stages 2+3 in one pass: writes the state entering each chunk into `prev` and the final state
@@ -71,5 +76,36 @@ hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, 
                             void *x, void *Bm, void *Cm, void *dt, hipStream_t stream);
 hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                              float eps, void *out, hipStream_t stream);
+
+// The memory-bound kernels of the backward pass (its three heavy products run on the stage launchers above with
+// the operands' roles swapped).  dtype: 0 = float32, 1 = bf16 activations and gradients.
+// gather_rows: dst[b, t', (g*rep + k)*W + w] = src[b, t, g*W + w] for t' < Ldst, with t = Ldst-1-t' if reverse
+// else t'; rows with t >= Lsrc are zero.  W a multiple of 8.
+hipError_t launch_gather_rows(int dtype, const void *src, void *dst, int B, int Lsrc, int Ldst, int groups, int W,
+                              int rep, bool reverse, hipStream_t stream);
+// [BH, P, N] -> [BH, N, P]
+hipError_t launch_transpose_state(const float *src, float *dst, long long BH, int P, int N, hipStream_t stream);
+// per (b,t,h): dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1.  r_rev (and yB_rev below) hold
+// Lrev >= L rows per batch row, row Lrev-1-t for timestep t.
+hipError_t launch_bwd_rows(const ScanShape &s, int Lrev, int dtype, const void *x, const void *dy, const void *dt, const void *Cm,
+                           const float *D, const float *r_rev, const float *yC, void *dx, float *e1, float *dd,
+                           float *u, hipStream_t stream);
+// dB = sum over a group's heads of dt yB (yB_rev time-reversed), dC = the same of yC
+hipError_t launch_bwd_group_sums(const ScanShape &s, int Lrev, int dtype, const void *dt, const float *yB_rev, const float *yC,
+                                 void *dB, void *dC, hipStream_t stream);
+// anchor [B,nc+1,H]: q at the first step of chunk c = exp(dt A) <adjoint state, forward state> entering the chunk:
+// fwd_prev [B,nc,H,N,P] are the forward-time transposed scan's chunk states, rev_prev those of the reversed one
+// (chunk nc-c there), rev_final its final state and init_t the transposed initial state (NULL = zero) for c = 0;
+// c = nc is the end of the sequence, <dfin_t, fwd_final> (zero when dfin_t is NULL).
+hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, const float *A, const float *fwd_prev,
+                              const float *rev_prev, const float *rev_final, const float *init_t, const float *fwd_final,
+                              const float *dfin_t, double *anchor, hipStream_t stream);
+// q_t between the anchors of its chunk (chunk <= 64 steps); ddt = e1 + A q; dA_part[b,h] = sum_t dt q
+hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
+                          const double *anchor, void *ddt, double *dA_part, hipStream_t stream);
+hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const float *dd, float *dA, float *dD,
+                                hipStream_t stream);
+hipError_t launch_bwd_dinit(const ScanShape &s, int dtype, const void *dt, const float *A, const float *gfin,
+                            float *dinit, hipStream_t stream);
 
 }  // namespace ssd

@@ -23,7 +23,8 @@ template <typename T, int EPL>  // EPL = elements per lane = max(Q/64, 1)
 __global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__ dt,
                                                            const float *__restrict__ A,
                                                            const unsigned char *__restrict__ reset,
-                                                           float *__restrict__ dtcs, ScanShape s) {
+                                                           float *__restrict__ dtcs, ScanShape s, int mode,
+                                                           int dt_len) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *tile = reinterpret_cast<float *>(smem);  // [H][Q+1]
     const int ldt = s.Q + 1;
@@ -33,7 +34,12 @@ __global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__
     for (int idx = threadIdx.x; idx < s.Q * s.H; idx += blockDim.x) {
         const int l = idx / s.H, h = idx % s.H;
         const int t = t0 + l;
-        const float v = (t < s.L) ? (float)dt[((size_t)b * s.L + t) * s.H + h] : 0.f;
+        // mode 1 (the time-reversed adjoint recurrence): step t decays by the dt of step L - t of a dt tensor
+        // of dt_len <= L rows; steps that fall outside it (step 0, and the L - dt_len leading steps that pad
+        // the reversed sequence to whole chunks) do not decay
+        float v;
+        if (mode == 0) v = (t < s.L) ? (float)dt[((size_t)b * s.L + t) * s.H + h] : 0.f;
+        else v = (t < s.L && s.L - t >= 1 && s.L - t < dt_len) ? (float)dt[((size_t)b * dt_len + (s.L - t)) * s.H + h] : 0.f;
         tile[h * ldt + l] = v;
     }
     for (int l = threadIdx.x; l < s.Q; l += blockDim.x)
@@ -67,8 +73,10 @@ __global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__
                 const float hi = (float)al;
                 row[e] = hi;
                 row[s.Q + e] = (float)(al - (double)hi);
-                row[2 * s.Q + e] = dtv[e];
-                row[3 * s.Q + e] = exp2_hw(fminf((float)((total - cum) * kLog2e), 0.f)) * dtv[e];
+                // the input weight: dt, or in mode 1 one for every step of the sequence (padding steps stay no-ops)
+                const float wv = mode == 0 ? dtv[e] : ((t0 + l0 + e < s.L) ? 1.f : 0.f);
+                row[2 * s.Q + e] = wv;
+                row[3 * s.Q + e] = exp2_hw(fminf((float)((total - cum) * kLog2e), 0.f)) * wv;
             }
         }
     }
@@ -270,23 +278,25 @@ __global__ __launch_bounds__(256) void steps_kernel(float *__restrict__ state, c
 // ------------------------------------------------------------------------------------------
 template <typename T>
 static hipError_t cumsum_dispatch(const ScanShape &s, const void *dt, const float *A, const unsigned char *reset,
-                                  float *dtcs, hipStream_t st) {
+                                  float *dtcs, hipStream_t st, int mode, int dt_len) {
     const dim3 grid(s.B * s.nc), block(256);
     const size_t lds = ((size_t)s.H * (s.Q + 1) + s.Q) * sizeof(float);
     const T *d = static_cast<const T *>(dt);
     if (s.Q <= 64) {
-        chunk_cumsum_kernel<T, 1><<<grid, block, lds, st>>>(d, A, reset, dtcs, s);
+        chunk_cumsum_kernel<T, 1><<<grid, block, lds, st>>>(d, A, reset, dtcs, s, mode, dt_len);
     } else if (s.Q == 128) {
-        chunk_cumsum_kernel<T, 2><<<grid, block, lds, st>>>(d, A, reset, dtcs, s);
+        chunk_cumsum_kernel<T, 2><<<grid, block, lds, st>>>(d, A, reset, dtcs, s, mode, dt_len);
     } else {
-        chunk_cumsum_kernel<T, 4><<<grid, block, lds, st>>>(d, A, reset, dtcs, s);
+        chunk_cumsum_kernel<T, 4><<<grid, block, lds, st>>>(d, A, reset, dtcs, s, mode, dt_len);
     }
     return hipGetLastError();
 }
 
 hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A,
-                               const unsigned char *reset, float *dtcs, hipStream_t st) {
-    return dtype ? cumsum_dispatch<__bf16>(s, dt, A, reset, dtcs, st) : cumsum_dispatch<float>(s, dt, A, reset, dtcs, st);
+                               const unsigned char *reset, float *dtcs, hipStream_t st, int mode, int dt_len) {
+    if (dt_len <= 0) dt_len = s.L;
+    return dtype ? cumsum_dispatch<__bf16>(s, dt, A, reset, dtcs, st, mode, dt_len)
+                 : cumsum_dispatch<float>(s, dt, A, reset, dtcs, st, mode, dt_len);
 }
 
 hipError_t launch_state_passing(const ScanShape &s, const float *states, const float *dtcs, const float *init,

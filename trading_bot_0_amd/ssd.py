@@ -43,6 +43,8 @@ EXPORTED_SYMBOLS = (
     "ssd_steps_fwd",
     "ssd_block_pre_fwd",
     "ssd_block_post_fwd",
+    "ssd_chunk_scan_bwd_workspace_bytes",
+    "ssd_chunk_scan_bwd",
 )
 
 
@@ -100,6 +102,8 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
         lib.ssd_steps_fwd.argtypes = [POINTER(SsdStepDims), c_int64, c_int, P, P, P, P, P, P, P, P, P, P]
+        lib.ssd_chunk_scan_bwd_workspace_bytes.argtypes = [POINTER(SsdDims), c_int, POINTER(c_size_t)]
+        lib.ssd_chunk_scan_bwd.argtypes = [POINTER(SsdDims), c_int] + [P] * 17 + [c_size_t, P]
         for name in EXPORTED_SYMBOLS[2:]:
             getattr(lib, name).restype = c_int   # (argument types of the block stages: block.py)
         _lib = lib
@@ -261,6 +265,48 @@ def ssd_chunk_scan(
                                       _stream_ptr(x))
     _check(lib, rc)
     return y, final
+
+
+def ssd_chunk_scan_backward(x, dt, A, Bm, Cm, D, dy, chunk: int = 128, initial_states=None, dfinal_states=None,
+                            need_dinitial_states: bool = False, workspace=None) -> dict:
+    """Gradients of the scan's outputs (y weighted by `dy`, the final state by `dfinal_states`) with respect to
+    its inputs.  Returns a dict with dx, ddt, dB, dC (input dtype), dA, dD (None without D) and, if asked for,
+    dinitial_states (float32)."""
+    lib = load_library()
+    dims = _scan_dims(x, Bm, chunk)
+    _validate_scan_inputs(x, dt, A, Bm, Cm, D, initial_states, dims)
+    code = _dtype_code(x)
+    _require(dy, "dy", x.shape, x.dtype)
+    sshape = (dims.batch, dims.nheads, dims.headdim, dims.dstate)
+    if dfinal_states is not None:
+        _require(dfinal_states, "dfinal_states", sshape, torch.float32)
+    dev = x.device
+    out = {"dx": torch.empty_like(x), "ddt": torch.empty_like(dt), "dB": torch.empty_like(Bm), "dC": torch.empty_like(Cm),
+           "dA": torch.empty(dims.nheads, dtype=torch.float32, device=dev),
+           "dD": None if D is None else torch.empty(dims.nheads, dtype=torch.float32, device=dev),
+           "dinitial_states": torch.empty(sshape, dtype=torch.float32, device=dev) if need_dinitial_states else None}
+    need = c_size_t(0)
+    _check(lib, lib.ssd_chunk_scan_bwd_workspace_bytes(byref(dims), code, byref(need)))
+    if workspace is None:
+        workspace = torch.empty(need.value, dtype=torch.uint8, device=dev)
+    elif (not workspace.is_cuda) or workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+        raise ValueError("SSD workspace must be a contiguous uint8 GPU tensor")
+    rc = lib.ssd_chunk_scan_bwd(byref(dims), code, x.data_ptr(), dt.data_ptr(), A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(),
+                                _ptr(D), _ptr(initial_states), dy.data_ptr(), _ptr(dfinal_states),
+                                out["dx"].data_ptr(), out["ddt"].data_ptr(), out["dA"].data_ptr(), out["dB"].data_ptr(),
+                                out["dC"].data_ptr(), _ptr(out["dD"]), _ptr(out["dinitial_states"]),
+                                workspace.data_ptr(), workspace.numel(), _stream_ptr(x))
+    _check(lib, rc)
+    return out
+
+
+def backward_workspace_bytes(batch, seqlen, nheads, headdim, dstate, ngroups, chunk, dtype=torch.bfloat16) -> int:
+    lib = load_library()
+    dims = SsdDims(batch, seqlen, nheads, headdim, dstate, ngroups, chunk)
+    need = c_size_t(0)
+    code = SSD_DTYPE_F32 if dtype == torch.float32 else SSD_DTYPE_BF16
+    _check(lib, lib.ssd_chunk_scan_bwd_workspace_bytes(byref(dims), code, byref(need)))
+    return need.value
 
 
 class PreparedChunkScan:
