@@ -179,7 +179,7 @@ BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
     w.dd = take(BL * s.H * sizeof(float));
     w.u = take(BL * s.H * sizeof(float));
     w.anchor = take((size_t)s.B * (s.nc + 1) * s.H * sizeof(double));
-    w.da_part = take((size_t)s.B * s.H * sizeof(double));
+    w.da_part = take((size_t)2 * s.B * s.H * sizeof(double));  // and the parts of dD behind them
     w.total = off;
     return w;
 }
@@ -413,10 +413,19 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         BWD_LAUNCH(ssd::launch_transpose_state(dfinal_states, atf(w.dfin_t), (long long)s.B * s.H, s.P, s.N, st), "transpose");
         dfin_t = atf(w.dfin_t);
     }
-    // r = g B: the adjoint recurrence, reversed in time; its last state is g_0
-    if (int rc = run_staged(sR, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states, nullptr, 1,
-                            at(w.r_rev), atf(w.gfin), dtcs, states, st, s.L))
+    // r = g B: the adjoint recurrence, reversed in time; its last state is g_0.  It has the forward's own shape,
+    // so large bf16 batches take the one-pass kernel.
+    if (takes_one_pass(sR, inner)) {
+        ssd::ScanShape f = sR;
+        f.mode = 1;
+        f.dt_len = s.L;
+        BWD_LAUNCH(ssd::launch_fused_scan(f, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states,
+                                          nullptr, at(w.r_rev), atf(w.gfin), st),
+                   "one-pass adjoint scan");
+    } else if (int rc = run_staged(sR, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states, nullptr,
+                                   1, at(w.r_rev), atf(w.gfin), dtcs, states, st, s.L)) {
         return rc;
+    }
     // yB = x . g: the same recurrence with the state transposed; its chunk states stay in `states`
     if (int rc = run_staged(sTR, inner, at(w.c_rev_h), dt, A, at(w.dy_rev), at(w.x_rev), nullptr, dfin_t, nullptr, 1,
                             at(w.yb_rev), atf(w.gfin_t), dtcs, states, st, s.L))
@@ -432,8 +441,10 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, anchor, st),
                "backward anchors");
     double *da_part = reinterpret_cast<double *>(base + w.da_part);
-    BWD_LAUNCH(ssd::launch_bwd_ddt(s, el, dt, A, atf(w.e1), atf(w.u), anchor, ddt, da_part, st), "backward ddt");
-    BWD_LAUNCH(ssd::launch_bwd_head_sums(s, da_part, atf(w.dd), dA, dD, st), "backward head sums");
+    double *dd_part = da_part + (size_t)s.B * s.H;
+    BWD_LAUNCH(ssd::launch_bwd_ddt(s, el, dt, A, atf(w.e1), atf(w.u), atf(w.dd), anchor, ddt, da_part, dd_part, st),
+               "backward ddt");
+    BWD_LAUNCH(ssd::launch_bwd_head_sums(s, da_part, dd_part, dA, dD, st), "backward head sums");
     if (dinitial_states != nullptr)
         BWD_LAUNCH(ssd::launch_bwd_dinit(s, el, dt, A, atf(w.gfin), dinitial_states, st), "backward dinit");
 #undef BWD_LAUNCH

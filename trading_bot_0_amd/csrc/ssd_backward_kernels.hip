@@ -88,8 +88,9 @@ __global__ __launch_bounds__(256) void transpose_state_kernel(const float *__res
     dst[gid] = src[bh * pn + (size_t)p * N + n];
 }
 
-// One thread per (b, t, h): dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1.
-// r_rev is the reversed scan's float output (time reversed), yC the forward-time transposed scan's.
+// Eight lanes per (b, t, h), one 8-element piece of a row each (headdim and dstate are at most 64):
+// dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1; the three dot products are summed over the
+// eight lanes.  r_rev is the reversed scan's float output (time reversed), yC the forward-time transposed scan's.
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                                                        const T *__restrict__ dt, const T *__restrict__ Cm,
@@ -97,19 +98,22 @@ __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, 
                                                        const float *__restrict__ yC, T *__restrict__ dx,
                                                        float *__restrict__ e1, float *__restrict__ dd,
                                                        float *__restrict__ u, ScanShape s, int Lrev, long long total) {
-    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long gid = tid >> 3;  // the row; whole groups of eight lanes leave together
     if (gid >= total) return;
+    const int piece = (int)(tid & 7) * 8;
     const int h = (int)(gid % s.H);
     const long long bt = gid / s.H;
     const int t = (int)(bt % s.L);
     const long long b = bt / s.L;
     const int g = h / (s.H / s.G);
     const float dtv = (float)dt[gid], dh = D ? D[h] : 0.f;
-    const size_t row = (size_t)gid * s.P, rrow = ((size_t)(b * Lrev + (Lrev - 1 - t)) * s.H + h) * s.P;
-    float se1 = 0.f, sdd = 0.f;
-    for (int p = 0; p < s.P; p += 8) {
-        const Row8<T> xv = Row8<T>::load(x + row + p), dv = Row8<T>::load(dy + row + p);
-        const Row8<float> rv = Row8<float>::load(r_rev + rrow + p);
+    float se1 = 0.f, sdd = 0.f, sc = 0.f;
+    if (piece < s.P) {
+        const size_t row = (size_t)gid * s.P + piece;
+        const size_t rrow = ((size_t)(b * Lrev + (Lrev - 1 - t)) * s.H + h) * s.P + piece;
+        const Row8<T> xv = Row8<T>::load(x + row), dv = Row8<T>::load(dy + row);
+        const Row8<float> rv = Row8<float>::load(r_rev + rrow);
         Row8<T> o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -117,20 +121,25 @@ __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, 
             se1 += xv.v[i] * rv.v[i];
             sdd += dv.v[i] * xv.v[i];
         }
-        o.store(dx + row + p);
+        o.store(dx + row);
     }
-    float sc = 0.f;
-    const T *crow = Cm + ((size_t)bt * s.G + g) * s.N;
-    const float *yrow = yC + (size_t)gid * s.N;
-    for (int n = 0; n < s.N; n += 8) {
-        const Row8<T> cv = Row8<T>::load(crow + n);
-        const Row8<float> yv = Row8<float>::load(yrow + n);
+    if (piece < s.N) {
+        const Row8<T> cv = Row8<T>::load(Cm + ((size_t)bt * s.G + g) * s.N + piece);
+        const Row8<float> yv = Row8<float>::load(yC + (size_t)gid * s.N + piece);
 #pragma unroll
         for (int i = 0; i < 8; ++i) sc += cv.v[i] * yv.v[i];
     }
-    e1[gid] = se1;
-    dd[gid] = sdd;
-    u[gid] = sc - dtv * se1;
+#pragma unroll
+    for (int m = 1; m < 8; m <<= 1) {
+        se1 += __shfl_xor(se1, m, 8);
+        sdd += __shfl_xor(sdd, m, 8);
+        sc += __shfl_xor(sc, m, 8);
+    }
+    if (piece == 0) {
+        e1[gid] = se1;
+        dd[gid] = sdd;
+        u[gid] = sc - dtv * se1;
+    }
 }
 
 // One thread per (b, t, g, 8 state columns): dB = sum over the group's heads of dt yB, dC = the same of yC.
@@ -211,12 +220,13 @@ __global__ __launch_bounds__(256) void bwd_anchor_kernel(const T *__restrict__ d
 // chunk (the anchors) and obeys q_t - q_{t+1} = u_t in between; the computed u do not sum exactly to the
 // difference of the anchors, and the mismatch is spread evenly over the chunk's steps:
 // q_t = anchor_c - sum_{v < t in the chunk} u_v - mismatch * (steps before t) / (steps of the chunk).
-// ddt_t = e1_t + A q_t and this sequence's part of dA = sum dt_t q_t.  Sums in float64.
+// ddt_t = e1_t + A q_t and this sequence's parts of dA = sum dt_t q_t and of dD = sum dd_t.  Sums in float64.
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, const float *__restrict__ A,
                                                       const float *__restrict__ e1, const float *__restrict__ u,
-                                                      const double *__restrict__ anchor, T *__restrict__ ddt,
-                                                      double *__restrict__ dA_part, ScanShape s) {
+                                                      const float *__restrict__ dd, const double *__restrict__ anchor,
+                                                      T *__restrict__ ddt, double *__restrict__ dA_part,
+                                                      double *__restrict__ dD_part, ScanShape s) {
     const int lane = threadIdx.x & 63;
     const long long bh = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (bh >= (long long)s.B * s.H) return;
@@ -227,7 +237,7 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
                                 __builtin_amdgcn_readlane(__double2loint(v), 63));
     };
     const double a = (double)A[h];
-    double da = 0.0;
+    double da = 0.0, sdd = 0.0;
     for (int c = 0; c < s.nc; ++c) {
         const double q0 = anchor[((size_t)b * (s.nc + 1) + c) * s.H + h];
         const double q1 = anchor[((size_t)b * (s.nc + 1) + c + 1) * s.H + h];
@@ -241,21 +251,26 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
             const double q = q0 - (incl - uv) - mismatch * (double)lane / (double)len;
             ddt[at] = (T)(float)((double)e1[at] + a * q);
             da += (double)(float)dt[at] * q;
+            sdd += (double)dd[at];
         }
     }
-    const double tot = last_lane(wave_inclusive_scan(da));
-    if (lane == 0) dA_part[bh] = tot;
+    const double tot = last_lane(wave_inclusive_scan(da)), totd = last_lane(wave_inclusive_scan(sdd));
+    if (lane == 0) {
+        dA_part[bh] = tot;
+        dD_part[bh] = totd;
+    }
 }
 
-// One workgroup per head: dA[h] = sum_b dA_part[b,h]; dD[h] = sum_{b,t} dd[b,t,h] (float64 sums).
-__global__ __launch_bounds__(256) void bwd_head_sums_kernel(const double *__restrict__ dA_part, const float *__restrict__ dd,
+// One workgroup per head: dA[h] = sum_b dA_part[b,h], dD[h] = sum_b dD_part[b,h] (float64 sums).
+__global__ __launch_bounds__(256) void bwd_head_sums_kernel(const double *__restrict__ dA_part, const double *__restrict__ dD_part,
                                                             float *__restrict__ dA, float *__restrict__ dD, ScanShape s) {
     __shared__ double red[2][256];
     const int h = blockIdx.x;
     double sa = 0.0, sd = 0.0;
-    for (long long i = threadIdx.x; i < s.B; i += blockDim.x) sa += dA_part[i * s.H + h];
-    if (dD != nullptr)
-        for (long long i = threadIdx.x; i < (long long)s.B * s.L; i += blockDim.x) sd += (double)dd[i * s.H + h];
+    for (long long i = threadIdx.x; i < s.B; i += blockDim.x) {
+        sa += dA_part[i * s.H + h];
+        sd += dD_part[i * s.H + h];
+    }
     red[0][threadIdx.x] = sa;
     red[1][threadIdx.x] = sd;
     __syncthreads();
@@ -301,7 +316,7 @@ template <typename T>
 hipError_t rows_t(const ScanShape &s, int Lrev, const void *x, const void *dy, const void *dt, const void *Cm, const float *D,
                   const float *r_rev, const float *yC, void *dx, float *e1, float *dd, float *u, hipStream_t st) {
     const long long total = (long long)s.B * s.L * s.H;
-    bwd_rows_kernel<T><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(
+    bwd_rows_kernel<T><<<dim3(blocks_for(total * 8)), dim3(256), 0, st>>>(
         static_cast<const T *>(x), static_cast<const T *>(dy), static_cast<const T *>(dt), static_cast<const T *>(Cm), D,
         r_rev, yC, static_cast<T *>(dx), e1, dd, u, s, Lrev, total);
     return hipGetLastError();
@@ -327,12 +342,12 @@ hipError_t anchors_t(const ScanShape &s, const void *dt, const float *A, const f
 }
 
 template <typename T>
-hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float *e1, const float *u, const double *anchor,
-                 void *ddt, double *dA_part, hipStream_t st) {
+hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float *e1, const float *u, const float *dd,
+                 const double *anchor, void *ddt, double *dA_part, double *dD_part, hipStream_t st) {
     if (s.Q > 64) return hipErrorInvalidValue;  // one pass of the wave per chunk
     const long long waves = (long long)s.B * s.H;
-    bwd_ddt_kernel<T><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, e1, u, anchor,
-                                                                              static_cast<T *>(ddt), dA_part, s);
+    bwd_ddt_kernel<T><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, e1, u, dd, anchor,
+                                                                              static_cast<T *>(ddt), dA_part, dD_part, s);
     return hipGetLastError();
 }
 
@@ -378,14 +393,15 @@ hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, con
 }
 
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
-                          const double *anchor, void *ddt, double *dA_part, hipStream_t st) {
-    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, anchor, ddt, dA_part, st)
-                 : ddt_t<float>(s, dt, A, e1, u, anchor, ddt, dA_part, st);
+                          const float *dd, const double *anchor, void *ddt, double *dA_part, double *dD_part,
+                          hipStream_t st) {
+    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, st)
+                 : ddt_t<float>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, st);
 }
 
-hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const float *dd, float *dA, float *dD,
+hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,
                                 hipStream_t st) {
-    bwd_head_sums_kernel<<<dim3(s.H), dim3(256), 0, st>>>(dA_part, dd, dA, dD, s);
+    bwd_head_sums_kernel<<<dim3(s.H), dim3(256), 0, st>>>(dA_part, dD_part, dA, dD, s);
     return hipGetLastError();
 }
 

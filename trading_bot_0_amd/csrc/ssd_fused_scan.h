@@ -158,7 +158,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     const T *xb = x + (size_t)b * s.L * HP + xcol0;
     const T *Bb = Bm + ((size_t)b * s.L * s.G + g) * N;
     const T *Cb = Cm + ((size_t)b * s.L * s.G + g) * N;
-    const T *dtb = dt + (size_t)b * s.L * s.H + h;
+    // mode 1 (the time-reversed adjoint recurrence): step t decays by the dt of step L - t of a dt tensor of
+    // dt_len rows, steps outside it do not decay, and every step's input weighs one instead of dt
+    const int dt_rows = s.mode ? s.dt_len : s.L;
+    const T *dtb = dt + (size_t)b * dt_rows * s.H + h;
     const unsigned char *rsb = reset ? reset + (size_t)b * s.L : nullptr;  // state restarts, see kResetLog2
     TO *yb = y + (size_t)b * s.L * HP + h * s.P + pb * 32;
     const float dh = D ? D[h] : 0.f;
@@ -190,6 +193,15 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         const unsigned dt_off0 = (tv & 63) * EPL * s.H;
         const T *bp = Bb + (size_t)t0 * s.G * N, *cp = Cb + (size_t)t0 * s.G * N;
         const T *xp = xb + (size_t)t0 * HP, *dp = dtb + (size_t)t0 * s.H;
+        auto dt_bits = [&](int e, bool ok) {  // dt of row t0 + lane*EPL + e as raw bits, zero where it does not apply
+            const int row = t0 + (tv & 63) * EPL + e;
+            if (s.mode) {
+                const int src = s.L - row;
+                return (ok && src >= 1 && src < dt_rows) ? __builtin_bit_cast(unsigned short, dtb[(size_t)src * s.H])
+                                                         : (unsigned short)0;
+            }
+            return ok ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
+        };
         // (a conditional expression over *ptr and a zero constant would become a load through a selected
         // pointer, with the constant in scratch memory)
         auto ld16 = [](const T *ptr, bool ok) {
@@ -208,7 +220,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
             for (int u = 0; u < UX; ++u) xq[u] = *reinterpret_cast<const uint4 *>(xp + (size_t)u * 16 * HP + x_off0);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
-                dq[e] = (Q >= 64 || (tv & 63) < Q) ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
+                dq[e] = dt_bits(e, Q >= 64 || (tv & 63) < Q);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
                 rq[e] = (rsb != nullptr && (Q >= 64 || (tv & 63) < Q)) ? rsb[t0 + (tv & 63) * EPL + e] : (unsigned char)0;
@@ -223,7 +235,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
             for (int u = 0; u < UX; ++u) xq[u] = ld16(xp + (size_t)u * 16 * HP + x_off0, x_row0 + u * 16 < rows);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
-                dq[e] = ((tv & 63) * EPL + e < rows) ? __builtin_bit_cast(unsigned short, dp[dt_off0 + e * s.H]) : (unsigned short)0;
+                dq[e] = dt_bits(e, (tv & 63) * EPL + e < rows);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
                 rq[e] = (rsb != nullptr && (tv & 63) * EPL + e < rows) ? rsb[t0 + (tv & 63) * EPL + e] : (unsigned char)0;
@@ -289,6 +301,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
             for (int e = 0; e < EPL; ++e) {
                 dtv[e] = (float)__builtin_bit_cast(__bf16, dq[e]);
                 run += (double)dtv[e] * a_h - (rq[e] ? kResetDrop : 0.0);
+                if (s.mode) dtv[e] = (t0 + lane * EPL + e < s.L) ? 1.f : 0.f;  // from here on dtv is the input weight
                 cs[e] = run;
             }
             const double excl = wave_inclusive_scan(run) - run;

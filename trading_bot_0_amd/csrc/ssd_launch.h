@@ -9,6 +9,9 @@ namespace ssd {
 
 struct ScanShape {
     int B, L, H, P, N, G, Q, nc;
+    // The one-pass kernel only (the staged path takes these as arguments of launch_chunk_cumsum): decays and input
+    // weights of the time-reversed adjoint recurrence, read from a dt tensor of dt_len <= L rows per batch row.
+    int mode = 0, dt_len = 0;
 };
 
 struct StepShape {
@@ -100,10 +103,13 @@ hipError_t launch_bwd_group_sums(const ScanShape &s, int Lrev, int dtype, const 
 hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, const float *A, const float *fwd_prev,
                               const float *rev_prev, const float *rev_final, const float *init_t, const float *fwd_final,
                               const float *dfin_t, double *anchor, hipStream_t stream);
-// q_t between the anchors of its chunk (chunk <= 64 steps); ddt = e1 + A q; dA_part[b,h] = sum_t dt q
+// q_t between the anchors of its chunk (chunk <= 64 steps); ddt = e1 + A q; dA_part[b,h] = sum_t dt q,
+// dD_part[b,h] = sum_t dd
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
-                          const double *anchor, void *ddt, double *dA_part, hipStream_t stream);
-hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const float *dd, float *dA, float *dD,
+                          const float *dd, const double *anchor, void *ddt, double *dA_part, double *dD_part,
+                          hipStream_t stream);
+// dA[h], dD[h] (NULL allowed) = the sums over the batch of the parts
+hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,
                                 hipStream_t stream);
 hipError_t launch_bwd_dinit(const ScanShape &s, int dtype, const void *dt, const float *A, const float *gfin,
                             float *dinit, hipStream_t stream);
