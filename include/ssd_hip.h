@@ -182,15 +182,15 @@ int ssd_steps_fwd(const ssd_step_dims *dims, int64_t nsteps, int dtype, float *s
  * update this would run in; the reference's historical benchmark case is mamba2_fwd_bwd_train,
  * benchmark_results/bench_20260112_070055.json:16-23).  dtype 0 = float32, 1 = bf16 (activations and their
  * gradients in that type; A, D, states and their gradients float32).
- * In: the forward's inputs, dy [B,L,H,P], and optionally dfinal_states [B,H,P,N] (NULL if the final state does
- * not reach the loss).
+ * In: the forward's inputs (reset [B,L] as for ssd_chunk_scan_reset_fwd, NULL = none), dy [B,L,H,P], and
+ * optionally dfinal_states [B,H,P,N] (NULL if the final state does not reach the loss).
  * Out: dx [B,L,H,P], ddt [B,L,H], dA [H], dB, dC [B,L,G,N], dD [H] (NULL allowed; must be NULL without D),
  * dinitial_states [B,H,P,N] (NULL allowed; defined also when the forward had no initial state).
  * dstate <= 64 and headdim 16, 32 or 64 (the pass runs the forward's kernels on the transposed state);
  * other shapes return SSD_ERR_UNSUPPORTED.  Workspace size from ssd_chunk_scan_bwd_workspace_bytes. */
 int ssd_chunk_scan_bwd_workspace_bytes(const ssd_dims *dims, int dtype, size_t *out_bytes);
 int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A, const void *Bm,
-                       const void *Cm, const float *D, const float *initial_states, const void *dy,
+                       const void *Cm, const float *D, const float *initial_states, const uint8_t *reset, const void *dy,
                        const float *dfinal_states, void *dx, void *ddt, float *dA, void *dB, void *dC, float *dD,
                        float *dinitial_states, void *workspace, size_t workspace_bytes, void *hip_stream);
 

@@ -9,13 +9,15 @@ import numpy as np
 from . import ssd_oracle as orc
 
 
-def ssd_backward_sequential(x, dt, A, Bm, Cm, D, init, dy, dfinal=None):
+def ssd_backward_sequential(x, dt, A, Bm, Cm, D, init, dy, dfinal=None, reset=None):
     """Adjoint of ssd_sequential, one timestep at a time, backwards.
     With h_t = a_t h_{t-1} + dt_t x_t (x) B_t, y_t = h_t C_t + D x_t, a_t = exp(dt_t A) and g_t = dLoss/dh_t:
         g_t   = dy_t (x) C_t + a_{t+1} g_{t+1}                    (g_{L-1} also takes dfinal)
         dC_t  = sum_{h in group} dy_t . h_t            dB_t = sum_{h in group} dt_t x_t . g_t
         dx_t  = D dy_t + dt_t g_t B_t                  ddt_t = <g_t, x_t (x) B_t> + A a_t <g_t, h_{t-1}>
         dA    = sum_t dt_t a_t <g_t, h_{t-1}>          dD = sum dy_t x_t        dinit = a_0 g_0
+    reset [B,L] (optional) as in ssd_sequential: h_{t-1} is zero for a row that restarts before step t, and its
+    adjoint does not reach the steps before.
     Returns a dict with dx, ddt, dA, dB, dC, dD (None without D), dinit, and dA_scale, dD_scale [H]: the 2-norms
     of the terms that dA and dD sum over batch and time (the scale rounding errors of such sums are measured on)."""
     x = np.asarray(x, np.float64)
@@ -31,8 +33,13 @@ def ssd_backward_sequential(x, dt, A, Bm, Cm, D, init, dy, dfinal=None):
     hs = np.empty((L + 1, Bsz, H, P, N))
     hs[0] = 0.0 if init is None else np.asarray(init, np.float64)
     a = np.exp(dt * A[None, None, :])                                   # [B,L,H]
+    rs = None if reset is None else (np.asarray(reset) != 0)
+    starts = hs if rs is None else np.empty((L, Bsz, H, P, N))          # the state step t starts from
     for t in range(L):
-        hs[t + 1] = a[:, t, :, None, None] * hs[t] + (dt[:, t, :, None] * x[:, t])[..., None] * Bm[:, t, gh, None, :]
+        if rs is not None:
+            starts[t] = hs[t]
+            starts[t][rs[:, t]] = 0.0
+        hs[t + 1] = a[:, t, :, None, None] * starts[t] + (dt[:, t, :, None] * x[:, t])[..., None] * Bm[:, t, gh, None, :]
     dx = np.zeros_like(x)
     ddt = np.zeros_like(dt)
     dBh = np.zeros((Bsz, L, H, N))
@@ -47,11 +54,13 @@ def ssd_backward_sequential(x, dt, A, Bm, Cm, D, init, dy, dfinal=None):
         gB = np.einsum("bhpn,bhn->bhp", g, Bt)
         dx[:, t] = dt[:, t, :, None] * gB
         dBh[:, t] = dt[:, t, :, None] * np.einsum("bhpn,bhp->bhn", g, x[:, t])
-        gh_prev = np.einsum("bhpn,bhpn->bh", g, hs[t])                   # <g_t, h_{t-1}>
+        gh_prev = np.einsum("bhpn,bhpn->bh", g, starts[t])               # <g_t, h_{t-1}>
         ddt[:, t] = np.einsum("bhp,bhp->bh", gB, x[:, t]) + A[None, :] * a[:, t] * gh_prev
         dA += (dt[:, t] * a[:, t] * gh_prev).sum(0)
         dA_sq += ((dt[:, t] * a[:, t] * gh_prev) ** 2).sum(0)
         g = a[:, t, :, None, None] * g                                   # adjoint of h_{t-1}
+        if rs is not None:
+            g[rs[:, t]] = 0.0
     out = {"ddt": ddt, "dA": dA, "dinit": g, "dD": None, "dA_scale": np.sqrt(dA_sq), "dD_scale": None}
     if D is not None:
         dx = dx + np.asarray(D, np.float64)[None, None, :, None] * dy

@@ -22,8 +22,11 @@ def _case(seed, Bsz=2, L=7, H=4, P=3, N=5, G=2, with_D=True, with_init=True):
     return x, dt, A, Bm, Cm, D, init, dy, dfinal
 
 
+RESET = None
+
+
 def _loss(x, dt, A, Bm, Cm, D, init, dy, dfinal):
-    y, fin = orc.ssd_sequential(x, dt, A, Bm, Cm, D, init)
+    y, fin = orc.ssd_sequential(x, dt, A, Bm, Cm, D, init, reset=RESET)
     return (y * dy).sum() + (0.0 if dfinal is None else (fin * dfinal).sum())
 
 
@@ -96,3 +99,20 @@ def test_general_scan_is_the_forward_for_its_own_decays():
     y, fin = orc.ssd_sequential(x, dt, A, Bm, Cm, None, init)
     y2, fin2 = bwd.scan_general(x, dt * A[None, None, :], dt, Bm, Cm, init)
     assert np.abs(y - y2).max() < 1e-13 and np.abs(fin - fin2).max() < 1e-13
+
+
+def test_adjoint_with_restarts_matches_central_differences():
+    global RESET
+    args = list(_case(11, L=9, G=2))
+    RESET = np.zeros((2, 9), np.uint8)
+    RESET[0, 4] = 1
+    RESET[1, 0] = 1
+    RESET[1, 8] = 1
+    try:
+        got = bwd.ssd_backward_sequential(*args, reset=RESET)
+        for idx, name in {0: "dx", 1: "ddt", 2: "dA", 3: "dB", 4: "dC", 5: "dD", 6: "dinit"}.items():
+            num = _numeric(args, idx)
+            assert np.abs(got[name] - num).max() < 2e-7 * max(1.0, np.abs(num).max()), name
+        assert np.abs(got["dinit"][1]).max() == 0.0
+    finally:
+        RESET = None

@@ -343,7 +343,7 @@ int ssd_chunk_scan_bwd_workspace_bytes(const ssd_dims *dims, int dtype, size_t *
 }
 
 int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A, const void *Bm,
-                       const void *Cm, const float *D, const float *initial_states, const void *dy,
+                       const void *Cm, const float *D, const float *initial_states, const uint8_t *reset, const void *dy,
                        const float *dfinal_states, void *dx, void *ddt, float *dA, void *dB, void *dC, float *dD,
                        float *dinitial_states, void *workspace, size_t workspace_bytes, void *hip_stream) {
     ssd::ScanShape s, sT;
@@ -420,25 +420,26 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         f.mode = 1;
         f.dt_len = s.L;
         BWD_LAUNCH(ssd::launch_fused_scan(f, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states,
-                                          nullptr, at(w.r_rev), atf(w.gfin), st),
+                                          reset, at(w.r_rev), atf(w.gfin), st),
                    "one-pass adjoint scan");
-    } else if (int rc = run_staged(sR, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states, nullptr,
+    } else if (int rc = run_staged(sR, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states, reset,
                                    1, at(w.r_rev), atf(w.gfin), dtcs, states, st, s.L)) {
         return rc;
     }
     // yB = x . g: the same recurrence with the state transposed; its chunk states stay in `states`
-    if (int rc = run_staged(sTR, inner, at(w.c_rev_h), dt, A, at(w.dy_rev), at(w.x_rev), nullptr, dfin_t, nullptr, 1,
+    if (int rc = run_staged(sTR, inner, at(w.c_rev_h), dt, A, at(w.dy_rev), at(w.x_rev), nullptr, dfin_t, reset, 1,
                             at(w.yb_rev), atf(w.gfin_t), dtcs, states, st, s.L))
         return rc;
     // yC = dy . h: the forward recurrence with the state transposed; its chunk states go to `states2`
-    if (int rc = run_staged(sT, inner, b_heads, dt, A, x, dy, nullptr, init_t, nullptr, 0, at(w.yc), atf(w.ffin_t), dtcs,
+    if (int rc = run_staged(sT, inner, b_heads, dt, A, x, dy, nullptr, init_t, reset, 0, at(w.yc), atf(w.ffin_t), dtcs,
                             states2, st))
         return rc;
     BWD_LAUNCH(ssd::launch_bwd_rows(s, Lp, el, x, dy, dt, Cm, D, atf(w.r_rev), atf(w.yc), dx, atf(w.e1), atf(w.dd), atf(w.u), st),
                "backward rows");
     BWD_LAUNCH(ssd::launch_bwd_group_sums(s, Lp, el, dt, atf(w.yb_rev), atf(w.yc), dB, dC, st), "backward group sums");
     double *anchor = reinterpret_cast<double *>(base + w.anchor);
-    BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, anchor, st),
+    BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, reset, anchor,
+                                       st),
                "backward anchors");
     double *da_part = reinterpret_cast<double *>(base + w.da_part);
     double *dd_part = da_part + (size_t)s.B * s.H;
@@ -446,7 +447,7 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
                "backward ddt");
     BWD_LAUNCH(ssd::launch_bwd_head_sums(s, da_part, dd_part, dA, dD, st), "backward head sums");
     if (dinitial_states != nullptr)
-        BWD_LAUNCH(ssd::launch_bwd_dinit(s, el, dt, A, atf(w.gfin), dinitial_states, st), "backward dinit");
+        BWD_LAUNCH(ssd::launch_bwd_dinit(s, el, dt, A, atf(w.gfin), reset, dinitial_states, st), "backward dinit");
 #undef BWD_LAUNCH
     return SSD_OK;
 }

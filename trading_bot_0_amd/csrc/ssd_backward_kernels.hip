@@ -183,6 +183,7 @@ __global__ __launch_bounds__(256) void bwd_anchor_kernel(const T *__restrict__ d
                                                          const float *__restrict__ fwd_prev, const float *__restrict__ rev_prev,
                                                          const float *__restrict__ rev_final, const float *__restrict__ init_t,
                                                          const float *__restrict__ fwd_final, const float *__restrict__ dfin_t,
+                                                         const unsigned char *__restrict__ reset,
                                                          double *__restrict__ anchor, ScanShape s) {
     const int lane = threadIdx.x & 63;
     const long long id = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -211,7 +212,11 @@ __global__ __launch_bounds__(256) void bwd_anchor_kernel(const T *__restrict__ d
         }
     const double incl = wave_inclusive_scan(part);
     if (lane == 63) {
-        const double a = c == s.nc ? 1.0 : exp((double)(float)dt[((size_t)b * s.L + (size_t)c * s.Q) * s.H + h] * (double)A[h]);
+        double a = 1.0;
+        if (c < s.nc) {  // a restart before the chunk's first step: the state entering it does not reach the loss
+            const size_t t = (size_t)b * s.L + (size_t)c * s.Q;
+            a = (reset != nullptr && reset[t] != 0) ? 0.0 : exp((double)(float)dt[t * s.H + h] * (double)A[h]);
+        }
         anchor[id] = a * incl;
     }
 }
@@ -287,17 +292,17 @@ __global__ __launch_bounds__(256) void bwd_head_sums_kernel(const double *__rest
     }
 }
 
-// dinit = exp(dt_0 A) g_0, g_0 = the reversed scan's final state
+// dinit = exp(dt_0 A) g_0, g_0 = the reversed scan's final state; zero for a row that restarts before step 0
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_dinit_kernel(const T *__restrict__ dt, const float *__restrict__ A,
-                                                        const float *__restrict__ gfin, float *__restrict__ dinit,
-                                                        ScanShape s, long long total) {
+                                                        const float *__restrict__ gfin, const unsigned char *__restrict__ reset,
+                                                        float *__restrict__ dinit, ScanShape s, long long total) {
     const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= total) return;
     const long long bh = gid / (s.P * s.N);
     const int h = (int)(bh % s.H);
     const long long b = bh / s.H;
-    const float a0 = __expf((float)dt[(size_t)b * s.L * s.H + h] * A[h]);
+    const float a0 = (reset != nullptr && reset[(size_t)b * s.L] != 0) ? 0.f : __expf((float)dt[(size_t)b * s.L * s.H + h] * A[h]);
     dinit[gid] = a0 * gfin[gid];
 }
 
@@ -334,10 +339,10 @@ hipError_t group_sums_t(const ScanShape &s, int Lrev, const void *dt, const floa
 template <typename T>
 hipError_t anchors_t(const ScanShape &s, const void *dt, const float *A, const float *fwd_prev, const float *rev_prev,
                      const float *rev_final, const float *init_t, const float *fwd_final, const float *dfin_t,
-                     double *anchor, hipStream_t st) {
+                     const unsigned char *reset, double *anchor, hipStream_t st) {
     const long long waves = (long long)s.B * (s.nc + 1) * s.H;
     bwd_anchor_kernel<T><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st>>>(
-        static_cast<const T *>(dt), A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, anchor, s);
+        static_cast<const T *>(dt), A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, reset, anchor, s);
     return hipGetLastError();
 }
 
@@ -352,9 +357,10 @@ hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float
 }
 
 template <typename T>
-hipError_t dinit_t(const ScanShape &s, const void *dt, const float *A, const float *gfin, float *dinit, hipStream_t st) {
+hipError_t dinit_t(const ScanShape &s, const void *dt, const float *A, const float *gfin, const unsigned char *reset,
+                   float *dinit, hipStream_t st) {
     const long long total = (long long)s.B * s.H * s.P * s.N;
-    bwd_dinit_kernel<T><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, gfin, dinit, s, total);
+    bwd_dinit_kernel<T><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, gfin, reset, dinit, s, total);
     return hipGetLastError();
 }
 
@@ -387,9 +393,9 @@ hipError_t launch_bwd_group_sums(const ScanShape &s, int Lrev, int dtype, const 
 
 hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, const float *A, const float *fwd_prev,
                               const float *rev_prev, const float *rev_final, const float *init_t, const float *fwd_final,
-                              const float *dfin_t, double *anchor, hipStream_t st) {
-    return dtype ? anchors_t<__bf16>(s, dt, A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, anchor, st)
-                 : anchors_t<float>(s, dt, A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, anchor, st);
+                              const float *dfin_t, const unsigned char *reset, double *anchor, hipStream_t st) {
+    return dtype ? anchors_t<__bf16>(s, dt, A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, reset, anchor, st)
+                 : anchors_t<float>(s, dt, A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, reset, anchor, st);
 }
 
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
@@ -406,8 +412,8 @@ hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const
 }
 
 hipError_t launch_bwd_dinit(const ScanShape &s, int dtype, const void *dt, const float *A, const float *gfin,
-                            float *dinit, hipStream_t st) {
-    return dtype ? dinit_t<__bf16>(s, dt, A, gfin, dinit, st) : dinit_t<float>(s, dt, A, gfin, dinit, st);
+                            const unsigned char *reset, float *dinit, hipStream_t st) {
+    return dtype ? dinit_t<__bf16>(s, dt, A, gfin, reset, dinit, st) : dinit_t<float>(s, dt, A, gfin, reset, dinit, st);
 }
 
 }  // namespace ssd

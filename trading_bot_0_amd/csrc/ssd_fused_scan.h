@@ -111,7 +111,7 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
            (size_t)waves * ((size_t)fused_scan_xtile_elems(Q) * 2 + (size_t)(5 + Q / 32) * Q * 4 + 64);
 }
 
-template <typename TO, int NK, int QB, int WAVES, bool EARLY>  // N = 16*NK, Q = 32*QB
+template <typename TO, int NK, int QB, int WAVES, bool ADJ>  // N = 16*NK, Q = 32*QB; ADJ: reversed-adjoint mode
 __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_kernel(
     const __bf16 *__restrict__ x, const __bf16 *__restrict__ dt, const float *__restrict__ A,
     const __bf16 *__restrict__ Bm, const __bf16 *__restrict__ Cm, const float *__restrict__ D,
@@ -160,9 +160,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     const T *Cb = Cm + ((size_t)b * s.L * s.G + g) * N;
     // mode 1 (the time-reversed adjoint recurrence): step t decays by the dt of step L - t of a dt tensor of
     // dt_len rows, steps outside it do not decay, and every step's input weighs one instead of dt
-    const int dt_rows = s.mode ? s.dt_len : s.L;
+    const int dt_rows = ADJ ? s.dt_len : s.L;
     const T *dtb = dt + (size_t)b * dt_rows * s.H + h;
-    const unsigned char *rsb = reset ? reset + (size_t)b * s.L : nullptr;  // state restarts, see kResetLog2
+    const unsigned char *rsb = reset ? reset + (size_t)b * dt_rows : nullptr;  // state restarts, see kResetLog2
     TO *yb = y + (size_t)b * s.L * HP + h * s.P + pb * 32;
     const float dh = D ? D[h] : 0.f;
     const double a_h = (double)A[h];
@@ -193,9 +193,18 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         const unsigned dt_off0 = (tv & 63) * EPL * s.H;
         const T *bp = Bb + (size_t)t0 * s.G * N, *cp = Cb + (size_t)t0 * s.G * N;
         const T *xp = xb + (size_t)t0 * HP, *dp = dtb + (size_t)t0 * s.H;
+        auto reset_byte = [&](int e, bool ok) {  // the restart flag that applies at row t0 + lane*EPL + e
+            const int row = t0 + (tv & 63) * EPL + e;
+            if (rsb == nullptr || !ok) return (unsigned char)0;
+            if (ADJ) {  // the restart before forward step L - row cuts the adjoint at this reversed step
+                const int src = s.L - row;
+                return (src >= 1 && src < dt_rows) ? rsb[src] : (unsigned char)0;
+            }
+            return rsb[row];
+        };
         auto dt_bits = [&](int e, bool ok) {  // dt of row t0 + lane*EPL + e as raw bits, zero where it does not apply
             const int row = t0 + (tv & 63) * EPL + e;
-            if (s.mode) {
+            if (ADJ) {
                 const int src = s.L - row;
                 return (ok && src >= 1 && src < dt_rows) ? __builtin_bit_cast(unsigned short, dtb[(size_t)src * s.H])
                                                          : (unsigned short)0;
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
                 dq[e] = dt_bits(e, Q >= 64 || (tv & 63) < Q);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
-                rq[e] = (rsb != nullptr && (Q >= 64 || (tv & 63) < Q)) ? rsb[t0 + (tv & 63) * EPL + e] : (unsigned char)0;
+                rq[e] = reset_byte(e, Q >= 64 || (tv & 63) < Q);
         } else {  // ragged last chunk: rows past the sequence read as zero (dt = 0 makes them no-ops)
 #pragma unroll
             for (int u = 0; u < UBC; ++u) {
@@ -238,7 +247,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
                 dq[e] = dt_bits(e, (tv & 63) * EPL + e < rows);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
-                rq[e] = (rsb != nullptr && (tv & 63) * EPL + e < rows) ? rsb[t0 + (tv & 63) * EPL + e] : (unsigned char)0;
+                rq[e] = reset_byte(e, (tv & 63) * EPL + e < rows);
         }
     };
 
@@ -301,7 +310,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
             for (int e = 0; e < EPL; ++e) {
                 dtv[e] = (float)__builtin_bit_cast(__bf16, dq[e]);
                 run += (double)dtv[e] * a_h - (rq[e] ? kResetDrop : 0.0);
-                if (s.mode) dtv[e] = (t0 + lane * EPL + e < s.L) ? 1.f : 0.f;  // from here on dtv is the input weight
+                if (ADJ) dtv[e] = (t0 + lane * EPL + e < s.L) ? 1.f : 0.f;  // from here on dtv is the input weight
                 cs[e] = run;
             }
             const double excl = wave_inclusive_scan(run) - run;
@@ -347,7 +356,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
                 }
             }
         }
-        if (EARLY && c + 1 < s.nc) prefetch(c + 1);
         block_sync_lds();  // tiles and tables are visible
 
         // ---- phase 1: outputs of this chunk from the state entering it ----
@@ -471,7 +479,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         }
 
         // ---- phase 2: the state leaving this chunk ----
-        if (!EARLY && c + 1 < s.nc) prefetch(c + 1);
+        if (c + 1 < s.nc) prefetch(c + 1);
         const int lane = phase_tid() & 63, half = lane >> 5;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) st[nb] = st[nb] * a_end;
@@ -537,14 +545,24 @@ template <typename TO, int NK, int QB, int WAVES>
 static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
                                const void *Cm, const float *D, const float *init, const unsigned char *reset, void *y,
                                float *final_states, hipStream_t st) {
-    // requesting the next tile's inputs at the top of the tile instead of after phase 1 measured the same
-    // (217.6 us against 218.8 us) for 26 more live registers
-    constexpr bool EARLY = false;
+    // (requesting the next tile's inputs at the top of the tile instead of after phase 1 measured the same,
+    // 217.6 us against 218.8 us, for 26 more live registers)
     const int units = (s.H / s.G) * (s.P / 32);
     const int grid = s.B * s.G * (units / WAVES);
-    fused_scan_kernel<TO, NK, QB, WAVES, EARLY><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-        static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
-        static_cast<const __bf16 *>(Cm), D, init, reset, static_cast<TO *>(y), final_states, s);
+    const __bf16 *xx = static_cast<const __bf16 *>(x), *dd = static_cast<const __bf16 *>(dt);
+    const __bf16 *bb = static_cast<const __bf16 *>(Bm), *cc = static_cast<const __bf16 *>(Cm);
+    if (s.mode != 0) {
+        // the reversed-adjoint mode serves the backward pass, which takes float outputs only
+        if constexpr (sizeof(TO) == 4) {
+            fused_scan_kernel<TO, NK, QB, WAVES, true><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
+                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, s);
+            return hipGetLastError();
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
+    fused_scan_kernel<TO, NK, QB, WAVES, false><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
+        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, s);
     return hipGetLastError();
 }
 

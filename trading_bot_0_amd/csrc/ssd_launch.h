@@ -10,7 +10,8 @@ namespace ssd {
 struct ScanShape {
     int B, L, H, P, N, G, Q, nc;
     // The one-pass kernel only (the staged path takes these as arguments of launch_chunk_cumsum): decays and input
-    // weights of the time-reversed adjoint recurrence, read from a dt tensor of dt_len <= L rows per batch row.
+    // weights of the time-reversed adjoint recurrence, read from a dt tensor (and reset mask) of dt_len <= L rows
+    // per batch row.
     int mode = 0, dt_len = 0;
 };
 
@@ -35,7 +36,8 @@ size_t chunk_scan_lds_bytes(const ScanShape &s, int elem_bytes);
 // mode 0: decays exp(dt_t A) and input weights dt_t (the forward).  mode 1: the time-reversed adjoint
 // recurrence of the backward pass: step t decays by exp(dt_{L-t} A) and every step weighs one; dt then has
 // dt_len <= L rows per batch row (0 = L) and steps whose L-t falls outside 1..dt_len-1 do not decay, so a
-// reversed sequence can carry L - dt_len leading no-op steps that pad it to whole chunks.
+// reversed sequence can carry L - dt_len leading no-op steps that pad it to whole chunks.  reset is then the
+// forward sequence's mask ([B,dt_len]): a restart before forward step L-t cuts the adjoint at reversed step t.
 hipError_t launch_chunk_cumsum(const ScanShape &s, int dtype, const void *dt, const float *A,
                                const unsigned char *reset, float *dtcs, hipStream_t stream, int mode = 0,
                                int dt_len = 0);
@@ -99,10 +101,11 @@ hipError_t launch_bwd_group_sums(const ScanShape &s, int Lrev, int dtype, const 
 // anchor [B,nc+1,H]: q at the first step of chunk c = exp(dt A) <adjoint state, forward state> entering the chunk:
 // fwd_prev [B,nc,H,N,P] are the forward-time transposed scan's chunk states, rev_prev those of the reversed one
 // (chunk nc-c there), rev_final its final state and init_t the transposed initial state (NULL = zero) for c = 0;
-// c = nc is the end of the sequence, <dfin_t, fwd_final> (zero when dfin_t is NULL).
+// c = nc is the end of the sequence, <dfin_t, fwd_final> (zero when dfin_t is NULL).  reset [B,L] or NULL: an
+// anchor is zero where the sequence restarts before the chunk's first step.
 hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, const float *A, const float *fwd_prev,
                               const float *rev_prev, const float *rev_final, const float *init_t, const float *fwd_final,
-                              const float *dfin_t, double *anchor, hipStream_t stream);
+                              const float *dfin_t, const unsigned char *reset, double *anchor, hipStream_t stream);
 // q_t between the anchors of its chunk (chunk <= 64 steps); ddt = e1 + A q; dA_part[b,h] = sum_t dt q,
 // dD_part[b,h] = sum_t dd
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
@@ -112,6 +115,6 @@ hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const f
 hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,
                                 hipStream_t stream);
 hipError_t launch_bwd_dinit(const ScanShape &s, int dtype, const void *dt, const float *A, const float *gfin,
-                            float *dinit, hipStream_t stream);
+                            const unsigned char *reset, float *dinit, hipStream_t stream);
 
 }  // namespace ssd

@@ -43,7 +43,12 @@ __global__ __launch_bounds__(256) void chunk_cumsum_kernel(const T *__restrict__
         tile[h * ldt + l] = v;
     }
     for (int l = threadIdx.x; l < s.Q; l += blockDim.x)
-        drop[l] = (reset != nullptr && t0 + l < s.L && reset[(size_t)b * s.L + t0 + l] != 0) ? (float)kResetDrop : 0.f;
+    {
+        // in mode 1 the restart before step L - t of the forward sequence cuts the adjoint at reversed step t
+        const int t = t0 + l, src = mode == 0 ? t : s.L - t;
+        const bool in = mode == 0 ? t < s.L : (t < s.L && src >= 1 && src < dt_len);
+        drop[l] = (reset != nullptr && in && reset[(size_t)b * (mode == 0 ? s.L : dt_len) + src] != 0) ? (float)kResetDrop : 0.f;
+    }
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     constexpr double kLog2e = 1.4426950408889634;

@@ -103,7 +103,7 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
         lib.ssd_steps_fwd.argtypes = [POINTER(SsdStepDims), c_int64, c_int, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_chunk_scan_bwd_workspace_bytes.argtypes = [POINTER(SsdDims), c_int, POINTER(c_size_t)]
-        lib.ssd_chunk_scan_bwd.argtypes = [POINTER(SsdDims), c_int] + [P] * 17 + [c_size_t, P]
+        lib.ssd_chunk_scan_bwd.argtypes = [POINTER(SsdDims), c_int] + [P] * 18 + [c_size_t, P]
         for name in EXPORTED_SYMBOLS[2:]:
             getattr(lib, name).restype = c_int   # (argument types of the block stages: block.py)
         _lib = lib
@@ -268,9 +268,9 @@ def ssd_chunk_scan(
 
 
 def ssd_chunk_scan_backward(x, dt, A, Bm, Cm, D, dy, chunk: int = 128, initial_states=None, dfinal_states=None,
-                            need_dinitial_states: bool = False, workspace=None) -> dict:
+                            need_dinitial_states: bool = False, workspace=None, reset=None) -> dict:
     """Gradients of the scan's outputs (y weighted by `dy`, the final state by `dfinal_states`) with respect to
-    its inputs.  Returns a dict with dx, ddt, dB, dC (input dtype), dA, dD (None without D) and, if asked for,
+    its inputs; `reset` is the forward's restart mask.  Returns a dict with dx, ddt, dB, dC (input dtype), dA, dD (None without D) and, if asked for,
     dinitial_states (float32)."""
     lib = load_library()
     dims = _scan_dims(x, Bm, chunk)
@@ -291,8 +291,9 @@ def ssd_chunk_scan_backward(x, dt, A, Bm, Cm, D, dy, chunk: int = 128, initial_s
         workspace = torch.empty(need.value, dtype=torch.uint8, device=dev)
     elif (not workspace.is_cuda) or workspace.dtype != torch.uint8 or not workspace.is_contiguous():
         raise ValueError("SSD workspace must be a contiguous uint8 GPU tensor")
+    reset = _reset_mask(reset, dims)
     rc = lib.ssd_chunk_scan_bwd(byref(dims), code, x.data_ptr(), dt.data_ptr(), A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(),
-                                _ptr(D), _ptr(initial_states), dy.data_ptr(), _ptr(dfinal_states),
+                                _ptr(D), _ptr(initial_states), _ptr(reset), dy.data_ptr(), _ptr(dfinal_states),
                                 out["dx"].data_ptr(), out["ddt"].data_ptr(), out["dA"].data_ptr(), out["dB"].data_ptr(),
                                 out["dC"].data_ptr(), _ptr(out["dD"]), _ptr(out["dinitial_states"]),
                                 workspace.data_ptr(), workspace.numel(), _stream_ptr(x))
