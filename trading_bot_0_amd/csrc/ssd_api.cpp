@@ -397,11 +397,23 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     BWD_LAUNCH(ssd::launch_gather_rows(el, x, at(w.x_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather x");
     BWD_LAUNCH(ssd::launch_gather_rows(el, Cm, at(w.c_rev_g), s.B, s.L, Lp, s.G, s.N, 1, true, st), "gather C");
     BWD_LAUNCH(ssd::launch_gather_rows(el, Bm, at(w.b_rev_g), s.B, s.L, Lp, s.G, s.N, 1, true, st), "gather B");
-    BWD_LAUNCH(ssd::launch_gather_rows(el, Cm, at(w.c_rev_h), s.B, s.L, Lp, s.G, s.N, rep, true, st), "gather C per head");
-    const void *b_heads = Bm;
-    if (rep > 1) {
+    // Which scans take the one-pass kernel (it then also writes the state entering every 64-step tile, which is
+    // what the staged kernels leave in their state array).
+    auto one_pass = [&](const ssd::ScanShape &shape) {
+        const int waves = ssd::fused_scan_waves(shape, inner);
+        if (waves == 0 || shape.Q != 64) return false;
+        const int64_t groups = (int64_t)shape.B * shape.G * ((shape.H / shape.G) * (shape.P / 32) / waves);
+        return (waves == 8 && groups >= kOnePassMinWorkgroups) || (waves == 2 && groups >= 4 * kOnePassMinWorkgroups);
+    };
+    // The transposed scans take C (reversed) and B as their x operand, once per head -- unless they run on the
+    // one-pass kernel, which reads an x that groups of heads share in place.
+    const bool shared_x = one_pass(sT);
+    const void *c_heads = at(w.c_rev_g), *b_heads = Bm;
+    if (!shared_x && rep > 1) {
+        BWD_LAUNCH(ssd::launch_gather_rows(el, Cm, at(w.c_rev_h), s.B, s.L, Lp, s.G, s.N, rep, true, st), "gather C per head");
         BWD_LAUNCH(ssd::launch_gather_rows(el, Bm, at(w.b_fwd_h), s.B, s.L, s.L, s.G, s.N, rep, false, st),
                    "gather B per head");
+        c_heads = at(w.c_rev_h);
         b_heads = at(w.b_fwd_h);
     }
     const float *init_t = nullptr, *dfin_t = nullptr;
@@ -413,27 +425,28 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         BWD_LAUNCH(ssd::launch_transpose_state(dfinal_states, atf(w.dfin_t), (long long)s.B * s.H, s.P, s.N, st), "transpose");
         dfin_t = atf(w.dfin_t);
     }
-    // r = g B: the adjoint recurrence, reversed in time; its last state is g_0.  It has the forward's own shape,
-    // so large bf16 batches take the one-pass kernel.
-    if (takes_one_pass(sR, inner)) {
-        ssd::ScanShape f = sR;
-        f.mode = 1;
-        f.dt_len = s.L;
-        BWD_LAUNCH(ssd::launch_fused_scan(f, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states,
-                                          reset, at(w.r_rev), atf(w.gfin), st),
-                   "one-pass adjoint scan");
-    } else if (int rc = run_staged(sR, inner, at(w.dy_rev), dt, A, at(w.c_rev_g), at(w.b_rev_g), nullptr, dfinal_states, reset,
-                                   1, at(w.r_rev), atf(w.gfin), dtcs, states, st, s.L)) {
+    auto scan = [&](const ssd::ScanShape &shape, const void *sx, const void *sb, const void *sc, const float *sinit, int mode,
+                    void *sy, float *sfinal, float *sstates, bool keep_states, int x_groups) -> int {
+        if (one_pass(shape)) {
+            ssd::ScanShape f = shape;
+            f.mode = mode;
+            f.dt_len = s.L;
+            f.x_groups = x_groups;
+            hipError_t err = ssd::launch_fused_scan(f, inner, sx, dt, A, sb, sc, nullptr, sinit, reset, sy, sfinal, st,
+                                                     keep_states ? sstates : nullptr);
+            return err == hipSuccess ? SSD_OK : hip_fail(err, "one-pass scan launch (backward)");
+        }
+        return run_staged(shape, inner, sx, dt, A, sb, sc, nullptr, sinit, reset, mode, sy, sfinal, dtcs, sstates, st, s.L);
+    };
+    // r = g B: the adjoint recurrence, reversed in time; its last state is g_0
+    if (int rc = scan(sR, at(w.dy_rev), at(w.c_rev_g), at(w.b_rev_g), dfinal_states, 1, at(w.r_rev), atf(w.gfin), states, false, 0))
         return rc;
-    }
     // yB = x . g: the same recurrence with the state transposed; its chunk states stay in `states`
-    if (int rc = run_staged(sTR, inner, at(w.c_rev_h), dt, A, at(w.dy_rev), at(w.x_rev), nullptr, dfin_t, reset, 1,
-                            at(w.yb_rev), atf(w.gfin_t), dtcs, states, st, s.L))
+    const int xg = (shared_x && rep > 1) ? s.G : 0;
+    if (int rc = scan(sTR, c_heads, at(w.dy_rev), at(w.x_rev), dfin_t, 1, at(w.yb_rev), atf(w.gfin_t), states, true, xg))
         return rc;
     // yC = dy . h: the forward recurrence with the state transposed; its chunk states go to `states2`
-    if (int rc = run_staged(sT, inner, b_heads, dt, A, x, dy, nullptr, init_t, reset, 0, at(w.yc), atf(w.ffin_t), dtcs,
-                            states2, st))
-        return rc;
+    if (int rc = scan(sT, b_heads, x, dy, init_t, 0, at(w.yc), atf(w.ffin_t), states2, true, xg)) return rc;
     BWD_LAUNCH(ssd::launch_bwd_rows(s, Lp, el, x, dy, dt, Cm, D, atf(w.r_rev), atf(w.yc), dx, atf(w.e1), atf(w.dd), atf(w.u), st),
                "backward rows");
     BWD_LAUNCH(ssd::launch_bwd_group_sums(s, Lp, el, dt, atf(w.yb_rev), atf(w.yc), dB, dC, st), "backward group sums");

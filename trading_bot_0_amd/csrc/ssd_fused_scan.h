@@ -116,7 +116,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     const __bf16 *__restrict__ x, const __bf16 *__restrict__ dt, const float *__restrict__ A,
     const __bf16 *__restrict__ Bm, const __bf16 *__restrict__ Cm, const float *__restrict__ D,
     const float *init, const unsigned char *__restrict__ reset, TO *__restrict__ y, float *final_states,
-    ScanShape s) {
+    float *tile_states, ScanShape s) {
     using T = __bf16;
     constexpr int N = 16 * NK, NB = NK / 2, Q = 32 * QB, nthr = 64 * WAVES;
     constexpr int EPL = Q >= 64 ? Q / 64 : 1;  // chunk positions per lane in the scan
@@ -155,7 +155,11 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     const int h = g * HG + unit / PBn, pb = unit % PBn;
     const int xcol0 = g * HG * s.P + unit0 * 32;  // first element of the workgroup's slice of an x row
     const int HP = s.H * s.P;
-    const T *xb = x + (size_t)b * s.L * HP + xcol0;
+    // x rows: one per timestep, HP wide -- or, when x is shared by groups of heads (s.x_groups, with G == H so
+    // that the workgroup is one head), x_groups * P wide with this head's group's columns
+    const int XLD = s.x_groups ? s.x_groups * s.P : HP;
+    const int xcol = s.x_groups ? (h / (s.H / s.x_groups)) * s.P + (unit0 % PBn) * 32 : xcol0;
+    const T *xb = x + (size_t)b * s.L * XLD + xcol;
     const T *Bb = Bm + ((size_t)b * s.L * s.G + g) * N;
     const T *Cb = Cm + ((size_t)b * s.L * s.G + g) * N;
     // mode 1 (the time-reversed adjoint recurrence): step t decays by the dt of step L - t of a dt tensor of
@@ -189,10 +193,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         const int tv = phase_tid();
         const int bc_row0 = tv / BPR, x_row0 = tv / XPR;
         const unsigned bc_off0 = bc_row0 * s.G * N + (tv % BPR) * 8;
-        const unsigned x_off0 = x_row0 * HP + (tv % XPR) * 8;
+        const unsigned x_off0 = x_row0 * XLD + (tv % XPR) * 8;
         const unsigned dt_off0 = (tv & 63) * EPL * s.H;
         const T *bp = Bb + (size_t)t0 * s.G * N, *cp = Cb + (size_t)t0 * s.G * N;
-        const T *xp = xb + (size_t)t0 * HP, *dp = dtb + (size_t)t0 * s.H;
+        const T *xp = xb + (size_t)t0 * XLD, *dp = dtb + (size_t)t0 * s.H;
         auto reset_byte = [&](int e, bool ok) {  // the restart flag that applies at row t0 + lane*EPL + e
             const int row = t0 + (tv & 63) * EPL + e;
             if (rsb == nullptr || !ok) return (unsigned char)0;
@@ -226,7 +230,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
                 cq[u] = ld16(cp + (size_t)u * BRP * s.G * N + bc_off0, ok);
             }
 #pragma unroll
-            for (int u = 0; u < UX; ++u) xq[u] = *reinterpret_cast<const uint4 *>(xp + (size_t)u * 16 * HP + x_off0);
+            for (int u = 0; u < UX; ++u) xq[u] = *reinterpret_cast<const uint4 *>(xp + (size_t)u * 16 * XLD + x_off0);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
                 dq[e] = dt_bits(e, Q >= 64 || (tv & 63) < Q);
@@ -241,7 +245,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
                 cq[u] = ld16(cp + (size_t)u * BRP * s.G * N + bc_off0, ok);
             }
 #pragma unroll
-            for (int u = 0; u < UX; ++u) xq[u] = ld16(xp + (size_t)u * 16 * HP + x_off0, x_row0 + u * 16 < rows);
+            for (int u = 0; u < UX; ++u) xq[u] = ld16(xp + (size_t)u * 16 * XLD + x_off0, x_row0 + u * 16 < rows);
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
                 dq[e] = dt_bits(e, (tv & 63) * EPL + e < rows);
@@ -268,10 +272,24 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         }
     }
 
+    // this lane's part of the unit's [32 columns, N] block of a [P,N] state
+    auto store_state = [&](float *state_bh) {
+        float *fb = state_bh + (size_t)(pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq)
+                *reinterpret_cast<float4 *>(fb + 32 * nb + 8 * gq) =
+                    make_float4(st[nb][4 * gq], st[nb][4 * gq + 1], st[nb][4 * gq + 2], st[nb][4 * gq + 3]);
+        }
+    };
+
     prefetch(0);
     for (int c = 0; c < s.nc; ++c) {
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
+        // the state entering every tile, for a caller that needs it (the backward pass): [B, nc, H, P, N]
+        if (tile_states) store_state(tile_states + (((size_t)b * s.nc + c) * s.H + h) * s.P * N);
         block_sync_lds();  // every wave is done reading the previous chunk's tiles
         // ---- registers -> LDS tiles ----
         // where the pieces go: the swizzle repeats every 32 rows, so all passes of a thread share the
@@ -526,16 +544,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         }
     }
 
-    if (final_states) {
-        float *fb = final_states + (((size_t)b * s.H + h) * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-            for (int gq = 0; gq < 4; ++gq)
-                *reinterpret_cast<float4 *>(fb + 32 * nb + 8 * gq) =
-                    make_float4(st[nb][4 * gq], st[nb][4 * gq + 1], st[nb][4 * gq + 2], st[nb][4 * gq + 3]);
-        }
-    }
+    if (final_states) store_state(final_states + ((size_t)b * s.H + h) * s.P * N);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -544,7 +553,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 template <typename TO, int NK, int QB, int WAVES>
 static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
                                const void *Cm, const float *D, const float *init, const unsigned char *reset, void *y,
-                               float *final_states, hipStream_t st) {
+                               float *final_states, float *tile_states, hipStream_t st) {
     // (requesting the next tile's inputs at the top of the tile instead of after phase 1 measured the same,
     // 217.6 us against 218.8 us, for 26 more live registers)
     const int units = (s.H / s.G) * (s.P / 32);
@@ -555,32 +564,40 @@ static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt
         // the reversed-adjoint mode serves the backward pass, which takes float outputs only
         if constexpr (sizeof(TO) == 4) {
             fused_scan_kernel<TO, NK, QB, WAVES, true><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, s);
+                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, s);
             return hipGetLastError();
         } else {
             return hipErrorInvalidValue;
         }
     }
     fused_scan_kernel<TO, NK, QB, WAVES, false><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, s);
+        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, s);
     return hipGetLastError();
 }
 
 template <typename TO, int NK, int QB>
 static hipError_t fused_dispatch_w(const ScanShape &s, int waves, const void *x, const void *dt, const float *A,
                                    const void *Bm, const void *Cm, const float *D, const float *init,
-                                   const unsigned char *reset, void *y, float *final_states, hipStream_t st) {
-    return waves == 8 ? fused_launch<TO, NK, QB, 8>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st)
-                      : fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
+                                   const unsigned char *reset, void *y, float *final_states, float *tile_states,
+                                   hipStream_t st) {
+    if (waves == 8) return fused_launch<TO, NK, QB, 8>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
+    if (waves == 4) return fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
+    // two waves: one head of 64 columns with its own B and C (the transposed scans of the backward pass);
+    // the staging offsets fit a 32-wide state only, and only the float-output library instantiates it
+    if constexpr (NK == 2 && sizeof(TO) == 4) {
+        if (waves == 2)
+            return fused_launch<TO, NK, QB, 2>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
+    }
+    return hipErrorInvalidValue;
 }
 
 template <typename TO>
 hipError_t fused_dispatch(const ScanShape &s, int waves, const void *x, const void *dt, const float *A,
                           const void *Bm, const void *Cm, const float *D, const float *init,
-                          const unsigned char *reset, void *y, float *final_states, hipStream_t st) {
+                          const unsigned char *reset, void *y, float *final_states, float *tile_states, hipStream_t st) {
 #define SSD_FUSED_CASE(NKv, QBv) \
     if (s.N == 16 * NKv && s.Q == 32 * QBv) \
-        return fused_dispatch_w<TO, NKv, QBv>(s, waves, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
+        return fused_dispatch_w<TO, NKv, QBv>(s, waves, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
     SSD_FUSED_CASE(2, kOnePassTile / 32)
     SSD_FUSED_CASE(4, kOnePassTile / 32)
 #undef SSD_FUSED_CASE

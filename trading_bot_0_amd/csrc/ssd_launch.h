@@ -13,6 +13,9 @@ struct ScanShape {
     // weights of the time-reversed adjoint recurrence, read from a dt tensor (and reset mask) of dt_len <= L rows
     // per batch row.
     int mode = 0, dt_len = 0;
+    // The one-pass kernel only, shapes with B and C per head (G == H): x is given once per x_groups groups of
+    // heads, as a [B, L, x_groups, P] tensor, instead of once per head (0 = per head, [B, L, H, P]).
+    int x_groups = 0;
 };
 
 struct StepShape {
@@ -55,10 +58,12 @@ hipError_t launch_chunk_scan(const ScanShape &s, int dtype, const void *x, const
                              void *y, hipStream_t stream);
 // The whole forward in one pass (bf16 inputs): no workspace, nothing but x, dt, B, C read and y, final written.
 // fused_scan_waves is 0 when the shape cannot run there, else the waves per workgroup it would use.
+// tile_states (optional, [B, ceil(L/64), H, P, N]): the state entering every tile of 64 steps.
 int fused_scan_waves(const ScanShape &s, int dtype);
 hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const void *dt, const float *A,
                              const void *Bm, const void *Cm, const float *D, const float *init,
-                             const unsigned char *reset, void *y, float *final_states, hipStream_t stream);
+                             const unsigned char *reset, void *y, float *final_states, hipStream_t stream,
+                             float *tile_states = nullptr);
 hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *x, const void *dt,
                        const float *A, const void *Bm, const void *Cm, const float *D, void *y,
                        hipStream_t stream);
