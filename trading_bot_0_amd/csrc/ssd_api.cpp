@@ -392,29 +392,33 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     sR.L = Lp;
     sTR.L = Lp;
     float *states2 = atf(w.states2);
-    // operands: time-reversed dy, x, C, B; C (reversed) and B (forward) once per head for the transposed scans
-    BWD_LAUNCH(ssd::launch_gather_rows(el, dy, at(w.dy_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather dy");
-    BWD_LAUNCH(ssd::launch_gather_rows(el, x, at(w.x_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather x");
-    BWD_LAUNCH(ssd::launch_gather_rows(el, Cm, at(w.c_rev_g), s.B, s.L, Lp, s.G, s.N, 1, true, st), "gather C");
-    BWD_LAUNCH(ssd::launch_gather_rows(el, Bm, at(w.b_rev_g), s.B, s.L, Lp, s.G, s.N, 1, true, st), "gather B");
-    // Which scans take the one-pass kernel (it then also writes the state entering every 64-step tile, which is
-    // what the staged kernels leave in their state array).
+    // Which scans take the one-pass kernel.  It reverses time itself (reads the forward tensors, writes its output
+    // in forward order), reads an x that a group's heads share in place and writes the state entering every
+    // 64-step tile, which is what the staged kernels leave in their state array.  The staged kernels get their
+    // operands gathered: time-reversed copies, and one copy of a group's B or C per head.
     auto one_pass = [&](const ssd::ScanShape &shape) {
         const int waves = ssd::fused_scan_waves(shape, inner);
         if (waves == 0 || shape.Q != 64) return false;
         const int64_t groups = (int64_t)shape.B * shape.G * ((shape.H / shape.G) * (shape.P / 32) / waves);
         return (waves == 8 && groups >= kOnePassMinWorkgroups) || (waves == 2 && groups >= 4 * kOnePassMinWorkgroups);
     };
-    // The transposed scans take C (reversed) and B as their x operand, once per head -- unless they run on the
-    // one-pass kernel, which reads an x that groups of heads share in place.
-    const bool shared_x = one_pass(sT);
-    const void *c_heads = at(w.c_rev_g), *b_heads = Bm;
-    if (!shared_x && rep > 1) {
+    const bool fast_r = one_pass(sR), fast_t = one_pass(sT);
+    const void *c_heads = Cm, *b_heads = Bm;
+    if (!fast_r || !fast_t)
+        BWD_LAUNCH(ssd::launch_gather_rows(el, dy, at(w.dy_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather dy");
+    if (!fast_r) {
+        BWD_LAUNCH(ssd::launch_gather_rows(el, Cm, at(w.c_rev_g), s.B, s.L, Lp, s.G, s.N, 1, true, st), "gather C");
+        BWD_LAUNCH(ssd::launch_gather_rows(el, Bm, at(w.b_rev_g), s.B, s.L, Lp, s.G, s.N, 1, true, st), "gather B");
+    }
+    if (!fast_t) {
+        BWD_LAUNCH(ssd::launch_gather_rows(el, x, at(w.x_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather x");
         BWD_LAUNCH(ssd::launch_gather_rows(el, Cm, at(w.c_rev_h), s.B, s.L, Lp, s.G, s.N, rep, true, st), "gather C per head");
-        BWD_LAUNCH(ssd::launch_gather_rows(el, Bm, at(w.b_fwd_h), s.B, s.L, s.L, s.G, s.N, rep, false, st),
-                   "gather B per head");
         c_heads = at(w.c_rev_h);
-        b_heads = at(w.b_fwd_h);
+        if (rep > 1) {
+            BWD_LAUNCH(ssd::launch_gather_rows(el, Bm, at(w.b_fwd_h), s.B, s.L, s.L, s.G, s.N, rep, false, st),
+                       "gather B per head");
+            b_heads = at(w.b_fwd_h);
+        }
     }
     const float *init_t = nullptr, *dfin_t = nullptr;
     if (initial_states != nullptr) {
@@ -425,9 +429,9 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         BWD_LAUNCH(ssd::launch_transpose_state(dfinal_states, atf(w.dfin_t), (long long)s.B * s.H, s.P, s.N, st), "transpose");
         dfin_t = atf(w.dfin_t);
     }
-    auto scan = [&](const ssd::ScanShape &shape, const void *sx, const void *sb, const void *sc, const float *sinit, int mode,
-                    void *sy, float *sfinal, float *sstates, bool keep_states, int x_groups) -> int {
-        if (one_pass(shape)) {
+    auto scan = [&](const ssd::ScanShape &shape, bool fast, const void *sx, const void *sb, const void *sc, const float *sinit,
+                    int mode, void *sy, float *sfinal, float *sstates, bool keep_states, int x_groups) -> int {
+        if (fast) {
             ssd::ScanShape f = shape;
             f.mode = mode;
             f.dt_len = s.L;
@@ -439,17 +443,23 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         return run_staged(shape, inner, sx, dt, A, sb, sc, nullptr, sinit, reset, mode, sy, sfinal, dtcs, sstates, st, s.L);
     };
     // r = g B: the adjoint recurrence, reversed in time; its last state is g_0
-    if (int rc = scan(sR, at(w.dy_rev), at(w.c_rev_g), at(w.b_rev_g), dfinal_states, 1, at(w.r_rev), atf(w.gfin), states, false, 0))
+    if (int rc = fast_r ? scan(sR, true, dy, Cm, Bm, dfinal_states, 1, at(w.r_rev), atf(w.gfin), states, false, 0)
+                        : scan(sR, false, at(w.dy_rev), at(w.c_rev_g), at(w.b_rev_g), dfinal_states, 1, at(w.r_rev),
+                               atf(w.gfin), states, false, 0))
         return rc;
     // yB = x . g: the same recurrence with the state transposed; its chunk states stay in `states`
-    const int xg = (shared_x && rep > 1) ? s.G : 0;
-    if (int rc = scan(sTR, c_heads, at(w.dy_rev), at(w.x_rev), dfin_t, 1, at(w.yb_rev), atf(w.gfin_t), states, true, xg))
+    const int xg = (fast_t && rep > 1) ? s.G : 0;
+    if (int rc = fast_t ? scan(sTR, true, Cm, dy, x, dfin_t, 1, at(w.yb_rev), atf(w.gfin_t), states, true, xg)
+                        : scan(sTR, false, c_heads, at(w.dy_rev), at(w.x_rev), dfin_t, 1, at(w.yb_rev), atf(w.gfin_t),
+                               states, true, 0))
         return rc;
     // yC = dy . h: the forward recurrence with the state transposed; its chunk states go to `states2`
-    if (int rc = scan(sT, b_heads, x, dy, init_t, 0, at(w.yc), atf(w.ffin_t), states2, true, xg)) return rc;
-    BWD_LAUNCH(ssd::launch_bwd_rows(s, Lp, el, x, dy, dt, Cm, D, atf(w.r_rev), atf(w.yc), dx, atf(w.e1), atf(w.dd), atf(w.u), st),
+    if (int rc = scan(sT, fast_t, b_heads, x, dy, init_t, 0, at(w.yc), atf(w.ffin_t), states2, true, xg)) return rc;
+    BWD_LAUNCH(ssd::launch_bwd_rows(s, fast_r ? 0 : Lp, el, x, dy, dt, Cm, D, atf(w.r_rev), atf(w.yc), dx, atf(w.e1), atf(w.dd),
+                                    atf(w.u), st),
                "backward rows");
-    BWD_LAUNCH(ssd::launch_bwd_group_sums(s, Lp, el, dt, atf(w.yb_rev), atf(w.yc), dB, dC, st), "backward group sums");
+    BWD_LAUNCH(ssd::launch_bwd_group_sums(s, fast_t ? 0 : Lp, el, dt, atf(w.yb_rev), atf(w.yc), dB, dC, st),
+               "backward group sums");
     double *anchor = reinterpret_cast<double *>(base + w.anchor);
     BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, reset, anchor,
                                        st),

@@ -90,7 +90,8 @@ __global__ __launch_bounds__(256) void transpose_state_kernel(const float *__res
 
 // Eight lanes per (b, t, h), one 8-element piece of a row each (headdim and dstate are at most 64):
 // dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1; the three dot products are summed over the
-// eight lanes.  r_rev is the reversed scan's float output (time reversed), yC the forward-time transposed scan's.
+// eight lanes.  r_rev is the reversed scan's float output (row Lrev-1-t of Lrev rows holds timestep t; Lrev = 0:
+// already in forward order), yC the forward-time transposed scan's.
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                                                        const T *__restrict__ dt, const T *__restrict__ Cm,
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, 
     float se1 = 0.f, sdd = 0.f, sc = 0.f;
     if (piece < s.P) {
         const size_t row = (size_t)gid * s.P + piece;
-        const size_t rrow = ((size_t)(b * Lrev + (Lrev - 1 - t)) * s.H + h) * s.P + piece;
+        const size_t rrow = (Lrev ? ((size_t)(b * Lrev + (Lrev - 1 - t)) * s.H + h) * s.P : (size_t)gid * s.P) + piece;
         const Row8<T> xv = Row8<T>::load(x + row), dv = Row8<T>::load(dy + row);
         const Row8<float> rv = Row8<float>::load(r_rev + rrow);
         Row8<T> o;
@@ -162,7 +163,8 @@ __global__ __launch_bounds__(256) void bwd_group_sums_kernel(const T *__restrict
     for (int k = 0; k < hpg; ++k) {
         const int h = g * hpg + k;
         const float dtv = (float)dt[(size_t)bt * s.H + h];
-        const Row8<float> vb = Row8<float>::load(yB_rev + ((size_t)(b * Lrev + (Lrev - 1 - t)) * s.H + h) * s.N + n);
+        const size_t brow = Lrev ? (size_t)(b * Lrev + (Lrev - 1 - t)) : (size_t)bt;
+        const Row8<float> vb = Row8<float>::load(yB_rev + (brow * s.H + h) * s.N + n);
         const Row8<float> vc = Row8<float>::load(yC + ((size_t)bt * s.H + h) * s.N + n);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {

@@ -159,15 +159,18 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     // that the workgroup is one head), x_groups * P wide with this head's group's columns
     const int XLD = s.x_groups ? s.x_groups * s.P : HP;
     const int xcol = s.x_groups ? (h / (s.H / s.x_groups)) * s.P + (unit0 % PBn) * 32 : xcol0;
-    const T *xb = x + (size_t)b * s.L * XLD + xcol;
-    const T *Bb = Bm + ((size_t)b * s.L * s.G + g) * N;
-    const T *Cb = Cm + ((size_t)b * s.L * s.G + g) * N;
+    // ADJ: x, B, C, dt, the reset mask and y are the forward sequence's tensors, dt_len rows per batch row, and row
+    // tau of the scan is their row L - 1 - tau (rows outside them are no-op steps in front of the reversed sequence)
+    const int trows = ADJ ? s.dt_len : s.L;
+    const T *xb = x + (size_t)b * trows * XLD + xcol;
+    const T *Bb = Bm + ((size_t)b * trows * s.G + g) * N;
+    const T *Cb = Cm + ((size_t)b * trows * s.G + g) * N;
     // mode 1 (the time-reversed adjoint recurrence): step t decays by the dt of step L - t of a dt tensor of
     // dt_len rows, steps outside it do not decay, and every step's input weighs one instead of dt
     const int dt_rows = ADJ ? s.dt_len : s.L;
     const T *dtb = dt + (size_t)b * dt_rows * s.H + h;
     const unsigned char *rsb = reset ? reset + (size_t)b * dt_rows : nullptr;  // state restarts, see kResetLog2
-    TO *yb = y + (size_t)b * s.L * HP + h * s.P + pb * 32;
+    TO *yb = y + (size_t)b * trows * HP + h * s.P + pb * 32;
     const float dh = D ? D[h] : 0.f;
     const double a_h = (double)A[h];
 
@@ -222,7 +225,25 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
             if (ok) v = *reinterpret_cast<const uint4 *>(ptr);
             return v;
         };
-        if (rows == Q) {
+        if (ADJ) {
+            const int first = s.L - 1 - t0;  // the tensors' row of this tile's first row; later rows count down
+#pragma unroll
+            for (int u = 0; u < UBC; ++u) {
+                const int src = first - (bc_row0 + u * BRP);
+                const bool ok = (BSL % nthr == 0 || tv + u * nthr < BSL) && src >= 0 && src < trows;
+                bq[u] = ld16(Bb + (size_t)src * s.G * N + (tv % BPR) * 8, ok);
+                cq[u] = ld16(Cb + (size_t)src * s.G * N + (tv % BPR) * 8, ok);
+            }
+#pragma unroll
+            for (int u = 0; u < UX; ++u) {
+                const int src = first - (x_row0 + u * 16);
+                xq[u] = ld16(xb + (size_t)src * XLD + (tv % XPR) * 8, src >= 0 && src < trows);
+            }
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) dq[e] = dt_bits(e, (tv & 63) * EPL + e < rows);
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) rq[e] = reset_byte(e, (tv & 63) * EPL + e < rows);
+        } else if (rows == Q) {
 #pragma unroll
             for (int u = 0; u < UBC; ++u) {
                 const bool ok = BSL % nthr == 0 || tv + u * nthr < BSL;
@@ -491,7 +512,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 #pragma unroll
                         for (int i = 0; i < 4; ++i) o[vg * 4 + i] = acc[vg * 4 + i] + dh * (float)x4[i];
                     }
-                    store_column<TO>(yb + (size_t)(t0 + ll) * HP, o, he, 32, ll < rows);
+                    const int yrow = ADJ ? s.L - 1 - (t0 + ll) : t0 + ll;
+                    store_column<TO>(yb + (size_t)yrow * HP, o, he, 32, ll < rows && (!ADJ || (yrow >= 0 && yrow < trows)));
                 }
             }
         }

@@ -10,8 +10,9 @@ namespace ssd {
 struct ScanShape {
     int B, L, H, P, N, G, Q, nc;
     // The one-pass kernel only (the staged path takes these as arguments of launch_chunk_cumsum): decays and input
-    // weights of the time-reversed adjoint recurrence, read from a dt tensor (and reset mask) of dt_len <= L rows
-    // per batch row.
+    // weights of the time-reversed adjoint recurrence.  All tensors are then the forward sequence's, dt_len <= L
+    // rows per batch row: the kernel reads x, B, C at row L-1-t for its step t and writes y there (rows outside
+    // the tensors are no-op steps), dt and the reset mask at row L-t.
     int mode = 0, dt_len = 0;
     // The one-pass kernel only, shapes with B and C per head (G == H): x is given once per x_groups groups of
     // heads, as a [B, L, x_groups, P] tensor, instead of once per head (0 = per head, [B, L, H, P]).
@@ -96,7 +97,7 @@ hipError_t launch_gather_rows(int dtype, const void *src, void *dst, int B, int 
 // [BH, P, N] -> [BH, N, P]
 hipError_t launch_transpose_state(const float *src, float *dst, long long BH, int P, int N, hipStream_t stream);
 // per (b,t,h): dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1.  r_rev (and yB_rev below) hold
-// Lrev >= L rows per batch row, row Lrev-1-t for timestep t.
+// Lrev >= L rows per batch row, row Lrev-1-t for timestep t; Lrev = 0: L rows in forward order.
 hipError_t launch_bwd_rows(const ScanShape &s, int Lrev, int dtype, const void *x, const void *dy, const void *dt, const void *Cm,
                            const float *D, const float *r_rev, const float *yC, void *dx, float *e1, float *dd,
                            float *u, hipStream_t stream);
