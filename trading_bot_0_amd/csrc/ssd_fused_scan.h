@@ -36,6 +36,9 @@
 #pragma once
 #include "ssd_device.h"
 
+#ifndef SSD_EARLY_W2
+#define SSD_EARLY_W2 1
+#endif
 namespace ssd {
 
 template <int COLS> struct ChunkTile {  // bf16 [rows][COLS], COLS = 32 or 64
@@ -187,6 +190,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         if (kRecomputeOffsets) asm volatile("" : "+v"(t));
         return t;
     };
+    // When the next tile's inputs are requested: after phase 1 (they are then in flight during phase 2 only, but
+    // hold no registers through phase 1), or, for the two-wave workgroups, whose per-head B and C rows are short
+    // and slow to arrive, before phase 1.
+    constexpr bool kEarlyPrefetch = SSD_EARLY_W2 && WAVES == 2;
     uint4 bq[UBC], cq[UBC], xq[UX];
     unsigned short dq[EPL];
     unsigned char rq[EPL];
@@ -395,6 +402,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
                 }
             }
         }
+        if (kEarlyPrefetch && c + 1 < s.nc) prefetch(c + 1);
         block_sync_lds();  // tiles and tables are visible
 
         // ---- phase 1: outputs of this chunk from the state entering it ----
@@ -519,7 +527,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
         }
 
         // ---- phase 2: the state leaving this chunk ----
-        if (c + 1 < s.nc) prefetch(c + 1);
+        if (!kEarlyPrefetch && c + 1 < s.nc) prefetch(c + 1);
         const int lane = phase_tid() & 63, half = lane >> 5;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) st[nb] = st[nb] * a_end;
