@@ -63,6 +63,7 @@ SHAPES = [
     Workload("bwd_groups", 3, 77, 4, 16, 16, 2, 64, init_std=0.5),
     Workload("bwd_per_head_bc", 2, 256, 4, 64, 32, 4, 32, init_std=0.5),
     Workload("bwd_tiny_state", 2, 130, 2, 16, 64, 1, 64, init_std=0.5),
+    Workload("bwd_three_heads_per_group", 2, 100, 6, 32, 32, 2, 64, init_std=0.5),   # group sums in their own kernel
 ]
 
 

@@ -455,11 +455,17 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         return rc;
     // yC = dy . h: the forward recurrence with the state transposed; its chunk states go to `states2`
     if (int rc = scan(sT, fast_t, b_heads, x, dy, init_t, 0, at(w.yc), atf(w.ffin_t), states2, true, xg)) return rc;
-    BWD_LAUNCH(ssd::launch_bwd_rows(s, fast_r ? 0 : Lp, el, x, dy, dt, Cm, D, atf(w.r_rev), atf(w.yc), dx, atf(w.e1), atf(w.dd),
-                                    atf(w.u), st),
-               "backward rows");
-    BWD_LAUNCH(ssd::launch_bwd_group_sums(s, fast_t ? 0 : Lp, el, dt, atf(w.yb_rev), atf(w.yc), dB, dC, st),
-               "backward group sums");
+    if (ssd::bwd_rows_can_sum(s)) {  // dB and dC in the same pass
+        BWD_LAUNCH(ssd::launch_bwd_rows(s, fast_r ? 0 : Lp, el, x, dy, dt, Cm, D, atf(w.r_rev), atf(w.yc), dx, atf(w.e1),
+                                        atf(w.dd), atf(w.u), st, atf(w.yb_rev), fast_t ? 0 : Lp, dB, dC),
+                   "backward rows");
+    } else {
+        BWD_LAUNCH(ssd::launch_bwd_rows(s, fast_r ? 0 : Lp, el, x, dy, dt, Cm, D, atf(w.r_rev), atf(w.yc), dx, atf(w.e1),
+                                        atf(w.dd), atf(w.u), st),
+                   "backward rows");
+        BWD_LAUNCH(ssd::launch_bwd_group_sums(s, fast_t ? 0 : Lp, el, dt, atf(w.yb_rev), atf(w.yc), dB, dC, st),
+                   "backward group sums");
+    }
     double *anchor = reinterpret_cast<double *>(base + w.anchor);
     BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, reset, anchor,
                                        st),

@@ -92,13 +92,17 @@ __global__ __launch_bounds__(256) void transpose_state_kernel(const float *__res
 // dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1; the three dot products are summed over the
 // eight lanes.  r_rev is the reversed scan's float output (row Lrev-1-t of Lrev rows holds timestep t; Lrev = 0:
 // already in forward order), yC the forward-time transposed scan's.
-template <typename T>
+// SUMS: the same pass also sums dt yB and yC over the heads of a group into dB and dC (a group's heads are
+// adjacent rows, i.e. adjacent blocks of eight lanes of one wave: H/G must be 1, 2, 4 or 8), so that yC is read
+// once; otherwise bwd_group_sums_kernel does that.
+template <typename T, bool SUMS>
 __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                                                        const T *__restrict__ dt, const T *__restrict__ Cm,
                                                        const float *__restrict__ D, const float *__restrict__ r_rev,
-                                                       const float *__restrict__ yC, T *__restrict__ dx,
-                                                       float *__restrict__ e1, float *__restrict__ dd,
-                                                       float *__restrict__ u, ScanShape s, int Lrev, long long total) {
+                                                       const float *__restrict__ yC, const float *__restrict__ yB_rev,
+                                                       T *__restrict__ dx, float *__restrict__ e1, float *__restrict__ dd,
+                                                       float *__restrict__ u, T *__restrict__ dB, T *__restrict__ dC,
+                                                       ScanShape s, int Lrev, int LrevB, long long total) {
     const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const long long gid = tid >> 3;  // the row; whole groups of eight lanes leave together
     if (gid >= total) return;
@@ -124,11 +128,40 @@ __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, 
         }
         o.store(dx + row);
     }
+    Row8<float> sb, sy;  // this head's dt yB and yC pieces
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sb.v[i] = sy.v[i] = 0.f;
     if (piece < s.N) {
         const Row8<T> cv = Row8<T>::load(Cm + ((size_t)bt * s.G + g) * s.N + piece);
-        const Row8<float> yv = Row8<float>::load(yC + (size_t)gid * s.N + piece);
+        sy = Row8<float>::load(yC + (size_t)gid * s.N + piece);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) sc += cv.v[i] * yv.v[i];
+        for (int i = 0; i < 8; ++i) sc += cv.v[i] * sy.v[i];
+        if (SUMS) {
+            const size_t brow = LrevB ? (size_t)(b * LrevB + (LrevB - 1 - t)) : (size_t)bt;
+            sb = Row8<float>::load(yB_rev + (brow * s.H + h) * s.N + piece);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sb.v[i] *= dtv;
+        }
+    }
+    if (SUMS) {
+        const int hpg = s.H / s.G;
+        for (int m = 8; m < 8 * hpg; m <<= 1) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                sb.v[i] += __shfl_xor(sb.v[i], m, 64);
+                sy.v[i] += __shfl_xor(sy.v[i], m, 64);
+            }
+        }
+        if (h % hpg == 0 && piece < s.N) {
+            Row8<T> ob, oc;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                ob.v[i] = sb.v[i];
+                oc.v[i] = sy.v[i];
+            }
+            ob.store(dB + ((size_t)bt * s.G + g) * s.N + piece);
+            oc.store(dC + ((size_t)bt * s.G + g) * s.N + piece);
+        }
     }
 #pragma unroll
     for (int m = 1; m < 8; m <<= 1) {
@@ -321,11 +354,18 @@ hipError_t gather_t(const void *src, void *dst, int B, int Lsrc, int L, int grou
 
 template <typename T>
 hipError_t rows_t(const ScanShape &s, int Lrev, const void *x, const void *dy, const void *dt, const void *Cm, const float *D,
-                  const float *r_rev, const float *yC, void *dx, float *e1, float *dd, float *u, hipStream_t st) {
+                  const float *r_rev, const float *yC, void *dx, float *e1, float *dd, float *u, const float *yB_rev,
+                  int LrevB, void *dB, void *dC, hipStream_t st) {
     const long long total = (long long)s.B * s.L * s.H;
-    bwd_rows_kernel<T><<<dim3(blocks_for(total * 8)), dim3(256), 0, st>>>(
-        static_cast<const T *>(x), static_cast<const T *>(dy), static_cast<const T *>(dt), static_cast<const T *>(Cm), D,
-        r_rev, yC, static_cast<T *>(dx), e1, dd, u, s, Lrev, total);
+    const T *xx = static_cast<const T *>(x), *yy = static_cast<const T *>(dy), *tt = static_cast<const T *>(dt);
+    const T *cc = static_cast<const T *>(Cm);
+    if (yB_rev != nullptr)
+        bwd_rows_kernel<T, true><<<dim3(blocks_for(total * 8)), dim3(256), 0, st>>>(
+            xx, yy, tt, cc, D, r_rev, yC, yB_rev, static_cast<T *>(dx), e1, dd, u, static_cast<T *>(dB), static_cast<T *>(dC), s,
+            Lrev, LrevB, total);
+    else
+        bwd_rows_kernel<T, false><<<dim3(blocks_for(total * 8)), dim3(256), 0, st>>>(
+            xx, yy, tt, cc, D, r_rev, yC, nullptr, static_cast<T *>(dx), e1, dd, u, nullptr, nullptr, s, Lrev, 0, total);
     return hipGetLastError();
 }
 
@@ -380,11 +420,17 @@ hipError_t launch_transpose_state(const float *src, float *dst, long long BH, in
     return hipGetLastError();
 }
 
+bool bwd_rows_can_sum(const ScanShape &s) {
+    const int hpg = s.H / s.G;
+    return hpg == 1 || hpg == 2 || hpg == 4 || hpg == 8;
+}
+
 hipError_t launch_bwd_rows(const ScanShape &s, int Lrev, int dtype, const void *x, const void *dy, const void *dt,
                            const void *Cm, const float *D, const float *r_rev, const float *yC, void *dx, float *e1,
-                           float *dd, float *u, hipStream_t st) {
-    return dtype ? rows_t<__bf16>(s, Lrev, x, dy, dt, Cm, D, r_rev, yC, dx, e1, dd, u, st)
-                 : rows_t<float>(s, Lrev, x, dy, dt, Cm, D, r_rev, yC, dx, e1, dd, u, st);
+                           float *dd, float *u, hipStream_t st, const float *yB_rev, int LrevB, void *dB, void *dC) {
+    if (yB_rev != nullptr && !bwd_rows_can_sum(s)) return hipErrorInvalidValue;
+    return dtype ? rows_t<__bf16>(s, Lrev, x, dy, dt, Cm, D, r_rev, yC, dx, e1, dd, u, yB_rev, LrevB, dB, dC, st)
+                 : rows_t<float>(s, Lrev, x, dy, dt, Cm, D, r_rev, yC, dx, e1, dd, u, yB_rev, LrevB, dB, dC, st);
 }
 
 hipError_t launch_bwd_group_sums(const ScanShape &s, int Lrev, int dtype, const void *dt, const float *yB_rev,

@@ -98,9 +98,13 @@ hipError_t launch_gather_rows(int dtype, const void *src, void *dst, int B, int 
 hipError_t launch_transpose_state(const float *src, float *dst, long long BH, int P, int N, hipStream_t stream);
 // per (b,t,h): dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1.  r_rev (and yB_rev below) hold
 // Lrev >= L rows per batch row, row Lrev-1-t for timestep t; Lrev = 0: L rows in forward order.
+// With yB_rev (LrevB rows, as Lrev) the same pass also writes dB and dC, the sums over a group's heads of dt yB
+// and yC (what launch_bwd_group_sums does otherwise); bwd_rows_can_sum: nheads/ngroups is 1, 2, 4 or 8.
+bool bwd_rows_can_sum(const ScanShape &s);
 hipError_t launch_bwd_rows(const ScanShape &s, int Lrev, int dtype, const void *x, const void *dy, const void *dt, const void *Cm,
                            const float *D, const float *r_rev, const float *yC, void *dx, float *e1, float *dd,
-                           float *u, hipStream_t stream);
+                           float *u, hipStream_t stream, const float *yB_rev = nullptr, int LrevB = 0,
+                           void *dB = nullptr, void *dC = nullptr);
 // dB = sum over a group's heads of dt yB (yB_rev time-reversed), dC = the same of yC
 hipError_t launch_bwd_group_sums(const ScanShape &s, int Lrev, int dtype, const void *dt, const float *yB_rev, const float *yC,
                                  void *dB, void *dC, hipStream_t stream);
