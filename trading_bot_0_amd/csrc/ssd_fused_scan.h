@@ -36,9 +36,6 @@
 #pragma once
 #include "ssd_device.h"
 
-#ifndef SSD_EARLY_W2
-#define SSD_EARLY_W2 1
-#endif
 namespace ssd {
 
 template <int COLS> struct ChunkTile {  // bf16 [rows][COLS], COLS = 32 or 64
@@ -193,7 +190,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     // When the next tile's inputs are requested: after phase 1 (they are then in flight during phase 2 only, but
     // hold no registers through phase 1), or, for the two-wave workgroups, whose per-head B and C rows are short
     // and slow to arrive, before phase 1.
-    constexpr bool kEarlyPrefetch = SSD_EARLY_W2 && WAVES == 2;
+    constexpr bool kEarlyPrefetch = WAVES == 2;
     uint4 bq[UBC], cq[UBC], xq[UX];
     unsigned short dq[EPL];
     unsigned char rq[EPL];
