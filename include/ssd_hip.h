@@ -117,7 +117,7 @@ int ssd_chunk_state_passing_fwd(const ssd_dims *dims, int dtype, const void *x, 
  * is needed and nothing but x, dt, B, C is read and y, final_states written.  Same arguments (with the
  * optional reset mask of ssd_chunk_scan_reset_fwd) and results as ssd_chunk_scan_fwd.  Parallel over
  * (batch, head) sequences only; ssd_chunk_scan_fwd takes this path by itself when there are enough of them.  SSD_ERR_UNSUPPORTED unless dtype is bf16 (1 or 2), headdim is a
- * multiple of 32, dstate is 32 or 64 and (nheads/ngroups)*(headdim/32) is a multiple of 4.  dims->chunk must
+ * multiple of 32, dstate is 32, 64 or 128 and (nheads/ngroups)*(headdim/32) is a multiple of 4.  dims->chunk must
  * be a valid chunk length but does not enter: with no workspace layout to honour, the kernel tiles time by
  * its own block of 64 steps (results agree with every chunk length to rounding).  Replaces the same slot as ssd_chunk_scan_fwd (model/trading_model.rs:589-606). */
 int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,

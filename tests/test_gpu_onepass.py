@@ -49,6 +49,8 @@ SHAPES = {
     "short_chunk": (2, 512, 8, 32, 64, 1, 64),
     "small_state_short_chunk": (3, 256, 4, 32, 32, 1, 64),   # N=32, 4 waves
     "many_units": (1, 384, 16, 64, 64, 2, 128),      # 16 units per group: two workgroups per (batch, group)
+    "wide_state": (2, 320, 8, 32, 128, 1, 128),      # N=128: four waves, one per SIMD
+    "long_lookback_heads": (1, 300, 16, 64, 128, 2, 256),   # the long-lookback workload's head sizes, ragged length
 }
 
 
@@ -112,7 +114,7 @@ def test_unsupported_shapes_are_refused():
     cases = [
         WORKLOADS["plumbing_f32"],                                  # float32 inputs
         Workload("p16", 2, 128, 8, 16, 64, 1, 128),                 # headdim not a multiple of 32
-        Workload("n128", 2, 256, 8, 32, 128, 1, 128),               # state too wide for the accumulators
+        Workload("n16", 2, 256, 8, 32, 16, 1, 128),                 # state narrower than an MFMA tile
         Workload("units2", 2, 128, 2, 32, 64, 1, 128),              # 2 units per group
     ]
     for w in cases:

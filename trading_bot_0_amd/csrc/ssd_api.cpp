@@ -112,7 +112,9 @@ Workspace carve(const ssd::ScanShape &s) {
 }
 
 bool takes_one_pass(const ssd::ScanShape &s, int dtype) {
-    return ssd::fused_scan_waves(s, dtype) == 8 && (int64_t)s.B * s.H * (s.P / 32) / 8 >= kOnePassMinWorkgroups;
+    const int waves = ssd::fused_scan_waves(s, dtype);
+    const int full = s.N == 128 ? 4 : 8;  // waves of a workgroup that fills a CU
+    return waves == full && (int64_t)s.B * s.H * (s.P / 32) / full >= kOnePassMinWorkgroups;
 }
 
 int hip_fail(hipError_t e, const char *what) {

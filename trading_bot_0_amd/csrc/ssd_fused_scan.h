@@ -38,14 +38,18 @@
 
 namespace ssd {
 
-template <int COLS> struct ChunkTile {  // bf16 [rows][COLS], COLS = 32 or 64
-    static_assert(COLS == 32 || COLS == 64, "tile rows are 64 or 128 bytes");
+template <int COLS> struct ChunkTile {  // bf16 [rows][COLS], COLS = 32, 64 or 128
+    static_assert(COLS == 32 || COLS == 64 || COLS == 128, "tile rows are 64, 128 or 256 bytes");
     // XOR mask on the index of an 8-byte piece within its row.  32 consecutive rows map a fixed logical
     // piece to 32 different bank pairs, and 4 consecutive rows (first one a multiple of 4) keep their
     // 64-byte halves in different quarters of the banks.
     static __device__ inline int f(int row) {
         if constexpr (COLS == 32) {
             return (row >> 2) & 7;
+        } else if constexpr (COLS == 128) {
+            // a row fills all banks: the row's low two bits pick the 64-byte quarter, the next three the piece
+            // within it (the staging writes of four rows then share bank pairs two by two)
+            return ((row & 3) << 3) | ((row >> 2) & 7);
         } else {
             const int v = (row >> 1) & 15;
             return ((v & 1) << 3) | (v >> 1);
@@ -112,7 +116,7 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
 }
 
 template <typename TO, int NK, int QB, int WAVES, bool ADJ>  // N = 16*NK, Q = 32*QB; ADJ: reversed-adjoint mode
-__global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_kernel(
+__global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void fused_scan_kernel(
     const __bf16 *__restrict__ x, const __bf16 *__restrict__ dt, const float *__restrict__ A,
     const __bf16 *__restrict__ Bm, const __bf16 *__restrict__ Cm, const float *__restrict__ D,
     const float *init, const unsigned char *__restrict__ reset, TO *__restrict__ y, float *final_states,
@@ -126,7 +130,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
     constexpr int BRP = nthr / BPR;            // B rows per pass of the workgroup (a multiple of 32)
     constexpr int XPR = WAVES * 4;             // 16-byte pieces of one timestep's x for the workgroup
     constexpr int UX = Q / 16;                 // passes of 16 rows
-    static_assert(BRP % 32 == 0 && nthr / XPR == 16, "staging offsets rely on the swizzle period of 32 rows");
+    static_assert((BRP % 32 == 0 || BRP == 16) && nthr / XPR == 16, "staging offsets rely on the swizzle period of 32 rows");
+    constexpr bool kSharedBcOffsets = BRP % 32 == 0;  // else every pass of B and C computes its own offsets
     using XT = ChunkTile<32>;
     using BT = ChunkTile<N>;
     // static, so that LDS addresses are compile-time offsets
@@ -331,10 +336,12 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void fused_scan_ker
 #pragma unroll
         for (int u = 0; u < UBC; ++u) {
             if (BSL % nthr == 0 || tw + u * nthr < BSL) {
-                *reinterpret_cast<uint2 *>(Bs + bw[0] + u * BRP * N) = make_uint2(bq[u].x, bq[u].y);
-                *reinterpret_cast<uint2 *>(Bs + bw[1] + u * BRP * N) = make_uint2(bq[u].z, bq[u].w);
-                *reinterpret_cast<uint2 *>(Cs + bw[0] + u * BRP * N) = make_uint2(cq[u].x, cq[u].y);
-                *reinterpret_cast<uint2 *>(Cs + bw[1] + u * BRP * N) = make_uint2(cq[u].z, cq[u].w);
+                const int o0 = kSharedBcOffsets ? bw[0] + u * BRP * N : BT::off(tw / BPR + u * BRP, (tw % BPR) * 8);
+                const int o1 = kSharedBcOffsets ? bw[1] + u * BRP * N : BT::off(tw / BPR + u * BRP, (tw % BPR) * 8 + 4);
+                *reinterpret_cast<uint2 *>(Bs + o0) = make_uint2(bq[u].x, bq[u].y);
+                *reinterpret_cast<uint2 *>(Bs + o1) = make_uint2(bq[u].z, bq[u].w);
+                *reinterpret_cast<uint2 *>(Cs + o0) = make_uint2(cq[u].x, cq[u].y);
+                *reinterpret_cast<uint2 *>(Cs + o1) = make_uint2(cq[u].z, cq[u].w);
             }
         }
 #pragma unroll
@@ -607,6 +614,12 @@ static hipError_t fused_dispatch_w(const ScanShape &s, int waves, const void *x,
                                    const void *Bm, const void *Cm, const float *D, const float *init,
                                    const unsigned char *reset, void *y, float *final_states, float *tile_states,
                                    hipStream_t st) {
+    if constexpr (NK == 8) {
+        // a 128-wide state: four waves per workgroup, one per SIMD, each with the whole register file
+        if (waves == 4)
+            return fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
+        return hipErrorInvalidValue;
+    }
     if (waves == 8) return fused_launch<TO, NK, QB, 8>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
     if (waves == 4) return fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
     // two waves: one head of 64 columns with its own B and C (the transposed scans of the backward pass);
@@ -627,6 +640,7 @@ hipError_t fused_dispatch(const ScanShape &s, int waves, const void *x, const vo
         return fused_dispatch_w<TO, NKv, QBv>(s, waves, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
     SSD_FUSED_CASE(2, kOnePassTile / 32)
     SSD_FUSED_CASE(4, kOnePassTile / 32)
+    SSD_FUSED_CASE(8, kOnePassTile / 32)
 #undef SSD_FUSED_CASE
     return hipErrorInvalidValue;
 }

@@ -10,9 +10,11 @@ hipError_t launch_fused_scan_y32(const ScanShape &, int, const void *, const voi
 int fused_scan_waves(const ScanShape &s, int dtype) {
     if (dtype == 0) return 0;                         // float inputs take the staged kernels
     if (s.P % 32 != 0) return 0;
-    if (s.N != 32 && s.N != 64) return 0;             // the state block must fit the accumulators
+    if (s.N != 32 && s.N != 64 && s.N != 128) return 0;
     const int units = (s.H / s.G) * (s.P / 32);
     int waves = (units % 8 == 0) ? 8 : ((units % 4 == 0) ? 4 : 0);
+    // a 128-wide state takes a wave's whole register file: four waves per workgroup, one per SIMD
+    if (s.N == 128) waves = (units % 4 == 0) ? 4 : 0;
     if (waves == 0 && units % 2 == 0 && s.N == 32 && dtype == 2) waves = 2;  // float y only: the backward's scans
     if (waves == 0 || fused_scan_lds_bytes(s.N, kOnePassTile, waves) > kLdsLimitBytes) return 0;
     return waves;
