@@ -445,7 +445,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     ml[j] = fl.frag();
                 }
             };
-#pragma unroll 1
+            // rolled where registers are tight; the 128-wide-state instance has a wave's whole register file
+            constexpr int kUnrollBlocks = NK == 8 ? QB : 1;
+#pragma unroll kUnrollBlocks
             for (int lb = 0; lb < QB; ++lb) {
                 const int l = lb * 32 + r;
                 // non-negative floats order like their bit patterns: a scalar compare
