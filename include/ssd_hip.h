@@ -140,6 +140,12 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
  * touched), 0 if as the staged kernels.  A plan query like ssd_workspace_bytes; no reference counterpart. */
 int ssd_chunk_scan_is_onepass(const ssd_dims *dims, int dtype, int *is_onepass);
 
+/* *segments > 1 if ssd_chunk_scan_fwd runs these dims as the one-pass kernel on that many segments of the
+ * sequence side by side (batches too small to fill the chip with whole sequences, long enough to be worth
+ * cutting: a states-only pass per segment, a recurrence over the segments, then the forward per segment; the
+ * segment states live in the workspace).  1 otherwise.  A plan query; no reference counterpart. */
+int ssd_chunk_scan_segments(const ssd_dims *dims, int dtype, int *segments);
+
 /* Stage 3: sequential recurrence over chunks.  prev_states[c] receives the state entering
  * chunk c and may alias chunk_states (in place); final_states and initial_states may be NULL
  * and may alias each other. */

@@ -1,13 +1,15 @@
 """The one-pass forward (one kernel, running state in registers) through the C ABI against the float64
 oracle: the shapes that pick each of its template instances, ragged tails, initial states, strong decay
 (the exact diagonal path), and agreement with the staged kernels."""
+import numpy as np
 import pytest
 import torch
 
+from oracle import ssd_oracle as orc
 from trading_bot_0_amd import SsdError, ssd_chunk_scan, ssd_chunk_scan_onepass
 from trading_bot_0_amd.synthetic import WORKLOADS, Workload, make_inputs
 
-from _util import assert_close, check_y, oracle_scan, rel_err, to_dev
+from _util import assert_close, check_y, np64, oracle_scan, rel_err, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -151,3 +153,38 @@ def test_one_pass_kernel_on_a_side_stream_and_inside_a_captured_graph():
         torch.cuda.synchronize()
         y_e, f_e = run(dev, 128)
         assert torch.equal(out, y_e) and torch.equal(fin, f_e), f"replay {i}"
+
+
+@pytest.mark.parametrize("seqlen,with_reset", [(2048, False), (1990, True)])
+def test_mid_size_batches_run_cut_into_segments(seqlen, with_reset):
+    """48 sequences of 2048 steps: too few for one workgroup per 8 units to fill the chip, enough work for the
+    one-pass kernel on segments of the sequence to beat the staged kernels.  Rows against the oracle, with an
+    initial state, a ragged length and restarts that fall on and next to segment borders."""
+    from trading_bot_0_amd.ssd import chunk_scan_segments
+    w = Workload("segments", 48, seqlen, 8, 32, 64, 1, 128, init_std=0.5)
+    assert chunk_scan_segments(w.batch, seqlen, 8, 32, 64, 1, 128) == 4
+    assert chunk_scan_segments(4, 4096, 8, 32, 64, 1, 128) == 1          # little work in total: staged
+    assert chunk_scan_segments(256, 2048, 8, 32, 64, 1, 128) == 1        # fills the chip uncut
+    dev = make_inputs(w, seed=6, device="cuda")
+    reset = None
+    m = None
+    if with_reset:
+        m = (np.random.default_rng(3).random((w.batch, seqlen)) < 0.002).astype(np.uint8)
+        for t in (511, 512, 513, 1024, 1535, 1536):
+            m[1, t] = 1
+        reset = torch.from_numpy(m).cuda()
+    y32, final = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                                initial_states=dev["init"], y_dtype=torch.float32, reset=reset)
+    y16, final16 = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                                  initial_states=dev["init"], reset=reset)
+    assert torch.equal(y16, y32.to(torch.bfloat16)) and torch.equal(final, final16)
+    rows = [0, 1, 47]
+    yr, fr = orc.ssd_sequential(*(np64(dev[k][rows]) for k in ("x", "dt")), np64(dev["A"]), np64(dev["B"][rows]),
+                                np64(dev["C"][rows]), np64(dev["D"]), np64(dev["init"][rows]),
+                                reset=None if m is None else m[rows])
+    assert_close(y32[rows], yr, torch.bfloat16, "segmented y (float32 y)")
+    assert_close(final[rows], fr, torch.bfloat16, "segmented final")
+    # the uncut one-pass kernel gives the same result to rounding
+    y1, f1 = ssd_chunk_scan_onepass(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                                    initial_states=dev["init"], y_dtype=torch.float32, reset=reset)
+    assert rel_err(y32, np64(y1)) <= 1e-4 and rel_err(final, np64(f1)) <= 1e-4

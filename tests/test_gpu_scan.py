@@ -217,9 +217,10 @@ def full_size_properties(w, rows, seed=0):
     y1, f1 = run(a, w.chunk)
     b["init"] = f1
     y2, f2 = run(b, w.chunk)
-    assert torch.equal(y1, y[:, :h]), "first half does not depend on the future"
-    tail = y[:, h:].float()
-    assert ((y2.float() - tail).abs() <= 2.0 ** -7 * tail.abs() + 1e-3 * max(1.0, float(tail.abs().mean()))).all()
+    # the first half does not depend on the future.  (Not bit for bit: a small batch of long sequences runs cut
+    # into segments, and the half-length run is cut elsewhere, so the two differ by roundings.)
+    for part, ref in ((y1, y[:, :h].float()), (y2, y[:, h:].float())):
+        assert ((part.float() - ref).abs() <= 2.0 ** -7 * ref.abs() + 1e-3 * max(1.0, float(ref.abs().mean()))).all()
     assert rel_err(f2, np64(final)) <= 1e-4
 
 

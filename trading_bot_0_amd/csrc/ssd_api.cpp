@@ -333,6 +333,13 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
         e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states, st);
         return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
     }
+    if (const int segments = ssd::fused_scan_segments(s, dtype); segments > 1) {
+        // too few sequences for one workgroup per 8 units to fill the chip, but long ones: the one-pass kernel on
+        // segments of the sequence; the segment states (fewer than the chunk states) and decays use the workspace
+        e = ssd::launch_fused_scan_segmented(s, dtype, segments, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states,
+                                             states, dtcs, st);
+        return e == hipSuccess ? SSD_OK : hip_fail(e, "segmented one-pass scan launch");
+    }
     return run_staged(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, 0, y, final_states, dtcs, states, st);
 }
 
@@ -488,6 +495,14 @@ int ssd_chunk_scan_is_onepass(const ssd_dims *dims, int dtype, int *is_onepass) 
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
     *is_onepass = takes_one_pass(s, dtype) ? 1 : 0;
+    return SSD_OK;
+}
+
+int ssd_chunk_scan_segments(const ssd_dims *dims, int dtype, int *segments) {
+    if (segments == nullptr) return fail(SSD_ERR_INVALID, "ssd: segments must not be NULL");
+    ssd::ScanShape s;
+    if (int rc = make_shape(dims, dtype, &s)) return rc;
+    *segments = takes_one_pass(s, dtype) ? 1 : ssd::fused_scan_segments(s, dtype);
     return SSD_OK;
 }
 

@@ -115,13 +115,17 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
            (size_t)waves * ((size_t)fused_scan_xtile_elems(Q) * 2 + (size_t)(5 + Q / 32) * Q * 4 + 64);
 }
 
-template <typename TO, int NK, int QB, int WAVES, bool ADJ>  // N = 16*NK, Q = 32*QB; ADJ: reversed-adjoint mode
+// KIND 0: the forward.  KIND 1: the reversed-adjoint recurrence of the backward pass.  KIND 2: states only --
+// no outputs, no C: the state a segment of the sequence leaves behind (from its own initial state) and the
+// segment's total decay, for sequences cut into segments that run side by side.
+template <typename TO, int NK, int QB, int WAVES, int KIND>  // N = 16*NK, Q = 32*QB
 __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void fused_scan_kernel(
     const __bf16 *__restrict__ x, const __bf16 *__restrict__ dt, const float *__restrict__ A,
     const __bf16 *__restrict__ Bm, const __bf16 *__restrict__ Cm, const float *__restrict__ D,
     const float *init, const unsigned char *__restrict__ reset, TO *__restrict__ y, float *final_states,
-    float *tile_states, ScanShape s) {
+    float *tile_states, float *seg_decay, ScanShape s) {
     using T = __bf16;
+    constexpr bool ADJ = KIND == 1, STATES_ONLY = KIND == 2;
     constexpr int N = 16 * NK, NB = NK / 2, Q = 32 * QB, nthr = 64 * WAVES;
     constexpr int EPL = Q >= 64 ? Q / 64 : 1;  // chunk positions per lane in the scan
     constexpr int BPR = N / 8;                 // 16-byte pieces per B (or C) row
@@ -152,7 +156,13 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // ---- which units this workgroup owns ----
     const int PBn = s.P / 32, HG = s.H / s.G;
     const int UW = (HG * PBn) / WAVES;  // workgroups per (batch, group)
-    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    // A sequence may be cut into S segments of s.seg_tiles tiles that different workgroups walk: initial states
+    // are then given per segment ([B,S,H,P,N]) and, in KIND 2, final states and decays written per segment.
+    const int S = s.seg_tiles > 0 ? (s.nc + s.seg_tiles - 1) / s.seg_tiles : 1;
+    const int slot = xcd_remap(blockIdx.x, gridDim.x);
+    const int seg = slot % S, logical = slot / S;
+    const int c_first = seg * (s.seg_tiles > 0 ? s.seg_tiles : s.nc);
+    const int c_end = s.seg_tiles > 0 ? min(s.nc, c_first + s.seg_tiles) : s.nc;
     const int b = logical / (s.G * UW);
     const int g = (logical / UW) % s.G;
     const int unit0 = (logical % UW) * WAVES;
@@ -241,7 +251,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 const int src = first - (bc_row0 + u * BRP);
                 const bool ok = (BSL % nthr == 0 || tv + u * nthr < BSL) && src >= 0 && src < trows;
                 bq[u] = ld16(Bb + (size_t)src * s.G * N + (tv % BPR) * 8, ok);
-                cq[u] = ld16(Cb + (size_t)src * s.G * N + (tv % BPR) * 8, ok);
+                if (!STATES_ONLY) cq[u] = ld16(Cb + (size_t)src * s.G * N + (tv % BPR) * 8, ok);
             }
 #pragma unroll
             for (int u = 0; u < UX; ++u) {
@@ -257,7 +267,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             for (int u = 0; u < UBC; ++u) {
                 const bool ok = BSL % nthr == 0 || tv + u * nthr < BSL;
                 bq[u] = ld16(bp + (size_t)u * BRP * s.G * N + bc_off0, ok);
-                cq[u] = ld16(cp + (size_t)u * BRP * s.G * N + bc_off0, ok);
+                if (!STATES_ONLY) cq[u] = ld16(cp + (size_t)u * BRP * s.G * N + bc_off0, ok);
             }
 #pragma unroll
             for (int u = 0; u < UX; ++u) xq[u] = *reinterpret_cast<const uint4 *>(xp + (size_t)u * 16 * XLD + x_off0);
@@ -272,7 +282,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             for (int u = 0; u < UBC; ++u) {
                 const bool ok = (BSL % nthr == 0 || tv + u * nthr < BSL) && bc_row0 + u * BRP < rows;
                 bq[u] = ld16(bp + (size_t)u * BRP * s.G * N + bc_off0, ok);
-                cq[u] = ld16(cp + (size_t)u * BRP * s.G * N + bc_off0, ok);
+                if (!STATES_ONLY) cq[u] = ld16(cp + (size_t)u * BRP * s.G * N + bc_off0, ok);
             }
 #pragma unroll
             for (int u = 0; u < UX; ++u) xq[u] = ld16(xp + (size_t)u * 16 * XLD + x_off0, x_row0 + u * 16 < rows);
@@ -288,7 +298,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // ---- running state of this unit: st[nb][v] = H[p = r, n = 32 nb + 8 (v/4) + 4 half + v%4] ----
     f32x16 st[NB];
     {
-        const float *ib = init ? init + (((size_t)b * s.H + h) * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5) : nullptr;
+        const float *ib = init ? init + ((((size_t)b * S + seg) * s.H + h) * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5)
+                               : nullptr;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
@@ -314,8 +325,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         }
     };
 
-    prefetch(0);
-    for (int c = 0; c < s.nc; ++c) {
+    float seg_total = 1.f;  // product of the tiles' decays (KIND 2)
+    prefetch(c_first);
+    for (int c = c_first; c < c_end; ++c) {
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
         // the state entering every tile, for a caller that needs it (the backward pass): [B, nc, H, P, N]
@@ -340,8 +352,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 const int o1 = kSharedBcOffsets ? bw[1] + u * BRP * N : BT::off(tw / BPR + u * BRP, (tw % BPR) * 8 + 4);
                 *reinterpret_cast<uint2 *>(Bs + o0) = make_uint2(bq[u].x, bq[u].y);
                 *reinterpret_cast<uint2 *>(Bs + o1) = make_uint2(bq[u].z, bq[u].w);
-                *reinterpret_cast<uint2 *>(Cs + o0) = make_uint2(cq[u].x, cq[u].y);
-                *reinterpret_cast<uint2 *>(Cs + o1) = make_uint2(cq[u].z, cq[u].w);
+                if (!STATES_ONLY) {
+                    *reinterpret_cast<uint2 *>(Cs + o0) = make_uint2(cq[u].x, cq[u].y);
+                    *reinterpret_cast<uint2 *>(Cs + o1) = make_uint2(cq[u].z, cq[u].w);
+                }
             }
         }
 #pragma unroll
@@ -406,11 +420,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 }
             }
         }
-        if (kEarlyPrefetch && c + 1 < s.nc) prefetch(c + 1);
+        if (kEarlyPrefetch && c + 1 < c_end) prefetch(c + 1);
         block_sync_lds();  // tiles and tables are visible
 
         // ---- phase 1: outputs of this chunk from the state entering it ----
-        {
+        if constexpr (!STATES_ONLY) {
             const int lane = phase_tid() & 63;
             const int r = lane & 31, half = lane >> 5;
             Frag<T> Hhi[NK], Hlo[NK];
@@ -533,7 +547,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         }
 
         // ---- phase 2: the state leaving this chunk ----
-        if (!kEarlyPrefetch && c + 1 < s.nc) prefetch(c + 1);
+        if (!kEarlyPrefetch && c + 1 < c_end) prefetch(c + 1);
+        seg_total *= a_end;
         const int lane = phase_tid() & 63, half = lane >> 5;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) st[nb] = st[nb] * a_end;
@@ -580,7 +595,12 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         }
     }
 
-    if (final_states) store_state(final_states + ((size_t)b * s.H + h) * s.P * N);
+    if (STATES_ONLY) {
+        store_state(final_states + (((size_t)b * S + seg) * s.H + h) * s.P * N);
+        if (pb == 0 && lane0 == 0) seg_decay[((size_t)b * S + seg) * s.H + h] = seg_total;
+    } else if (final_states && seg == S - 1) {
+        store_state(final_states + ((size_t)b * s.H + h) * s.P * N);
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -593,21 +613,39 @@ static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt
     // (requesting the next tile's inputs at the top of the tile instead of after phase 1 measured the same,
     // 217.6 us against 218.8 us, for 26 more live registers)
     const int units = (s.H / s.G) * (s.P / 32);
-    const int grid = s.B * s.G * (units / WAVES);
+    const int segments = s.seg_tiles > 0 ? (s.nc + s.seg_tiles - 1) / s.seg_tiles : 1;
+    const int grid = s.B * s.G * (units / WAVES) * segments;
     const __bf16 *xx = static_cast<const __bf16 *>(x), *dd = static_cast<const __bf16 *>(dt);
     const __bf16 *bb = static_cast<const __bf16 *>(Bm), *cc = static_cast<const __bf16 *>(Cm);
     if (s.mode != 0) {
         // the reversed-adjoint mode serves the backward pass, which takes float outputs only
         if constexpr (sizeof(TO) == 4) {
-            fused_scan_kernel<TO, NK, QB, WAVES, true><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, s);
+            if (segments != 1) return hipErrorInvalidValue;
+            fused_scan_kernel<TO, NK, QB, WAVES, 1><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
+                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, s);
             return hipGetLastError();
         } else {
             return hipErrorInvalidValue;
         }
     }
-    fused_scan_kernel<TO, NK, QB, WAVES, false><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, s);
+    fused_scan_kernel<TO, NK, QB, WAVES, 0><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
+        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, s);
+    return hipGetLastError();
+}
+
+// States only (KIND 2): per segment, the state it leaves behind from `init` ([B,S,H,P,N] or NULL = zero) into
+// seg_states [B,S,H,P,N] and its total decay into seg_decay [B,S,H].
+template <int NK, int QB, int WAVES>
+static hipError_t fused_launch_states(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
+                                      const float *init, const unsigned char *reset, float *seg_states, float *seg_decay,
+                                      hipStream_t st) {
+    const int units = (s.H / s.G) * (s.P / 32);
+    const int segments = s.seg_tiles > 0 ? (s.nc + s.seg_tiles - 1) / s.seg_tiles : 1;
+    const int grid = s.B * s.G * (units / WAVES) * segments;
+    const __bf16 *bb = static_cast<const __bf16 *>(Bm);
+    fused_scan_kernel<__bf16, NK, QB, WAVES, 2><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
+        static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, bb, bb, nullptr, init, reset, nullptr, seg_states,
+        nullptr, seg_decay, s);
     return hipGetLastError();
 }
 

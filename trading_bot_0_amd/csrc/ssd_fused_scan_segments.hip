@@ -1,0 +1,84 @@
+// One-pass forward for batches too small to fill the chip with one workgroup per 8 units: the sequence is cut
+// into segments that different workgroups walk side by side.
+//   1. states only (no y, no C): what every segment adds to the state, from a zero state, and its total decay;
+//   2. the state entering every segment: a recurrence over the few segments, one lane per 4 state elements;
+//   3. the forward proper per segment, each from its entering state.
+// Step 1 costs about 0.4 of step 3 (staging, scan and the state update, without the output phase); the two
+// together run S times as many workgroups as the uncut kernel.
+#include "ssd_fused_scan.h"
+
+namespace ssd {
+
+namespace {
+
+constexpr int kSegmentMinTiles = 4;        // shorter segments are mostly prologue
+constexpr int kSegmentTargetGroups = 192;  // workgroups to aim for (256 CUs; the last quarter gains little)
+
+// enter[b,0] = init (or zero); enter[b,s+1] = decay[b,s] * enter[b,s] + local[b,s], written over local in place
+__global__ __launch_bounds__(256) void segment_states_kernel(float *states, const float *__restrict__ decay,
+                                                             const float *__restrict__ init, int S, int H, int pn4,
+                                                             long long total) {
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const int idx = (int)(gid % pn4);
+    const long long bh = gid / pn4;
+    const int h = (int)(bh % H);
+    const long long b = bh / H;
+    float4 cur = init ? reinterpret_cast<const float4 *>(init)[bh * pn4 + idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < S; ++s) {
+        float4 *slot = reinterpret_cast<float4 *>(states) + ((b * S + s) * H + h) * (long long)pn4 + idx;
+        const float4 loc = *slot;
+        const float a = decay[(b * S + s) * H + h];
+        *slot = cur;
+        cur = make_float4(a * cur.x + loc.x, a * cur.y + loc.y, a * cur.z + loc.z, a * cur.w + loc.w);
+    }
+}
+
+int tiles_of(const ScanShape &s) { return (s.L + kOnePassTile - 1) / kOnePassTile; }
+
+}  // namespace
+
+int fused_scan_segments(const ScanShape &s, int dtype) {
+    if (fused_scan_waves(s, dtype) != 8 || s.N == 128) return 1;
+    const long long groups = (long long)s.B * s.G * ((s.H / s.G) * (s.P / 32) / 8);
+    const int nc = tiles_of(s);
+    int S = 1;
+    while (groups * S < kSegmentTargetGroups && nc / (2 * S) >= kSegmentMinTiles) S *= 2;
+    if (S < 2) return 1;
+    const int seg_tiles = (nc + S - 1) / S;
+    const int segments = (nc + seg_tiles - 1) / seg_tiles;
+    // Worth it only against what the staged kernels would take, which run every tile of every sequence side by
+    // side and so win when there is little work in total.  Measured on MI355X, microseconds: a workgroup walks a
+    // tile in about 6.5 (states only: 0.4 of that), the staged kernels take about 510 per 2048 units x 32 tiles,
+    // and a launch costs about 5.
+    const double rounds = (double)((groups * segments + 255) / 256);
+    const double cut = 15.0 + 1.4 * 6.5 * seg_tiles * rounds;
+    const double staged = 20.0 + 510.0 * ((double)groups * 8 * nc) / (2048.0 * 32.0);
+    return cut < staged ? segments : 1;
+}
+
+hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segments, const void *x, const void *dt,
+                                       const float *A, const void *Bm, const void *Cm, const float *D, const float *init,
+                                       const unsigned char *reset, void *y, float *final_states, float *seg_states,
+                                       float *seg_decay, hipStream_t st) {
+    if (segments < 2 || fused_scan_waves(s, dtype) != 8 || s.N == 128) return hipErrorInvalidValue;
+    ScanShape t = s;
+    t.Q = kOnePassTile;
+    t.nc = tiles_of(s);
+    t.seg_tiles = (t.nc + segments - 1) / segments;
+    if ((t.nc + t.seg_tiles - 1) / t.seg_tiles != segments) return hipErrorInvalidValue;
+    hipError_t e = t.N == 32 ? fused_launch_states<2, kOnePassTile / 32, 8>(t, x, dt, A, Bm, nullptr, reset, seg_states, seg_decay, st)
+                             : fused_launch_states<4, kOnePassTile / 32, 8>(t, x, dt, A, Bm, nullptr, reset, seg_states, seg_decay, st);
+    if (e != hipSuccess) return e;
+    const int pn4 = s.P * s.N / 4;
+    const long long total = (long long)s.B * s.H * pn4;
+    segment_states_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(seg_states, seg_decay, init, segments, s.H,
+                                                                                     pn4, total);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    ScanShape f = s;
+    f.seg_tiles = t.seg_tiles;
+    return launch_fused_scan(f, dtype, x, dt, A, Bm, Cm, D, seg_states, reset, y, final_states, st);
+}
+
+}  // namespace ssd

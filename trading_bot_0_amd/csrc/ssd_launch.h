@@ -17,6 +17,9 @@ struct ScanShape {
     // The one-pass kernel only, shapes with B and C per head (G == H): x is given once per x_groups groups of
     // heads, as a [B, L, x_groups, P] tensor, instead of once per head (0 = per head, [B, L, H, P]).
     int x_groups = 0;
+    // The one-pass kernel only: the sequence cut into segments of seg_tiles tiles of 64 steps (0 = not cut) that
+    // different workgroups walk; initial states are then given per segment, [B, segments, H, P, N].
+    int seg_tiles = 0;
 };
 
 struct StepShape {
@@ -65,6 +68,16 @@ hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const
                              const void *Bm, const void *Cm, const float *D, const float *init,
                              const unsigned char *reset, void *y, float *final_states, hipStream_t stream,
                              float *tile_states = nullptr);
+// The one-pass forward with the sequence cut into segments that run side by side (bf16 inputs, dstate 32 or 64):
+// first every segment's own contribution to the state and its total decay (states only, no y, no C), then the
+// state entering every segment by a recurrence over the segments, then the forward proper per segment.
+// seg_states [B, segments, H, P, N] and seg_decay [B, segments, H] are scratch of the caller.
+// fused_scan_segments: into how many segments a shape would be cut (1 = not worth cutting, or not eligible).
+int fused_scan_segments(const ScanShape &s, int dtype);
+hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segments, const void *x, const void *dt,
+                                       const float *A, const void *Bm, const void *Cm, const float *D, const float *init,
+                                       const unsigned char *reset, void *y, float *final_states, float *seg_states,
+                                       float *seg_decay, hipStream_t stream);
 hipError_t launch_step(const StepShape &s, int dtype, float *state, const void *x, const void *dt,
                        const float *A, const void *Bm, const void *Cm, const float *D, void *y,
                        hipStream_t stream);

@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "ssd_chunk_state_passing_fwd",
     "ssd_chunk_scan_onepass_fwd",
     "ssd_chunk_scan_is_onepass",
+    "ssd_chunk_scan_segments",
     "ssd_chunk_scan_stage_fwd",
     "ssd_step_fwd",
     "ssd_steps_fwd",
@@ -99,6 +100,7 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_chunk_scan_onepass_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_chunk_scan_reset_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, P, c_size_t, P]
         lib.ssd_chunk_scan_is_onepass.argtypes = [POINTER(SsdDims), c_int, POINTER(c_int)]
+        lib.ssd_chunk_scan_segments.argtypes = [POINTER(SsdDims), c_int, POINTER(c_int)]
         lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
         lib.ssd_step_fwd.argtypes = [POINTER(SsdStepDims), c_int, P, P, P, P, P, P, P, P, P]
         lib.ssd_steps_fwd.argtypes = [POINTER(SsdStepDims), c_int64, c_int, P, P, P, P, P, P, P, P, P, P]
@@ -360,6 +362,17 @@ def chunk_scan_is_onepass(batch, seqlen, nheads, headdim, dstate, ngroups, chunk
     code = SSD_DTYPE_BF16 if dtype == torch.bfloat16 else SSD_DTYPE_F32
     _check(lib, lib.ssd_chunk_scan_is_onepass(byref(dims), code, byref(flag)))
     return bool(flag.value)
+
+
+def chunk_scan_segments(batch, seqlen, nheads, headdim, dstate, ngroups, chunk, dtype=torch.bfloat16) -> int:
+    """Into how many segments ssd_chunk_scan cuts the sequences of this shape to run them on the one-pass kernel
+    side by side (1 = not cut)."""
+    lib = load_library()
+    dims = SsdDims(batch, seqlen, nheads, headdim, dstate, ngroups, chunk)
+    n = c_int(0)
+    code = SSD_DTYPE_BF16 if dtype == torch.bfloat16 else SSD_DTYPE_F32
+    _check(lib, lib.ssd_chunk_scan_segments(byref(dims), code, byref(n)))
+    return n.value
 
 
 def ssd_chunk_scan_onepass(
