@@ -112,9 +112,8 @@ Workspace carve(const ssd::ScanShape &s) {
 }
 
 bool takes_one_pass(const ssd::ScanShape &s, int dtype) {
-    const int waves = ssd::fused_scan_waves(s, dtype);
-    const int full = s.N == 128 ? 4 : 8;  // waves of a workgroup that fills a CU
-    return waves == full && (int64_t)s.B * s.H * (s.P / 32) / full >= kOnePassMinWorkgroups;
+    int segments;
+    return ssd::fused_scan_plan(s, dtype, &segments) == 1;
 }
 
 int hip_fail(hipError_t e, const char *what) {
@@ -333,7 +332,7 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
         e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states, st);
         return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
     }
-    if (const int segments = ssd::fused_scan_segments(s, dtype); segments > 1) {
+    if (int segments = 1; ssd::fused_scan_plan(s, dtype, &segments) == 2) {
         // too few sequences for one workgroup per 8 units to fill the chip, but long ones: the one-pass kernel on
         // segments of the sequence; the segment states (fewer than the chunk states) and decays use the workspace
         e = ssd::launch_fused_scan_segmented(s, dtype, segments, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states,
@@ -502,7 +501,7 @@ int ssd_chunk_scan_segments(const ssd_dims *dims, int dtype, int *segments) {
     if (segments == nullptr) return fail(SSD_ERR_INVALID, "ssd: segments must not be NULL");
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
-    *segments = takes_one_pass(s, dtype) ? 1 : ssd::fused_scan_segments(s, dtype);
+    ssd::fused_scan_plan(s, dtype, segments);
     return SSD_OK;
 }
 

@@ -38,23 +38,35 @@ int tiles_of(const ScanShape &s) { return (s.L + kOnePassTile - 1) / kOnePassTil
 
 }  // namespace
 
-int fused_scan_segments(const ScanShape &s, int dtype) {
-    if (fused_scan_waves(s, dtype) != 8 || s.N == 128) return 1;
-    const long long groups = (long long)s.B * s.G * ((s.H / s.G) * (s.P / 32) / 8);
+// Which way a forward runs fastest: 0 = staged kernels, 1 = the one-pass kernel, 2 = the one-pass kernel on
+// *segments segments.  Estimates in microseconds from measurements on MI355X: a workgroup walks a tile of 64 steps
+// in about 6.5 (states only: 0.4 of that) and a CU holds one workgroup, so the one-pass kernel takes that times
+// the tiles of a sequence (or segment) times the rounds of 256 workgroups; the staged kernels run every tile of
+// every sequence side by side, about 510 per 2048 units x 32 tiles; a launch costs about 5.
+int fused_scan_plan(const ScanShape &s, int dtype, int *segments) {
+    *segments = 1;
+    const int waves = fused_scan_waves(s, dtype);
+    const int full = s.N == 128 ? 4 : 8;  // waves of a workgroup that fills a CU
+    if (waves != full) return 0;
+    const long long groups = (long long)s.B * s.G * ((s.H / s.G) * (s.P / 32) / full);
     const int nc = tiles_of(s);
+    const double staged = 20.0 + 510.0 * ((double)groups * full * nc) / (2048.0 * 32.0) * (s.N == 128 ? 2.0 : 1.0);
+    const double whole = 5.0 + 6.5 * nc * (double)((groups + 255) / 256);
+    double cut = 1e30;
     int S = 1;
-    while (groups * S < kSegmentTargetGroups && nc / (2 * S) >= kSegmentMinTiles) S *= 2;
-    if (S < 2) return 1;
-    const int seg_tiles = (nc + S - 1) / S;
-    const int segments = (nc + seg_tiles - 1) / seg_tiles;
-    // Worth it only against what the staged kernels would take, which run every tile of every sequence side by
-    // side and so win when there is little work in total.  Measured on MI355X, microseconds: a workgroup walks a
-    // tile in about 6.5 (states only: 0.4 of that), the staged kernels take about 510 per 2048 units x 32 tiles,
-    // and a launch costs about 5.
-    const double rounds = (double)((groups * segments + 255) / 256);
-    const double cut = 15.0 + 1.4 * 6.5 * seg_tiles * rounds;
-    const double staged = 20.0 + 510.0 * ((double)groups * 8 * nc) / (2048.0 * 32.0);
-    return cut < staged ? segments : 1;
+    if (s.N != 128) {
+        while (groups * S < kSegmentTargetGroups && nc / (2 * S) >= kSegmentMinTiles) S *= 2;
+        if (S >= 2) {
+            const int seg_tiles = (nc + S - 1) / S;
+            S = (nc + seg_tiles - 1) / seg_tiles;
+            cut = 15.0 + 1.4 * 6.5 * seg_tiles * (double)((groups * S + 255) / 256);
+        }
+    }
+    if (cut < whole && cut < staged) {
+        *segments = S;
+        return 2;
+    }
+    return whole < staged ? 1 : 0;
 }
 
 hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segments, const void *x, const void *dt,

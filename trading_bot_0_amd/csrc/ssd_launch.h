@@ -72,8 +72,9 @@ hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const
 // first every segment's own contribution to the state and its total decay (states only, no y, no C), then the
 // state entering every segment by a recurrence over the segments, then the forward proper per segment.
 // seg_states [B, segments, H, P, N] and seg_decay [B, segments, H] are scratch of the caller.
-// fused_scan_segments: into how many segments a shape would be cut (1 = not worth cutting, or not eligible).
-int fused_scan_segments(const ScanShape &s, int dtype);
+// fused_scan_plan: which way a forward of this shape runs fastest by the library's cost estimates: 0 = the
+// staged kernels, 1 = the one-pass kernel, 2 = the one-pass kernel on *segments segments.
+int fused_scan_plan(const ScanShape &s, int dtype, int *segments);
 hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segments, const void *x, const void *dt,
                                        const float *A, const void *Bm, const void *Cm, const float *D, const float *init,
                                        const unsigned char *reset, void *y, float *final_states, float *seg_states,
