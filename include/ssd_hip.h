@@ -136,8 +136,9 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
                              const uint8_t *reset, void *y, float *final_states, void *workspace,
                              size_t workspace_bytes, void *hip_stream);
 
-/* *is_onepass = 1 if ssd_chunk_scan_fwd runs these dims as the one-pass kernel (its workspace is then not
- * touched), 0 if as the staged kernels.  A plan query like ssd_workspace_bytes; no reference counterpart. */
+/* *is_onepass = 1 if ssd_chunk_scan_fwd runs these dims as one launch of the one-pass kernel (its workspace is
+ * then not touched), 0 otherwise (staged kernels, the one-pass kernel on segments, or a batch whose partial
+ * last round of workgroups runs as a batch of its own).  A plan query like ssd_workspace_bytes; no reference counterpart. */
 int ssd_chunk_scan_is_onepass(const ssd_dims *dims, int dtype, int *is_onepass);
 
 /* *segments > 1 if ssd_chunk_scan_fwd runs these dims as the one-pass kernel on that many segments of the

@@ -327,19 +327,49 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
     float *dtcs = reinterpret_cast<float *>(base + w.dtcs_off);
     float *states = reinterpret_cast<float *>(base + w.st_off);
     hipStream_t st = (hipStream_t)hip_stream;
-    hipError_t e;
-    if (takes_one_pass(s, dtype)) {
-        e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states, st);
-        return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
+    // One batch of sequences, the way the plan says.  The workspace is carved for the whole batch and so holds any
+    // part of it.
+    auto forward = [&](const ssd::ScanShape &part, const void *px, const void *pdt, const void *pb, const void *pc,
+                       const float *pinit, const uint8_t *preset, void *py, float *pfinal) -> int {
+        int segments = 1;
+        const int plan = ssd::fused_scan_plan(part, dtype, &segments);
+        hipError_t e;
+        if (plan == 1) {
+            e = ssd::launch_fused_scan(part, dtype, px, pdt, A, pb, pc, D, pinit, preset, py, pfinal, st);
+            return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");
+        }
+        if (plan == 2) {
+            // too few sequences for one workgroup per 8 units to fill the chip, but long ones: the one-pass kernel
+            // on segments of the sequence; the segment states (fewer than the chunk states) and decays use the
+            // workspace
+            e = ssd::launch_fused_scan_segmented(part, dtype, segments, px, pdt, A, pb, pc, D, pinit, preset, py, pfinal,
+                                                 states, dtcs, st);
+            return e == hipSuccess ? SSD_OK : hip_fail(e, "segmented one-pass scan launch");
+        }
+        return run_staged(part, dtype, px, pdt, A, pb, pc, D, pinit, preset, 0, py, pfinal, dtcs, states, st);
+    };
+    // A batch that fills the chip some whole number of times and a bit: the whole rounds run as one launch of the
+    // one-pass kernel, the rest as a batch of its own (cut into segments or staged, as the plan says for it) -- a
+    // last round of a few workgroups would cost as long as a full one.
+    const int tail_rows = ssd::fused_scan_tail_rows(s, dtype);
+    if (tail_rows > 0) {
+        const int main_rows = s.B - tail_rows;
+        const size_t eb = dtype == SSD_DTYPE_F32 ? 4 : 2, yb = dtype == SSD_DTYPE_BF16 ? 2 : 4;
+        const size_t row_x = (size_t)s.L * s.H * s.P, row_dt = (size_t)s.L * s.H, row_bc = (size_t)s.L * s.G * s.N;
+        const size_t row_st = (size_t)s.H * s.P * s.N;
+        auto off = [](const void *p, size_t bytes) { return p ? static_cast<const char *>(p) + bytes : nullptr; };
+        ssd::ScanShape head = s, tail = s;
+        head.B = main_rows;
+        tail.B = tail_rows;
+        if (int rc = forward(head, x, dt, Bm, Cm, initial_states, reset, y, final_states)) return rc;
+        return forward(tail, off(x, main_rows * row_x * eb), off(dt, main_rows * row_dt * eb), off(Bm, main_rows * row_bc * eb),
+                       off(Cm, main_rows * row_bc * eb),
+                       reinterpret_cast<const float *>(off(initial_states, main_rows * row_st * 4)),
+                       reinterpret_cast<const uint8_t *>(off(reset, (size_t)main_rows * s.L)),
+                       const_cast<char *>(off(y, main_rows * row_x * yb)),
+                       reinterpret_cast<float *>(const_cast<char *>(off(final_states, main_rows * row_st * 4))));
     }
-    if (int segments = 1; ssd::fused_scan_plan(s, dtype, &segments) == 2) {
-        // too few sequences for one workgroup per 8 units to fill the chip, but long ones: the one-pass kernel on
-        // segments of the sequence; the segment states (fewer than the chunk states) and decays use the workspace
-        e = ssd::launch_fused_scan_segmented(s, dtype, segments, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states,
-                                             states, dtcs, st);
-        return e == hipSuccess ? SSD_OK : hip_fail(e, "segmented one-pass scan launch");
-    }
-    return run_staged(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, 0, y, final_states, dtcs, states, st);
+    return forward(s, x, dt, Bm, Cm, initial_states, reset, y, final_states);
 }
 
 int ssd_chunk_scan_bwd_workspace_bytes(const ssd_dims *dims, int dtype, size_t *out_bytes) {
@@ -493,7 +523,7 @@ int ssd_chunk_scan_is_onepass(const ssd_dims *dims, int dtype, int *is_onepass) 
     if (is_onepass == nullptr) return fail(SSD_ERR_INVALID, "ssd: is_onepass must not be NULL");
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
-    *is_onepass = takes_one_pass(s, dtype) ? 1 : 0;
+    *is_onepass = (takes_one_pass(s, dtype) && ssd::fused_scan_tail_rows(s, dtype) == 0) ? 1 : 0;
     return SSD_OK;
 }
 

@@ -75,6 +75,9 @@ hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const
 // fused_scan_plan: which way a forward of this shape runs fastest by the library's cost estimates: 0 = the
 // staged kernels, 1 = the one-pass kernel, 2 = the one-pass kernel on *segments segments.
 int fused_scan_plan(const ScanShape &s, int dtype, int *segments);
+// fused_scan_tail_rows: for a batch that fills the chip a whole number of times and a bit, the batch rows of
+// that bit when it is cheaper run as a batch of its own than as one more round of the one-pass kernel; else 0.
+int fused_scan_tail_rows(const ScanShape &s, int dtype);
 hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segments, const void *x, const void *dt,
                                        const float *A, const void *Bm, const void *Cm, const float *D, const float *init,
                                        const unsigned char *reset, void *y, float *final_states, float *seg_states,
