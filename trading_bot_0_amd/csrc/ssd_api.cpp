@@ -146,7 +146,7 @@ int run_staged(const ssd::ScanShape &s, int dtype, const void *x, const void *dt
 // array), the gathered operands (reversed ones padded to whole chunks) and the scans' float outputs.
 struct BwdWorkspace {
     size_t scan_off, states2, dy_rev, x_rev, c_rev_g, b_rev_g, c_rev_h, b_fwd_h, r_rev, yb_rev, yc, gfin, gfin_t, ffin_t,
-        init_t, dfin_t, e1, dd, u, anchor, da_part, total;
+        init_t, dfin_t, e1, dd, u, parts, anchor, da_part, total;
 };
 
 BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
@@ -179,6 +179,7 @@ BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
     w.e1 = take(BL * s.H * sizeof(float));
     w.dd = take(BL * s.H * sizeof(float));
     w.u = take(BL * s.H * sizeof(float));
+    w.parts = take(BL * s.H * (size_t)((s.N + 31) / 32) * sizeof(float));
     w.anchor = take((size_t)s.B * (s.nc + 1) * s.H * sizeof(double));
     w.da_part = take((size_t)2 * s.B * s.H * sizeof(double));  // and the parts of dD behind them
     w.total = off;
@@ -440,7 +441,11 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         const int64_t groups = (int64_t)shape.B * shape.G * ((shape.H / shape.G) * (shape.P / 32) / waves);
         return (waves == 8 && groups >= kOnePassMinWorkgroups) || (waves == 2 && groups >= 4 * kOnePassMinWorkgroups);
     };
-    const bool fast_r = one_pass(sR), fast_t = one_pass(sT);
+    // The transposed scans with the sum over a group's heads taken on chip (they write dB and dC themselves): bf16,
+    // headdim 32, eight heads per group, enough workgroups.
+    const bool sum_on_chip = inner != SSD_DTYPE_F32 && ssd::transposed_scan_supported(sT, s.G) &&
+                             (int64_t)s.B * (s.H / 8) * (s.N / 32) >= kOnePassMinWorkgroups;
+    const bool fast_r = one_pass(sR), fast_t = sum_on_chip || one_pass(sT);
     const void *c_heads = Cm, *b_heads = Bm;
     if (!fast_r || !fast_t)
         BWD_LAUNCH(ssd::launch_gather_rows(el, dy, at(w.dy_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather dy");
@@ -485,6 +490,25 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
                         : scan(sR, false, at(w.dy_rev), at(w.c_rev_g), at(w.b_rev_g), dfinal_states, 1, at(w.r_rev),
                                atf(w.gfin), states, false, 0))
         return rc;
+    if (sum_on_chip) {
+        ssd::ScanShape f = sTR;
+        f.mode = 1;
+        f.dt_len = s.L;
+        f.x_groups = s.G;
+        // dB = sum over heads of dt (x . g): the adjoint recurrence with the state transposed; tile states in `states`
+        BWD_LAUNCH(ssd::launch_transposed_scan(f, true, Cm, dt, A, dy, x, nullptr, dfin_t, reset, dB, atf(w.gfin_t), states,
+                                               nullptr, st),
+                   "transposed adjoint scan");
+        f = sT;
+        f.x_groups = s.G;
+        // dC = sum over heads of dy . h: the forward recurrence with the state transposed; tile states in `states2`
+        BWD_LAUNCH(ssd::launch_transposed_scan(f, false, Bm, dt, A, x, dy, Cm, init_t, reset, dC, atf(w.ffin_t), states2,
+                                               atf(w.parts), st),
+                   "transposed forward scan");
+        BWD_LAUNCH(ssd::launch_bwd_rows_parts(s, fast_r ? 0 : Lp, el, x, dy, dt, D, atf(w.r_rev), atf(w.parts), s.N / 32, dx,
+                                              atf(w.e1), atf(w.dd), atf(w.u), st),
+                   "backward rows");
+    } else {
     // yB = x . g: the same recurrence with the state transposed; its chunk states stay in `states`
     const int xg = (fast_t && rep > 1) ? s.G : 0;
     if (int rc = fast_t ? scan(sTR, true, Cm, dy, x, dfin_t, 1, at(w.yb_rev), atf(w.gfin_t), states, true, xg)
@@ -503,6 +527,7 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
                    "backward rows");
         BWD_LAUNCH(ssd::launch_bwd_group_sums(s, fast_t ? 0 : Lp, el, dt, atf(w.yb_rev), atf(w.yc), dB, dC, st),
                    "backward group sums");
+    }
     }
     double *anchor = reinterpret_cast<double *>(base + w.anchor);
     BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, reset, anchor,

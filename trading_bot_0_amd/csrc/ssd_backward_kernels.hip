@@ -176,6 +176,53 @@ __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, 
     }
 }
 
+// The row products when the transposed scans summed dB and dC themselves: four lanes per (b, t, h) row (headdim 32),
+// dx = D dy + dt r, e1 = x . r, dd = dy . x, u = (sum of the parts of C . yC) - dt e1.
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_rows_parts_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                                                             const T *__restrict__ dt, const float *__restrict__ D,
+                                                             const float *__restrict__ r_rev, const float *__restrict__ parts,
+                                                             T *__restrict__ dx, float *__restrict__ e1, float *__restrict__ dd,
+                                                             float *__restrict__ u, ScanShape s, int Lrev, int nparts,
+                                                             long long total) {
+    const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long gid = tid >> 3;
+    if (gid >= total) return;
+    const int piece = (int)(tid & 7) * 8;
+    const int h = (int)(gid % s.H);
+    const long long bt = gid / s.H;
+    const int t = (int)(bt % s.L);
+    const long long b = bt / s.L;
+    const float dtv = (float)dt[gid], dh = D ? D[h] : 0.f;
+    float se1 = 0.f, sdd = 0.f;
+    if (piece < s.P) {
+        const size_t row = (size_t)gid * s.P + piece;
+        const size_t rrow = (Lrev ? ((size_t)(b * Lrev + (Lrev - 1 - t)) * s.H + h) * s.P : (size_t)gid * s.P) + piece;
+        const Row8<T> xv = Row8<T>::load(x + row), dv = Row8<T>::load(dy + row);
+        const Row8<float> rv = Row8<float>::load(r_rev + rrow);
+        Row8<T> o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            o.v[i] = dh * dv.v[i] + dtv * rv.v[i];
+            se1 += xv.v[i] * rv.v[i];
+            sdd += dv.v[i] * xv.v[i];
+        }
+        o.store(dx + row);
+    }
+#pragma unroll
+    for (int m = 1; m < 8; m <<= 1) {
+        se1 += __shfl_xor(se1, m, 8);
+        sdd += __shfl_xor(sdd, m, 8);
+    }
+    if (piece == 0) {
+        float sc = 0.f;
+        for (int k = 0; k < nparts; ++k) sc += parts[(size_t)gid * nparts + k];
+        e1[gid] = se1;
+        dd[gid] = sdd;
+        u[gid] = sc - dtv * se1;
+    }
+}
+
 // One thread per (b, t, g, 8 state columns): dB = sum over the group's heads of dt yB, dC = the same of yC.
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_group_sums_kernel(const T *__restrict__ dt, const float *__restrict__ yB_rev,
@@ -417,6 +464,21 @@ hipError_t launch_gather_rows(int dtype, const void *src, void *dst, int B, int 
 hipError_t launch_transpose_state(const float *src, float *dst, long long BH, int P, int N, hipStream_t st) {
     const long long total = BH * P * N;
     transpose_state_kernel<<<dim3(blocks_for(total)), dim3(256), 0, st>>>(src, dst, P, N, total);
+    return hipGetLastError();
+}
+
+hipError_t launch_bwd_rows_parts(const ScanShape &s, int Lrev, int dtype, const void *x, const void *dy, const void *dt,
+                                 const float *D, const float *r_rev, const float *parts, int nparts, void *dx,
+                                 float *e1, float *dd, float *u, hipStream_t st) {
+    const long long total = (long long)s.B * s.L * s.H;
+    if (dtype)
+        bwd_rows_parts_kernel<__bf16><<<dim3(blocks_for(total * 8)), dim3(256), 0, st>>>(
+            static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dy), static_cast<const __bf16 *>(dt), D, r_rev, parts,
+            static_cast<__bf16 *>(dx), e1, dd, u, s, Lrev, nparts, total);
+    else
+        bwd_rows_parts_kernel<float><<<dim3(blocks_for(total * 8)), dim3(256), 0, st>>>(
+            static_cast<const float *>(x), static_cast<const float *>(dy), static_cast<const float *>(dt), D, r_rev, parts,
+            static_cast<float *>(dx), e1, dd, u, s, Lrev, nparts, total);
     return hipGetLastError();
 }
 

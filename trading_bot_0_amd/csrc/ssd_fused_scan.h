@@ -118,14 +118,29 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
 // KIND 0: the forward.  KIND 1: the reversed-adjoint recurrence of the backward pass.  KIND 2: states only --
 // no outputs, no C: the state a segment of the sequence leaves behind (from its own initial state) and the
 // segment's total decay, for sequences cut into segments that run side by side.
+// KIND 3 and 4: the backward pass's two scans of the transposed state (3 forward in time, 4 reversed-adjoint).
+// There B and C are per head and x is shared by the heads of a group, the opposite of the forward, so a
+// workgroup is eight heads on one 32-column slice of x: every wave stages its own B and C tile, the x tile is
+// shared, and instead of writing y per head the waves add their tiles in LDS and the workgroup writes the sum
+// over its heads (dC, or dB with the heads' dt as weights) -- the per-head outputs never reach memory.  KIND 3
+// also writes, per head, the part of C_t . y_t that its slice holds.
+// LDS of a workgroup of the transposed scans: a B and a C tile per wave (eight waves), the shared x tile and
+// second-operand tile, the per-wave tables, and a [Q][33] float tile per wave for the heads' outputs (summed in a
+// fixed order when the workgroup writes them out, so that results do not depend on timing).
+constexpr size_t transposed_scan_lds_bytes(int Q) {
+    return (size_t)(2 * 8 + 2) * fused_scan_xtile_elems(Q) * 2 + (size_t)8 * ((5 + Q / 32) * Q * 4 + 64) +
+           (size_t)8 * Q * 33 * 4;
+}
+
 template <typename TO, int NK, int QB, int WAVES, int KIND>  // N = 16*NK, Q = 32*QB
 __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void fused_scan_kernel(
     const __bf16 *__restrict__ x, const __bf16 *__restrict__ dt, const float *__restrict__ A,
     const __bf16 *__restrict__ Bm, const __bf16 *__restrict__ Cm, const float *__restrict__ D,
     const float *init, const unsigned char *__restrict__ reset, TO *__restrict__ y, float *final_states,
-    float *tile_states, float *seg_decay, ScanShape s) {
+    float *tile_states, float *seg_decay, const __bf16 *__restrict__ aux, ScanShape s) {
     using T = __bf16;
-    constexpr bool ADJ = KIND == 1, STATES_ONLY = KIND == 2;
+    constexpr bool ADJ = KIND == 1 || KIND == 4, STATES_ONLY = KIND == 2, TR = KIND >= 3;
+    static_assert(!TR || (NK == 2 && WAVES == 8), "the transposed scans: 32-wide state, eight heads per workgroup");
     constexpr int N = 16 * NK, NB = NK / 2, Q = 32 * QB, nthr = 64 * WAVES;
     constexpr int EPL = Q >= 64 ? Q / 64 : 1;  // chunk positions per lane in the scan
     constexpr int BPR = N / 8;                 // 16-byte pieces per B (or C) row
@@ -139,17 +154,23 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     using XT = ChunkTile<32>;
     using BT = ChunkTile<N>;
     // static, so that LDS addresses are compile-time offsets
-    __shared__ __attribute__((aligned(16))) unsigned char smem[fused_scan_lds_bytes(N, Q, WAVES)];
-    T *Bs = reinterpret_cast<T *>(smem);  // [Q][N]
-    T *Cs = Bs + Q * N;                   // [Q][N]
-    T *xs_all = Cs + Q * N;               // [WAVES][Q][32] (+16 elements between tiles)
     constexpr int XS = fused_scan_xtile_elems(Q);
-
+    __shared__ __attribute__((aligned(16))) unsigned char smem[TR ? transposed_scan_lds_bytes(Q) : fused_scan_lds_bytes(N, Q, WAVES)];
     const int tid = threadIdx.x;
     const int lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    T *xs = xs_all + wave * XS;
-    float *wf = reinterpret_cast<float *>(xs_all + WAVES * XS) + wave * ((5 + QB) * Q + 16);
+    // forward: B and C tiles [Q][N] of the workgroup, then one x tile [Q][32] per wave (+16 elements between tiles).
+    // transposed: a B and a C tile [Q][32] per wave, then the shared x tile and the shared tile of the second
+    // operand of the C . y products, each [Q][32].
+    T *tiles = reinterpret_cast<T *>(smem);
+    T *Bs = TR ? tiles + wave * XS : tiles;
+    T *Cs = TR ? tiles + (WAVES + wave) * XS : tiles + Q * N;
+    T *xs_all = TR ? tiles + 2 * WAVES * XS : tiles + 2 * Q * N;
+    T *xs = TR ? xs_all : xs_all + wave * XS;
+    T *aux_s = xs_all + XS;  // transposed only
+    float *wf0 = reinterpret_cast<float *>(TR ? xs_all + 2 * XS : xs_all + WAVES * XS);
+    float *wf = wf0 + wave * ((5 + QB) * Q + 16);
+    float *red = wf0 + WAVES * ((5 + QB) * Q + 16);  // transposed only: [WAVES][Q][33], every head's output tile
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
     float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [8..8+QB): log2-decay across block lb
 
@@ -163,23 +184,31 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     const int seg = slot % S, logical = slot / S;
     const int c_first = seg * (s.seg_tiles > 0 ? s.seg_tiles : s.nc);
     const int c_end = s.seg_tiles > 0 ? min(s.nc, c_first + s.seg_tiles) : s.nc;
-    const int b = logical / (s.G * UW);
-    const int g = (logical / UW) % s.G;
-    const int unit0 = (logical % UW) * WAVES;
+    // transposed: the workgroup is heads h0 .. h0+7 (one per wave) on x slice pb; s.G == s.H there, and
+    // s.x_groups says how many groups of heads x is given for
+    const int TW = TR ? (s.H / 8) * PBn : 1;  // transposed workgroups per batch row
+    const int b = TR ? logical / TW : logical / (s.G * UW);
+    const int g = TR ? 0 : (logical / UW) % s.G;
+    const int unit0 = TR ? 0 : (logical % UW) * WAVES;
     const int unit = unit0 + wave;
-    const int h = g * HG + unit / PBn, pb = unit % PBn;
+    const int h0 = TR ? ((logical % TW) / PBn) * 8 : 0;
+    const int h = TR ? h0 + wave : g * HG + unit / PBn;
+    const int pb = TR ? (logical % TW) % PBn : unit % PBn;
     const int xcol0 = g * HG * s.P + unit0 * 32;  // first element of the workgroup's slice of an x row
     const int HP = s.H * s.P;
     // x rows: one per timestep, HP wide -- or, when x is shared by groups of heads (s.x_groups, with G == H so
-    // that the workgroup is one head), x_groups * P wide with this head's group's columns
+    // that the workgroup is one head, or eight heads of one group in the transposed scans), x_groups * P wide
+    // with this group's columns
     const int XLD = s.x_groups ? s.x_groups * s.P : HP;
-    const int xcol = s.x_groups ? (h / (s.H / s.x_groups)) * s.P + (unit0 % PBn) * 32 : xcol0;
+    const int xcol = TR ? (h0 / (s.H / s.x_groups)) * s.P + pb * 32
+                        : (s.x_groups ? (h / (s.H / s.x_groups)) * s.P + (unit0 % PBn) * 32 : xcol0);
     // ADJ: x, B, C, dt, the reset mask and y are the forward sequence's tensors, dt_len rows per batch row, and row
     // tau of the scan is their row L - 1 - tau (rows outside them are no-op steps in front of the reversed sequence)
     const int trows = ADJ ? s.dt_len : s.L;
     const T *xb = x + (size_t)b * trows * XLD + xcol;
-    const T *Bb = Bm + ((size_t)b * trows * s.G + g) * N;
-    const T *Cb = Cm + ((size_t)b * trows * s.G + g) * N;
+    const T *Bb = Bm + ((size_t)b * trows * s.G + (TR ? h0 : g)) * N;  // transposed: eight heads' rows side by side
+    const T *Cb = Cm + ((size_t)b * trows * s.G + (TR ? h0 : g)) * N;
+    const T *auxb = TR && aux ? aux + (size_t)b * trows * XLD + xcol : nullptr;
     // mode 1 (the time-reversed adjoint recurrence): step t decays by the dt of step L - t of a dt tensor of
     // dt_len rows, steps outside it do not decay, and every step's input weighs one instead of dt
     const int dt_rows = ADJ ? s.dt_len : s.L;
@@ -206,7 +235,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // hold no registers through phase 1), or, for the two-wave workgroups, whose per-head B and C rows are short
     // and slow to arrive, before phase 1.
     constexpr bool kEarlyPrefetch = WAVES == 2;
-    uint4 bq[UBC], cq[UBC], xq[UX];
+    // (transposed: UX passes of the eight heads' B and C rows, one piece of the shared x tile and of the second
+    // operand's tile)
+    uint4 bq[TR ? UX : UBC], cq[TR ? UX : UBC], xq[TR ? 1 : UX], auxq = make_uint4(0, 0, 0, 0);
     unsigned short dq[EPL];
     unsigned char rq[EPL];
     auto prefetch = [&](int c) {
@@ -244,7 +275,33 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             if (ok) v = *reinterpret_cast<const uint4 *>(ptr);
             return v;
         };
-        if (ADJ) {
+        if constexpr (TR) {
+            const int prow = tv / XPR, srow = tv / 4;
+            const unsigned pcol = (tv % XPR) * 8, scol = (tv % 4) * 8;
+            auto source = [&](int row, bool &ok) {  // the tensors' row of this tile's row `row`
+                const int src = ADJ ? s.L - 1 - t0 - row : t0 + row;
+                ok = ADJ ? (src >= 0 && src < trows) : row < rows;
+                return src;
+            };
+#pragma unroll
+            for (int u = 0; u < UX; ++u) {
+                bool ok;
+                const int src = source(prow + 16 * u, ok);
+                bq[u] = ld16(Bb + (size_t)src * s.G * N + pcol, ok);
+                cq[u] = ld16(Cb + (size_t)src * s.G * N + pcol, ok);
+            }
+            {
+                bool ok;
+                const int src = source(srow, ok);
+                ok = ok && tv < Q * 4;
+                xq[0] = ld16(xb + (size_t)src * XLD + scol, ok);
+                if (auxb != nullptr) auxq = ld16(auxb + (size_t)src * XLD + scol, ok);
+            }
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) dq[e] = dt_bits(e, (tv & 63) * EPL + e < rows);
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) rq[e] = reset_byte(e, (tv & 63) * EPL + e < rows);
+        } else if (ADJ) {
             const int first = s.L - 1 - t0;  // the tensors' row of this tile's first row; later rows count down
 #pragma unroll
             for (int u = 0; u < UBC; ++u) {
@@ -345,8 +402,22 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             for (int par = 0; par < 2; ++par)
                 xw[par][hf] = ((tw % XPR) / 4) * XS + XT::off(tw / XPR + 16 * par, ((tw % XPR) % 4) * 8 + 4 * hf);
         }
+        if constexpr (TR) {
 #pragma unroll
-        for (int u = 0; u < UBC; ++u) {
+            for (int u = 0; u < UX; ++u) {  // the eight heads' B and C rows, as the forward stages its x rows
+                T *tb = tiles + xw[u & 1][0] + (u >> 1) * 1024, *tb1 = tiles + xw[u & 1][1] + (u >> 1) * 1024;
+                *reinterpret_cast<uint2 *>(tb) = make_uint2(bq[u].x, bq[u].y);
+                *reinterpret_cast<uint2 *>(tb1) = make_uint2(bq[u].z, bq[u].w);
+                *reinterpret_cast<uint2 *>(tb + WAVES * XS) = make_uint2(cq[u].x, cq[u].y);
+                *reinterpret_cast<uint2 *>(tb1 + WAVES * XS) = make_uint2(cq[u].z, cq[u].w);
+            }
+            if (tw < Q * 4) {
+                XT::put16(xs_all, tw / 4, (tw % 4) * 8, xq[0]);
+                XT::put16(aux_s, tw / 4, (tw % 4) * 8, auxq);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < (TR ? 0 : UBC); ++u) {
             if (BSL % nthr == 0 || tw + u * nthr < BSL) {
                 const int o0 = kSharedBcOffsets ? bw[0] + u * BRP * N : BT::off(tw / BPR + u * BRP, (tw % BPR) * 8);
                 const int o1 = kSharedBcOffsets ? bw[1] + u * BRP * N : BT::off(tw / BPR + u * BRP, (tw % BPR) * 8 + 4);
@@ -359,7 +430,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             }
         }
 #pragma unroll
-        for (int u = 0; u < UX; ++u) {
+        for (int u = 0; u < (TR ? 0 : UX); ++u) {
             *reinterpret_cast<uint2 *>(xs_all + xw[u & 1][0] + (u >> 1) * 1024) = make_uint2(xq[u].x, xq[u].y);
             *reinterpret_cast<uint2 *>(xs_all + xw[u & 1][1] + (u >> 1) * 1024) = make_uint2(xq[u].z, xq[u].w);
         }
@@ -530,8 +601,31 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 for (int sb = 0; sb < QB - 1; ++sb)
                     if (sb < lb) block(sb, false);
                 block(lb, true);
-                // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]
-                {
+                if constexpr (TR) {
+                    // this head's tile goes into the workgroup's sum; acc[4 vg + i] is element (t = 32 lb + lane%32,
+                    // p = 8 vg + 4 half + i)
+                    const int le = phase_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
+                    const int trow = ADJ ? s.L - 1 - (t0 + ll) : t0 + ll;
+                    const bool live = ll < rows && trow >= 0 && trow < trows;
+                    float wt = 1.f;  // KIND 4: dB sums the heads' outputs weighted by their dt
+                    if (KIND == 4) wt = live ? (float)dt[((size_t)b * trows + trow) * s.H + h] : 0.f;
+                    float part = 0.f;  // KIND 3: this slice's part of C_t . y_t
+#pragma unroll
+                    for (int vg = 0; vg < 4; ++vg) {
+                        if (KIND == 3 && aux != nullptr) {
+                            const bf16x4 c4 = XT::row4(aux_s, ll, 8 * vg + 4 * he);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) part += acc[vg * 4 + i] * (float)c4[i];
+                        }
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) red[(wave * Q + ll) * 33 + 8 * vg + 4 * he + i] = wt * acc[vg * 4 + i];
+                    }
+                    if (KIND == 3 && seg_decay != nullptr) {  // (seg_decay: the per-head parts [B, L, H, P/32])
+                        part += __shfl_xor(part, 32, 64);
+                        if (he == 0 && live) seg_decay[(((size_t)b * trows + trow) * s.H + h) * PBn + pb] = part;
+                    }
+                } else {
+                    // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]
                     const int le = phase_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
                     float o[16];
 #pragma unroll
@@ -546,6 +640,31 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             }
         }
 
+        if constexpr (TR) {
+            // the sum over the workgroup's heads (a whole group: eight heads) of this tile's outputs, [Q][32], goes
+            // to the group's rows of the gradient
+            block_sync_lds();
+            const int tq = phase_tid();
+            const int ll = tq >> 3, p4 = (tq & 7) * 4;
+            float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < WAVES; ++wv) {  // heads in order
+                const float *rr = red + (wv * Q + ll) * 33 + p4;
+                v0 += rr[0];
+                v1 += rr[1];
+                v2 += rr[2];
+                v3 += rr[3];
+            }
+            const int trow = ADJ ? s.L - 1 - (t0 + ll) : t0 + ll;
+            if (ll < rows && trow >= 0 && trow < trows) {
+                TO *dst = y + ((size_t)b * trows + trow) * XLD + xcol + p4;
+                if constexpr (sizeof(TO) == 2) {
+                    *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_bf16x2(v0, v1), pack_bf16x2(v2, v3));
+                } else {
+                    *reinterpret_cast<float4 *>(dst) = make_float4(v0, v1, v2, v3);
+                }
+            }
+        }
         // ---- phase 2: the state leaving this chunk ----
         if (!kEarlyPrefetch && c + 1 < c_end) prefetch(c + 1);
         seg_total *= a_end;
@@ -622,14 +741,14 @@ static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt
         if constexpr (sizeof(TO) == 4) {
             if (segments != 1) return hipErrorInvalidValue;
             fused_scan_kernel<TO, NK, QB, WAVES, 1><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, s);
+                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, nullptr, s);
             return hipGetLastError();
         } else {
             return hipErrorInvalidValue;
         }
     }
     fused_scan_kernel<TO, NK, QB, WAVES, 0><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, s);
+        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, nullptr, s);
     return hipGetLastError();
 }
 
@@ -645,7 +764,26 @@ static hipError_t fused_launch_states(const ScanShape &s, const void *x, const v
     const __bf16 *bb = static_cast<const __bf16 *>(Bm);
     fused_scan_kernel<__bf16, NK, QB, WAVES, 2><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
         static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, bb, bb, nullptr, init, reset, nullptr, seg_states,
-        nullptr, seg_decay, s);
+        nullptr, seg_decay, nullptr, s);
+    return hipGetLastError();
+}
+
+// The backward pass's scans of the transposed state (KIND 3 forward in time, 4 reversed-adjoint): s is the
+// transposed shape (P = the forward's dstate, N = 32 = its headdim, G = H), x [B,L,x_groups,P] the operand the
+// heads of a group share, Bm, Cm [B,L,H,32] per head; out [B,L,x_groups,P] receives the sum over each group's
+// eight heads of the per-head outputs (weighted by dt in KIND 4); KIND 3 also writes, per head and 32-column
+// slice, aux_t . y_t into parts [B,L,H,P/32] (aux [B,L,x_groups,P]).
+template <typename TO, int KIND>
+static hipError_t fused_launch_transposed(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
+                                          const void *Cm, const void *aux, const float *init, const unsigned char *reset,
+                                          void *out, float *final_states, float *tile_states, float *parts, hipStream_t st) {
+    if (s.N != 32 || s.G != s.H || s.x_groups <= 0 || s.H != 8 * s.x_groups || s.P % 32 != 0 || s.seg_tiles != 0)
+        return hipErrorInvalidValue;
+    const int grid = s.B * (s.H / 8) * (s.P / 32);
+    fused_scan_kernel<TO, 2, kOnePassTile / 32, 8, KIND><<<dim3(grid), dim3(512), 0, st>>>(
+        static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
+        static_cast<const __bf16 *>(Cm), nullptr, init, reset, static_cast<TO *>(out), final_states, tile_states, parts,
+        static_cast<const __bf16 *>(aux), s);
     return hipGetLastError();
 }
 

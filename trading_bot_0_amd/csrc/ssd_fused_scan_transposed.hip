@@ -1,0 +1,25 @@
+// The backward pass's two scans of the transposed state on the one-pass kernel's transposed kinds: eight heads
+// per workgroup, the sum over a group's heads taken in LDS, bf16 gradients written directly.
+#include "ssd_fused_scan.h"
+
+namespace ssd {
+
+bool transposed_scan_supported(const ScanShape &sT, int x_groups) {
+    return sT.N == 32 && sT.G == sT.H && x_groups > 0 && sT.H == 8 * x_groups && sT.P % 32 == 0 && sT.P <= 64 &&
+           sT.Q == kOnePassTile;
+}
+
+hipError_t launch_transposed_scan(const ScanShape &sT, bool adjoint, const void *x, const void *dt, const float *A,
+                                  const void *Bm, const void *Cm, const void *aux, const float *init,
+                                  const unsigned char *reset, void *out, float *final_states, float *tile_states,
+                                  float *parts, hipStream_t st) {
+    ScanShape t = sT;
+    t.Q = kOnePassTile;
+    t.nc = (sT.L + kOnePassTile - 1) / kOnePassTile;
+    return adjoint ? fused_launch_transposed<__bf16, 4>(t, x, dt, A, Bm, Cm, nullptr, init, reset, out, final_states,
+                                                        tile_states, nullptr, st)
+                   : fused_launch_transposed<__bf16, 3>(t, x, dt, A, Bm, Cm, aux, init, reset, out, final_states,
+                                                        tile_states, parts, st);
+}
+
+}  // namespace ssd

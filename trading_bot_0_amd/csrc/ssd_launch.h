@@ -105,6 +105,18 @@ hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, 
 hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                              float eps, void *out, hipStream_t stream);
 
+// The backward pass's two scans of the transposed state with the sum over a group's heads taken on chip (bf16,
+// headdim 32, eight heads per group; sT is the transposed shape: P = dstate, N = 32, G = H; sT.mode / dt_len as
+// for the one-pass kernel when adjoint).  x [B,L,x_groups,P] is the operand a group's heads share, Bm and Cm
+// [B,L,H,32] are per head.  out [B,L,x_groups,P] (bf16) = the sum over each group's heads of the per-head
+// outputs, weighted by the heads' dt when adjoint.  Forward in time it also writes parts [B,L,H,P/32]: per head
+// and 32-column slice, aux_t . y_t (aux [B,L,x_groups,P]).  tile_states / final_states as for the one-pass kernel.
+bool transposed_scan_supported(const ScanShape &sT, int x_groups);
+hipError_t launch_transposed_scan(const ScanShape &sT, bool adjoint, const void *x, const void *dt, const float *A,
+                                  const void *Bm, const void *Cm, const void *aux, const float *init,
+                                  const unsigned char *reset, void *out, float *final_states, float *tile_states,
+                                  float *parts, hipStream_t stream);
+
 // The memory-bound kernels of the backward pass (its three heavy products run on the stage launchers above with
 // the operands' roles swapped).  dtype: 0 = float32, 1 = bf16 activations and gradients.
 // gather_rows: dst[b, t', (g*rep + k)*W + w] = src[b, t, g*W + w] for t' < Ldst, with t = Ldst-1-t' if reverse
@@ -122,6 +134,11 @@ hipError_t launch_bwd_rows(const ScanShape &s, int Lrev, int dtype, const void *
                            const float *D, const float *r_rev, const float *yC, void *dx, float *e1, float *dd,
                            float *u, hipStream_t stream, const float *yB_rev = nullptr, int LrevB = 0,
                            void *dB = nullptr, void *dC = nullptr);
+// The same without the transposed scans' per-head outputs: C . yC comes as parts [B,L,H,nparts] to add up
+// (launch_transposed_scan wrote them, and dB and dC).
+hipError_t launch_bwd_rows_parts(const ScanShape &s, int Lrev, int dtype, const void *x, const void *dy, const void *dt,
+                                 const float *D, const float *r_rev, const float *parts, int nparts, void *dx,
+                                 float *e1, float *dd, float *u, hipStream_t stream);
 // dB = sum over a group's heads of dt yB (yB_rev time-reversed), dC = the same of yC
 hipError_t launch_bwd_group_sums(const ScanShape &s, int Lrev, int dtype, const void *dt, const float *yB_rev, const float *yC,
                                  void *dB, void *dC, hipStream_t stream);
