@@ -197,6 +197,18 @@ def test_gradients_with_restarts_inside_the_sequence(dtype, seqlen):
     assert got["dinitial_states"][1].abs().max().item() == 0.0
 
 
+@pytest.mark.parametrize("w", [
+    Workload("bwd_sums_two_groups", 64, 150, 16, 32, 32, 2, 128, dtype="bf16", init_std=0.5),
+    Workload("bwd_sums_ragged", 96, 129, 8, 32, 64, 1, 64, dtype="bf16", init_std=0.5),
+    Workload("bwd_sums_short", 100, 5, 8, 32, 64, 1, 64, dtype="bf16", init_std=0.5),
+], ids=lambda w: w.name)
+@pytest.mark.parametrize("with_D,with_init,with_dfinal", [(True, True, True), (False, False, False)])
+def test_head_sums_taken_on_chip(w, with_D, with_init, with_dfinal):
+    """Batches of eight-head groups large enough for the scans that add a group's heads themselves: every
+    gradient of every row, with and without the optional operands, ragged last tiles, two groups."""
+    run_case(w, seed=21, with_D=with_D, with_init=with_init, with_dfinal=with_dfinal)
+
+
 def test_restarts_on_the_one_pass_adjoint_scan():
     """Enough bf16 sequences for the adjoint recurrence to take the one-pass kernel: rows against the oracle."""
     w = Workload("bwd_reset_onepass", 96, 200, 8, 32, 64, 1, 128, dtype="bf16")
