@@ -176,7 +176,7 @@ BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
     w.ffin_t = take(st);
     w.init_t = take(st);
     w.dfin_t = take(st);
-    w.e1 = take(BL * s.H * sizeof(float));
+    w.e1 = take(2 * BL * s.H * sizeof(float));  // or the (e1, dd) pairs of the adjoint scan with row products
     w.dd = take(BL * s.H * sizeof(float));
     w.u = take(BL * s.H * sizeof(float));
     w.parts = take(BL * s.H * (size_t)((s.N + 31) / 32) * sizeof(float));
@@ -446,6 +446,8 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     const bool sum_on_chip = inner != SSD_DTYPE_F32 && ssd::transposed_scan_supported(sT, s.G) &&
                              (int64_t)s.B * (s.H / 8) * (s.N / 32) >= kOnePassMinWorkgroups;
     const bool fast_r = one_pass(sR), fast_t = sum_on_chip || one_pass(sT);
+    // the adjoint scan with the row products in its epilogue (it writes dx; no float r, no row kernel)
+    const bool rows_in_scan = sum_on_chip && fast_r && ssd::adjoint_rows_scan_supported(sR);
     const void *c_heads = Cm, *b_heads = Bm;
     if (!fast_r || !fast_t)
         BWD_LAUNCH(ssd::launch_gather_rows(el, dy, at(w.dy_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather dy");
@@ -486,7 +488,13 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         return run_staged(shape, inner, sx, dt, A, sb, sc, nullptr, sinit, reset, mode, sy, sfinal, dtcs, sstates, st, s.L);
     };
     // r = g B: the adjoint recurrence, reversed in time; its last state is g_0
-    if (int rc = fast_r ? scan(sR, true, dy, Cm, Bm, dfinal_states, 1, at(w.r_rev), atf(w.gfin), states, false, 0)
+    if (rows_in_scan) {
+        ssd::ScanShape f = sR;
+        f.mode = 1;
+        f.dt_len = s.L;
+        BWD_LAUNCH(ssd::launch_adjoint_rows_scan(f, dy, dt, A, Cm, Bm, D, x, dfinal_states, reset, dx, atf(w.gfin), atf(w.e1), st),
+                   "adjoint scan with row products");
+    } else if (int rc = fast_r ? scan(sR, true, dy, Cm, Bm, dfinal_states, 1, at(w.r_rev), atf(w.gfin), states, false, 0)
                         : scan(sR, false, at(w.dy_rev), at(w.c_rev_g), at(w.b_rev_g), dfinal_states, 1, at(w.r_rev),
                                atf(w.gfin), states, false, 0))
         return rc;
@@ -505,9 +513,10 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         BWD_LAUNCH(ssd::launch_transposed_scan(f, false, Bm, dt, A, x, dy, Cm, init_t, reset, dC, atf(w.ffin_t), states2,
                                                atf(w.parts), st),
                    "transposed forward scan");
-        BWD_LAUNCH(ssd::launch_bwd_rows_parts(s, fast_r ? 0 : Lp, el, x, dy, dt, D, atf(w.r_rev), atf(w.parts), s.N / 32, dx,
-                                              atf(w.e1), atf(w.dd), atf(w.u), st),
-                   "backward rows");
+        if (!rows_in_scan)
+            BWD_LAUNCH(ssd::launch_bwd_rows_parts(s, fast_r ? 0 : Lp, el, x, dy, dt, D, atf(w.r_rev), atf(w.parts), s.N / 32, dx,
+                                                  atf(w.e1), atf(w.dd), atf(w.u), st),
+                       "backward rows");
     } else {
     // yB = x . g: the same recurrence with the state transposed; its chunk states stay in `states`
     const int xg = (fast_t && rep > 1) ? s.G : 0;
@@ -535,7 +544,8 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
                "backward anchors");
     double *da_part = reinterpret_cast<double *>(base + w.da_part);
     double *dd_part = da_part + (size_t)s.B * s.H;
-    BWD_LAUNCH(ssd::launch_bwd_ddt(s, el, dt, A, atf(w.e1), atf(w.u), atf(w.dd), anchor, ddt, da_part, dd_part, st),
+    BWD_LAUNCH(ssd::launch_bwd_ddt(s, el, dt, A, atf(w.e1), atf(w.u), atf(w.dd), anchor, ddt, da_part, dd_part, st,
+                                   rows_in_scan ? atf(w.parts) : nullptr, s.N / 32),
                "backward ddt");
     BWD_LAUNCH(ssd::launch_bwd_head_sums(s, da_part, dd_part, dA, dD, st), "backward head sums");
     if (dinitial_states != nullptr)

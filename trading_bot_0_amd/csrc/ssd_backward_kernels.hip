@@ -313,7 +313,8 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
                                                       const float *__restrict__ e1, const float *__restrict__ u,
                                                       const float *__restrict__ dd, const double *__restrict__ anchor,
                                                       T *__restrict__ ddt, double *__restrict__ dA_part,
-                                                      double *__restrict__ dD_part, ScanShape s) {
+                                                      double *__restrict__ dD_part, ScanShape s,
+                                                      const float *__restrict__ parts, int nparts) {
     const int lane = threadIdx.x & 63;
     const long long bh = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (bh >= (long long)s.B * s.H) return;
@@ -331,14 +332,30 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
         const int t0 = c * s.Q, len = min(s.Q, s.L - t0);
         const bool ok = lane < len;
         const size_t at = ((size_t)b * s.L + t0 + (ok ? lane : 0)) * s.H + h;
-        const double uv = ok ? (double)u[at] : 0.0;
+        float e1v = 0.f, ddv = 0.f, dtv = 0.f, uf = 0.f;
+        if (ok) {
+            dtv = (float)dt[at];
+            if (parts != nullptr) {  // (e1, dd) pairs; u from the pieces of C . yC
+                const float2 pr = *reinterpret_cast<const float2 *>(e1 + 2 * at);
+                e1v = pr.x;
+                ddv = pr.y;
+                float sc = 0.f;
+                for (int k = 0; k < nparts; ++k) sc += parts[at * nparts + k];
+                uf = sc - dtv * e1v;
+            } else {
+                e1v = e1[at];
+                ddv = dd[at];
+                uf = u[at];
+            }
+        }
+        const double uv = (double)uf;
         const double incl = wave_inclusive_scan(uv);
         const double mismatch = q0 - last_lane(incl) - q1;
         if (ok) {
             const double q = q0 - (incl - uv) - mismatch * (double)lane / (double)len;
-            ddt[at] = (T)(float)((double)e1[at] + a * q);
-            da += (double)(float)dt[at] * q;
-            sdd += (double)dd[at];
+            ddt[at] = (T)(float)((double)e1v + a * q);
+            da += (double)dtv * q;
+            sdd += (double)ddv;
         }
     }
     const double tot = last_lane(wave_inclusive_scan(da)), totd = last_lane(wave_inclusive_scan(sdd));
@@ -437,11 +454,13 @@ hipError_t anchors_t(const ScanShape &s, const void *dt, const float *A, const f
 
 template <typename T>
 hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float *e1, const float *u, const float *dd,
-                 const double *anchor, void *ddt, double *dA_part, double *dD_part, hipStream_t st) {
+                 const double *anchor, void *ddt, double *dA_part, double *dD_part, const float *parts, int nparts,
+                 hipStream_t st) {
     if (s.Q > 64) return hipErrorInvalidValue;  // one pass of the wave per chunk
     const long long waves = (long long)s.B * s.H;
     bwd_ddt_kernel<T><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, e1, u, dd, anchor,
-                                                                              static_cast<T *>(ddt), dA_part, dD_part, s);
+                                                                              static_cast<T *>(ddt), dA_part, dD_part, s, parts,
+                                                                              nparts);
     return hipGetLastError();
 }
 
@@ -510,9 +529,9 @@ hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, con
 
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
                           const float *dd, const double *anchor, void *ddt, double *dA_part, double *dD_part,
-                          hipStream_t st) {
-    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, st)
-                 : ddt_t<float>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, st);
+                          hipStream_t st, const float *parts, int nparts) {
+    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, st)
+                 : ddt_t<float>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, st);
 }
 
 hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,

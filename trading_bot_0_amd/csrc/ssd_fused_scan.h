@@ -124,6 +124,10 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
 // shared, and instead of writing y per head the waves add their tiles in LDS and the workgroup writes the sum
 // over its heads (dC, or dB with the heads' dt as weights) -- the per-head outputs never reach memory.  KIND 3
 // also writes, per head, the part of C_t . y_t that its slice holds.
+// KIND 5: the reversed-adjoint scan of the backward pass with the row products in its epilogue (headdim 32: a wave
+// holds a head's whole row).  With r_t the recurrence's output it writes dx_t = dt_t r_t + D x_t (x being the
+// scan's x operand, dy) instead of r, and per (b, t, h) the pair (aux_t . r_t, aux_t . x_t) -- aux is the forward's
+// x, so these are e1 = x . r and dd = dy . x -- into seg_decay as float2 [B, L, H].
 // LDS of a workgroup of the transposed scans: a B and a C tile per wave (eight waves), the shared x tile and
 // second-operand tile, the per-wave tables, and a [Q][33] float tile per wave for the heads' outputs (summed in a
 // fixed order when the workgroup writes them out, so that results do not depend on timing).
@@ -139,7 +143,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     const float *init, const unsigned char *__restrict__ reset, TO *__restrict__ y, float *final_states,
     float *tile_states, float *seg_decay, const __bf16 *__restrict__ aux, ScanShape s) {
     using T = __bf16;
-    constexpr bool ADJ = KIND == 1 || KIND == 4, STATES_ONLY = KIND == 2, TR = KIND >= 3;
+    constexpr bool ADJ = KIND == 1 || KIND == 4 || KIND == 5, STATES_ONLY = KIND == 2, TR = KIND == 3 || KIND == 4;
+    constexpr bool ROWS = KIND == 5;
     static_assert(!TR || (NK == 2 && WAVES == 8), "the transposed scans: 32-wide state, eight heads per workgroup");
     constexpr int N = 16 * NK, NB = NK / 2, Q = 32 * QB, nthr = 64 * WAVES;
     constexpr int EPL = Q >= 64 ? Q / 64 : 1;  // chunk positions per lane in the scan
@@ -537,6 +542,19 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 const int l = lb * 32 + r;
                 // non-negative floats order like their bit patterns: a scalar compare
                 const bool fast = __builtin_amdgcn_readfirstlane(__float_as_int(blk_s[8 + lb])) <= __float_as_int(kFastDiagSpan);
+                // KIND 5: this lane's pieces of the second operand's rows and the rows' dt, requested here and used in
+                // the epilogue (lane = (row l, half): elements 8 vg + 4 half .. + 3 of the head's row)
+                uint2 aq[4] = {make_uint2(0, 0), make_uint2(0, 0), make_uint2(0, 0), make_uint2(0, 0)};
+                float wt = 0.f;
+                if constexpr (ROWS) {
+                    const int arow = s.L - 1 - (t0 + l);
+                    if (l < rows && arow >= 0 && arow < trows) {
+                        const T *ar = aux + ((size_t)b * trows + arow) * HP + h * s.P + pb * 32 + 4 * half;
+#pragma unroll
+                        for (int vg = 0; vg < 4; ++vg) aq[vg] = *reinterpret_cast<const uint2 *>(ar + 8 * vg);
+                        wt = (float)dt[((size_t)b * trows + arow) * s.H + h];
+                    }
+                }
                 Frag<T> Cf[NK];
 #pragma unroll
                 for (int kk = 0; kk < NK; ++kk) Cf[kk] = BT::split_frag(Cs, l, 16 * kk + 4 * half);
@@ -624,6 +642,28 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                         part += __shfl_xor(part, 32, 64);
                         if (he == 0 && live) seg_decay[(((size_t)b * trows + trow) * s.H + h) * PBn + pb] = part;
                     }
+                } else if constexpr (ROWS) {
+                    // epilogue: dx[t, h, p] = dt[t, h] * rT[p, l] + D[h] * x[t, h, p], and the row's two inner products
+                    const int le = phase_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
+                    float o[16], pe = 0.f, pd = 0.f;
+#pragma unroll
+                    for (int vg = 0; vg < 4; ++vg) {
+                        const bf16x4 x4 = XT::row4(xs, ll, 8 * vg + 4 * he);
+                        const bf16x4 a4 = __builtin_bit_cast(bf16x4, aq[vg]);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            o[vg * 4 + i] = wt * acc[vg * 4 + i] + dh * (float)x4[i];
+                            pe += acc[vg * 4 + i] * (float)a4[i];
+                            pd += (float)x4[i] * (float)a4[i];
+                        }
+                    }
+                    pe += __shfl_xor(pe, 32, 64);
+                    pd += __shfl_xor(pd, 32, 64);
+                    const int yrow = s.L - 1 - (t0 + ll);
+                    const bool live = ll < rows && yrow >= 0 && yrow < trows;
+                    store_column<TO>(yb + (size_t)yrow * HP, o, he, 32, live);
+                    if (he == 0 && live)
+                        *reinterpret_cast<float2 *>(seg_decay + 2 * (((size_t)b * trows + yrow) * s.H + h)) = make_float2(pe, pd);
                 } else {
                     // epilogue: y[t, h, p] = yT[p, l] + D[h] * x[t, h, p]
                     const int le = phase_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
@@ -783,6 +823,25 @@ static hipError_t fused_launch_transposed(const ScanShape &s, const void *x, con
     fused_scan_kernel<TO, 2, kOnePassTile / 32, 8, KIND><<<dim3(grid), dim3(512), 0, st>>>(
         static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
         static_cast<const __bf16 *>(Cm), nullptr, init, reset, static_cast<TO *>(out), final_states, tile_states, parts,
+        static_cast<const __bf16 *>(aux), s);
+    return hipGetLastError();
+}
+
+// The reversed-adjoint scan with the row products (KIND 5): x, Bm, Cm, dt, aux are the forward sequence's tensors
+// (s.dt_len rows, s.L the padded length of the reversed sequence); dx [B,L,H,32] bf16, pairs float2 [B,L,H].
+template <int NK>
+static hipError_t fused_launch_adjoint_rows(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
+                                            const void *Cm, const float *D, const void *aux, const float *init,
+                                            const unsigned char *reset, void *dx, float *final_states, float *pairs,
+                                            hipStream_t st) {
+    const int units = (s.H / s.G) * (s.P / 32);
+    if (s.P != 32 || units % 8 != 0 || s.seg_tiles != 0 || s.x_groups != 0 || s.N != 16 * NK || aux == nullptr ||
+        pairs == nullptr)
+        return hipErrorInvalidValue;
+    const int grid = s.B * s.G * (units / 8);
+    fused_scan_kernel<__bf16, NK, kOnePassTile / 32, 8, 5><<<dim3(grid), dim3(512), 0, st>>>(
+        static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
+        static_cast<const __bf16 *>(Cm), D, init, reset, static_cast<__bf16 *>(dx), final_states, nullptr, pairs,
         static_cast<const __bf16 *>(aux), s);
     return hipGetLastError();
 }

@@ -117,6 +117,15 @@ hipError_t launch_transposed_scan(const ScanShape &sT, bool adjoint, const void 
                                   const unsigned char *reset, void *out, float *final_states, float *tile_states,
                                   float *parts, hipStream_t stream);
 
+// The backward pass's reversed-adjoint scan with the row products in its epilogue (bf16, headdim 32, heads per
+// group a multiple of eight, dstate 32 or 64).  sR is the forward shape with L padded to whole tiles, mode 1 and
+// dt_len = the true length; all tensors are the forward sequence's.  Writes dx = dt r + D dy [B,L,H,32] (bf16), the
+// adjoint state at step 0 into g0 [B,H,32,N], and per (b,t,h) the pair (x . r, dy . x) into pairs, float2 [B,L,H].
+bool adjoint_rows_scan_supported(const ScanShape &sR);
+hipError_t launch_adjoint_rows_scan(const ScanShape &sR, const void *dy, const void *dt, const float *A, const void *Cm,
+                                    const void *Bm, const float *D, const void *x, const float *dfinal,
+                                    const unsigned char *reset, void *dx, float *g0, float *pairs, hipStream_t stream);
+
 // The memory-bound kernels of the backward pass (its three heavy products run on the stage launchers above with
 // the operands' roles swapped).  dtype: 0 = float32, 1 = bf16 activations and gradients.
 // gather_rows: dst[b, t', (g*rep + k)*W + w] = src[b, t, g*W + w] for t' < Ldst, with t = Ldst-1-t' if reverse
@@ -151,10 +160,11 @@ hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, con
                               const float *rev_prev, const float *rev_final, const float *init_t, const float *fwd_final,
                               const float *dfin_t, const unsigned char *reset, double *anchor, hipStream_t stream);
 // q_t between the anchors of its chunk (chunk <= 64 steps); ddt = e1 + A q; dA_part[b,h] = sum_t dt q,
-// dD_part[b,h] = sum_t dd
+// dD_part[b,h] = sum_t dd.  With parts given ([B,L,H,nparts], the pieces of C . yC), e1 holds the pairs (e1, dd)
+// of the adjoint scan with row products and u = sum of the parts - dt e1 is formed here (u and dd unused).
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
                           const float *dd, const double *anchor, void *ddt, double *dA_part, double *dD_part,
-                          hipStream_t stream);
+                          hipStream_t stream, const float *parts = nullptr, int nparts = 0);
 // dA[h], dD[h] (NULL allowed) = the sums over the batch of the parts
 hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,
                                 hipStream_t stream);
