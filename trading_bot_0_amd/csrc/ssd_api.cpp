@@ -180,7 +180,7 @@ BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
     w.dd = take(BL * s.H * sizeof(float));
     w.u = take(BL * s.H * sizeof(float));
     w.parts = take(BL * s.H * (size_t)((s.N + 31) / 32) * sizeof(float));
-    w.anchor = take((size_t)s.B * (s.nc + 1) * s.H * sizeof(double));
+    w.anchor = take((size_t)s.B * (s.nc + 1) * s.H * sizeof(double) * (size_t)((s.N + 31) / 32));  // or its pieces
     w.da_part = take((size_t)2 * s.B * s.H * sizeof(double));  // and the parts of dD behind them
     w.total = off;
     return w;
@@ -505,13 +505,19 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
         f.x_groups = s.G;
         // dB = sum over heads of dt (x . g): the adjoint recurrence with the state transposed; tile states in `states`
         BWD_LAUNCH(ssd::launch_transposed_scan(f, true, Cm, dt, A, dy, x, nullptr, dfin_t, reset, dB, atf(w.gfin_t), states,
-                                               nullptr, st),
+                                               nullptr, ssd::ScanAnchors{}, st),
                    "transposed adjoint scan");
         f = sT;
         f.x_groups = s.G;
-        // dC = sum over heads of dy . h: the forward recurrence with the state transposed; tile states in `states2`
-        BWD_LAUNCH(ssd::launch_transposed_scan(f, false, Bm, dt, A, x, dy, Cm, init_t, reset, dC, atf(w.ffin_t), states2,
-                                               atf(w.parts), st),
+        // dC = sum over heads of dy . h: the forward recurrence with the state transposed; it meets the adjoint's
+        // tile states on the way and leaves the pieces of the anchors
+        ssd::ScanAnchors an;
+        an.adj_tiles = states;
+        an.adj_final = atf(w.gfin_t);
+        an.dfinal = dfin_t;
+        an.out = reinterpret_cast<double *>(base + w.anchor);
+        BWD_LAUNCH(ssd::launch_transposed_scan(f, false, Bm, dt, A, x, dy, Cm, init_t, reset, dC, nullptr, nullptr,
+                                               atf(w.parts), an, st),
                    "transposed forward scan");
         if (!rows_in_scan)
             BWD_LAUNCH(ssd::launch_bwd_rows_parts(s, fast_r ? 0 : Lp, el, x, dy, dt, D, atf(w.r_rev), atf(w.parts), s.N / 32, dx,
@@ -539,13 +545,14 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     }
     }
     double *anchor = reinterpret_cast<double *>(base + w.anchor);
-    BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, reset, anchor,
-                                       st),
-               "backward anchors");
+    if (!sum_on_chip)
+        BWD_LAUNCH(ssd::launch_bwd_anchors(s, el, dt, A, states2, states, atf(w.gfin_t), init_t, atf(w.ffin_t), dfin_t, reset,
+                                           anchor, st),
+                   "backward anchors");
     double *da_part = reinterpret_cast<double *>(base + w.da_part);
     double *dd_part = da_part + (size_t)s.B * s.H;
     BWD_LAUNCH(ssd::launch_bwd_ddt(s, el, dt, A, atf(w.e1), atf(w.u), atf(w.dd), anchor, ddt, da_part, dd_part, st,
-                                   rows_in_scan ? atf(w.parts) : nullptr, s.N / 32),
+                                   rows_in_scan ? atf(w.parts) : nullptr, s.N / 32, reset, sum_on_chip ? s.N / 32 : 0),
                "backward ddt");
     BWD_LAUNCH(ssd::launch_bwd_head_sums(s, da_part, dd_part, dA, dD, st), "backward head sums");
     if (dinitial_states != nullptr)

@@ -314,7 +314,8 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
                                                       const float *__restrict__ dd, const double *__restrict__ anchor,
                                                       T *__restrict__ ddt, double *__restrict__ dA_part,
                                                       double *__restrict__ dD_part, ScanShape s,
-                                                      const float *__restrict__ parts, int nparts) {
+                                                      const float *__restrict__ parts, int nparts,
+                                                      const unsigned char *__restrict__ reset, int raw_anchors) {
     const int lane = threadIdx.x & 63;
     const long long bh = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (bh >= (long long)s.B * s.H) return;
@@ -325,10 +326,24 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
                                 __builtin_amdgcn_readlane(__double2loint(v), 63));
     };
     const double a = (double)A[h];
+    // raw_anchors > 0: `anchor` holds that many pieces per (b, c, h) of the inner product of the two states at the
+    // chunk's start, still without the first step's decay (zero where the sequence restarts there)
+    auto anchor_at = [&](int c) {
+        const size_t at = ((size_t)b * (s.nc + 1) + c) * s.H + h;
+        if (raw_anchors == 0) return anchor[at];
+        double v = 0.0;
+        for (int k = 0; k < raw_anchors; ++k) v += anchor[at * raw_anchors + k];
+        if (c < s.nc) {
+            const size_t t = (size_t)b * s.L + (size_t)c * s.Q;
+            v *= (reset != nullptr && reset[t] != 0) ? 0.0 : exp((double)(float)dt[t * s.H + h] * a);
+        }
+        return v;
+    };
     double da = 0.0, sdd = 0.0;
+    double q1 = anchor_at(0);
     for (int c = 0; c < s.nc; ++c) {
-        const double q0 = anchor[((size_t)b * (s.nc + 1) + c) * s.H + h];
-        const double q1 = anchor[((size_t)b * (s.nc + 1) + c + 1) * s.H + h];
+        const double q0 = q1;
+        q1 = anchor_at(c + 1);
         const int t0 = c * s.Q, len = min(s.Q, s.L - t0);
         const bool ok = lane < len;
         const size_t at = ((size_t)b * s.L + t0 + (ok ? lane : 0)) * s.H + h;
@@ -455,12 +470,12 @@ hipError_t anchors_t(const ScanShape &s, const void *dt, const float *A, const f
 template <typename T>
 hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float *e1, const float *u, const float *dd,
                  const double *anchor, void *ddt, double *dA_part, double *dD_part, const float *parts, int nparts,
-                 hipStream_t st) {
+                 const unsigned char *reset, int raw_anchors, hipStream_t st) {
     if (s.Q > 64) return hipErrorInvalidValue;  // one pass of the wave per chunk
     const long long waves = (long long)s.B * s.H;
     bwd_ddt_kernel<T><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, e1, u, dd, anchor,
                                                                               static_cast<T *>(ddt), dA_part, dD_part, s, parts,
-                                                                              nparts);
+                                                                              nparts, reset, raw_anchors);
     return hipGetLastError();
 }
 
@@ -529,9 +544,9 @@ hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, con
 
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
                           const float *dd, const double *anchor, void *ddt, double *dA_part, double *dD_part,
-                          hipStream_t st, const float *parts, int nparts) {
-    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, st)
-                 : ddt_t<float>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, st);
+                          hipStream_t st, const float *parts, int nparts, const unsigned char *reset, int raw_anchors) {
+    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, reset, raw_anchors, st)
+                 : ddt_t<float>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, reset, raw_anchors, st);
 }
 
 hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,

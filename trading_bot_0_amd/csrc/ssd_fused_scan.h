@@ -123,7 +123,8 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
 // workgroup is eight heads on one 32-column slice of x: every wave stages its own B and C tile, the x tile is
 // shared, and instead of writing y per head the waves add their tiles in LDS and the workgroup writes the sum
 // over its heads (dC, or dB with the heads' dt as weights) -- the per-head outputs never reach memory.  KIND 3
-// also writes, per head, the part of C_t . y_t that its slice holds.
+// also writes, per head, the part of C_t . y_t that its slice holds, and (ScanAnchors) the inner products of the
+// state entering each tile with the adjoint scan's state at the same timestep, which the decay gradient hangs on.
 // KIND 5: the reversed-adjoint scan of the backward pass with the row products in its epilogue (headdim 32: a wave
 // holds a head's whole row).  With r_t the recurrence's output it writes dx_t = dt_t r_t + D x_t (x being the
 // scan's x operand, dy) instead of r, and per (b, t, h) the pair (aux_t . r_t, aux_t . x_t) -- aux is the forward's
@@ -141,7 +142,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     const __bf16 *__restrict__ x, const __bf16 *__restrict__ dt, const float *__restrict__ A,
     const __bf16 *__restrict__ Bm, const __bf16 *__restrict__ Cm, const float *__restrict__ D,
     const float *init, const unsigned char *__restrict__ reset, TO *__restrict__ y, float *final_states,
-    float *tile_states, float *seg_decay, const __bf16 *__restrict__ aux, ScanShape s) {
+    float *tile_states, float *seg_decay, const __bf16 *__restrict__ aux, ScanShape s, ScanAnchors an) {
     using T = __bf16;
     constexpr bool ADJ = KIND == 1 || KIND == 4 || KIND == 5, STATES_ONLY = KIND == 2, TR = KIND == 3 || KIND == 4;
     constexpr bool ROWS = KIND == 5;
@@ -386,6 +387,42 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     make_float4(st[nb][4 * gq], st[nb][4 * gq + 1], st[nb][4 * gq + 2], st[nb][4 * gq + 3]);
         }
     };
+
+    // KIND 3: this slice's part of <state, adjoint state> at the start of tile k (k = nc: the end of the sequence).
+    // The adjoint scan ran over the reversed sequence, so its tile nc - k begins where forward tile k does.
+    auto adjoint_state = [&](int k) -> const float * {
+        const float *g = k == 0 ? an.adj_final : k == s.nc ? an.dfinal : an.adj_tiles;
+        if (g == nullptr) return nullptr;
+        const size_t bh = k == 0 || k == s.nc ? (size_t)b * s.H + h : ((size_t)b * s.nc + (s.nc - k)) * s.H + h;
+        return g + (bh * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
+    };
+    auto load_adjoint = [&](const float *g, float4 (&gq)[NB][4]) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+                gq[nb][q4] = g ? *reinterpret_cast<const float4 *>(g + 32 * nb + 8 * q4) : make_float4(0, 0, 0, 0);
+        }
+    };
+    auto write_anchor = [&](int k, const float4 (&gq)[NB][4]) {
+        double part = 0.0;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+                part += (double)st[nb][4 * q4] * gq[nb][q4].x + (double)st[nb][4 * q4 + 1] * gq[nb][q4].y +
+                        (double)st[nb][4 * q4 + 2] * gq[nb][q4].z + (double)st[nb][4 * q4 + 3] * gq[nb][q4].w;
+        }
+        part = wave_inclusive_scan(part);
+        if (lane0 == 63) an.out[(((size_t)b * (s.nc + 1) + k) * s.H + h) * PBn + pb] = part;
+    };
+    if constexpr (KIND == 3) {
+        if (an.out != nullptr) {
+            float4 gq[NB][4];
+            load_adjoint(init ? adjoint_state(0) : nullptr, gq);  // no initial state: the first anchor is zero
+            write_anchor(0, gq);
+        }
+    }
 
     float seg_total = 1.f;  // product of the tiles' decays (KIND 2)
     prefetch(c_first);
@@ -707,6 +744,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         }
         // ---- phase 2: the state leaving this chunk ----
         if (!kEarlyPrefetch && c + 1 < c_end) prefetch(c + 1);
+        float4 gq[KIND == 3 ? NB : 1][4];  // the adjoint state where this tile ends, in flight during phase 2
+        if constexpr (KIND == 3) {
+            if (an.out != nullptr) load_adjoint(adjoint_state(c + 1), gq);
+        }
         seg_total *= a_end;
         const int lane = phase_tid() & 63, half = lane >> 5;
 #pragma unroll
@@ -752,6 +793,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 st[nb] = mma32(bf[nb], xlf, st[nb]);
             }
         }
+        if constexpr (KIND == 3) {
+            if (an.out != nullptr) write_anchor(c + 1, gq);
+        }
     }
 
     if (STATES_ONLY) {
@@ -781,14 +825,14 @@ static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt
         if constexpr (sizeof(TO) == 4) {
             if (segments != 1) return hipErrorInvalidValue;
             fused_scan_kernel<TO, NK, QB, WAVES, 1><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, nullptr, s);
+                xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, nullptr, s, ScanAnchors{});
             return hipGetLastError();
         } else {
             return hipErrorInvalidValue;
         }
     }
     fused_scan_kernel<TO, NK, QB, WAVES, 0><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
-        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, nullptr, s);
+        xx, dd, A, bb, cc, D, init, reset, static_cast<TO *>(y), final_states, tile_states, nullptr, nullptr, s, ScanAnchors{});
     return hipGetLastError();
 }
 
@@ -804,7 +848,7 @@ static hipError_t fused_launch_states(const ScanShape &s, const void *x, const v
     const __bf16 *bb = static_cast<const __bf16 *>(Bm);
     fused_scan_kernel<__bf16, NK, QB, WAVES, 2><<<dim3(grid), dim3(64 * WAVES), 0, st>>>(
         static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, bb, bb, nullptr, init, reset, nullptr, seg_states,
-        nullptr, seg_decay, nullptr, s);
+        nullptr, seg_decay, nullptr, s, ScanAnchors{});
     return hipGetLastError();
 }
 
@@ -812,18 +856,19 @@ static hipError_t fused_launch_states(const ScanShape &s, const void *x, const v
 // transposed shape (P = the forward's dstate, N = 32 = its headdim, G = H), x [B,L,x_groups,P] the operand the
 // heads of a group share, Bm, Cm [B,L,H,32] per head; out [B,L,x_groups,P] receives the sum over each group's
 // eight heads of the per-head outputs (weighted by dt in KIND 4); KIND 3 also writes, per head and 32-column
-// slice, aux_t . y_t into parts [B,L,H,P/32] (aux [B,L,x_groups,P]).
+// slice, aux_t . y_t into parts [B,L,H,P/32] (aux [B,L,x_groups,P]), and the anchors `an` asks for.
 template <typename TO, int KIND>
 static hipError_t fused_launch_transposed(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
                                           const void *Cm, const void *aux, const float *init, const unsigned char *reset,
-                                          void *out, float *final_states, float *tile_states, float *parts, hipStream_t st) {
+                                          void *out, float *final_states, float *tile_states, float *parts,
+                                          const ScanAnchors &an, hipStream_t st) {
     if (s.N != 32 || s.G != s.H || s.x_groups <= 0 || s.H != 8 * s.x_groups || s.P % 32 != 0 || s.seg_tiles != 0)
         return hipErrorInvalidValue;
     const int grid = s.B * (s.H / 8) * (s.P / 32);
     fused_scan_kernel<TO, 2, kOnePassTile / 32, 8, KIND><<<dim3(grid), dim3(512), 0, st>>>(
         static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
         static_cast<const __bf16 *>(Cm), nullptr, init, reset, static_cast<TO *>(out), final_states, tile_states, parts,
-        static_cast<const __bf16 *>(aux), s);
+        static_cast<const __bf16 *>(aux), s, an);
     return hipGetLastError();
 }
 
@@ -842,7 +887,7 @@ static hipError_t fused_launch_adjoint_rows(const ScanShape &s, const void *x, c
     fused_scan_kernel<__bf16, NK, kOnePassTile / 32, 8, 5><<<dim3(grid), dim3(512), 0, st>>>(
         static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
         static_cast<const __bf16 *>(Cm), D, init, reset, static_cast<__bf16 *>(dx), final_states, nullptr, pairs,
-        static_cast<const __bf16 *>(aux), s);
+        static_cast<const __bf16 *>(aux), s, ScanAnchors{});
     return hipGetLastError();
 }
 

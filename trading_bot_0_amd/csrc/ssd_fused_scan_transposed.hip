@@ -12,14 +12,14 @@ bool transposed_scan_supported(const ScanShape &sT, int x_groups) {
 hipError_t launch_transposed_scan(const ScanShape &sT, bool adjoint, const void *x, const void *dt, const float *A,
                                   const void *Bm, const void *Cm, const void *aux, const float *init,
                                   const unsigned char *reset, void *out, float *final_states, float *tile_states,
-                                  float *parts, hipStream_t st) {
+                                  float *parts, const ScanAnchors &an, hipStream_t st) {
     ScanShape t = sT;
     t.Q = kOnePassTile;
     t.nc = (sT.L + kOnePassTile - 1) / kOnePassTile;
     return adjoint ? fused_launch_transposed<__bf16, 4>(t, x, dt, A, Bm, Cm, nullptr, init, reset, out, final_states,
-                                                        tile_states, nullptr, st)
+                                                        tile_states, nullptr, ScanAnchors{}, st)
                    : fused_launch_transposed<__bf16, 3>(t, x, dt, A, Bm, Cm, aux, init, reset, out, final_states,
-                                                        tile_states, parts, st);
+                                                        tile_states, parts, an, st);
 }
 
 }  // namespace ssd

@@ -111,11 +111,19 @@ hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, cons
 // [B,L,H,32] are per head.  out [B,L,x_groups,P] (bf16) = the sum over each group's heads of the per-head
 // outputs, weighted by the heads' dt when adjoint.  Forward in time it also writes parts [B,L,H,P/32]: per head
 // and 32-column slice, aux_t . y_t (aux [B,L,x_groups,P]).  tile_states / final_states as for the one-pass kernel.
+// With `an.out` given, the forward scan also writes, per (b, k, h) for k = 0 .. nc and per 32-column slice, the inner
+// product of its state at the start of tile k (k = nc: its final state) with the adjoint scan's state at the same
+// timestep -- adj_tiles[b, nc - k, h] for 0 < k < nc, adj_final for k = 0 (zero without an initial state), dfinal
+// for k = nc (zero when NULL): out [B, nc+1, H, P/32], float64.
+struct ScanAnchors {
+    const float *adj_tiles = nullptr, *adj_final = nullptr, *dfinal = nullptr;
+    double *out = nullptr;
+};
 bool transposed_scan_supported(const ScanShape &sT, int x_groups);
 hipError_t launch_transposed_scan(const ScanShape &sT, bool adjoint, const void *x, const void *dt, const float *A,
                                   const void *Bm, const void *Cm, const void *aux, const float *init,
                                   const unsigned char *reset, void *out, float *final_states, float *tile_states,
-                                  float *parts, hipStream_t stream);
+                                  float *parts, const ScanAnchors &an, hipStream_t stream);
 
 // The backward pass's reversed-adjoint scan with the row products in its epilogue (bf16, headdim 32, heads per
 // group a multiple of eight, dstate 32 or 64).  sR is the forward shape with L padded to whole tiles, mode 1 and
@@ -162,9 +170,13 @@ hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, con
 // q_t between the anchors of its chunk (chunk <= 64 steps); ddt = e1 + A q; dA_part[b,h] = sum_t dt q,
 // dD_part[b,h] = sum_t dd.  With parts given ([B,L,H,nparts], the pieces of C . yC), e1 holds the pairs (e1, dd)
 // of the adjoint scan with row products and u = sum of the parts - dt e1 is formed here (u and dd unused).
+// With raw_anchors > 0, anchor holds that many pieces per (b, c, h) ([B, nc+1, H, raw_anchors], as ScanAnchors
+// writes them) of the two states' inner product, and the first step's decay exp(dt A) -- zero where `reset` marks
+// the chunk's first step -- is applied here.
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
                           const float *dd, const double *anchor, void *ddt, double *dA_part, double *dD_part,
-                          hipStream_t stream, const float *parts = nullptr, int nparts = 0);
+                          hipStream_t stream, const float *parts = nullptr, int nparts = 0,
+                          const unsigned char *reset = nullptr, int raw_anchors = 0);
 // dA[h], dD[h] (NULL allowed) = the sums over the batch of the parts
 hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,
                                 hipStream_t stream);
