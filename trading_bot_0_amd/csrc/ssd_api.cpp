@@ -181,7 +181,7 @@ BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
     w.u = take(BL * s.H * sizeof(float));
     w.parts = take(BL * s.H * (size_t)((s.N + 31) / 32) * sizeof(float));
     w.anchor = take((size_t)s.B * (s.nc + 1) * s.H * sizeof(double) * (size_t)((s.N + 31) / 32));  // or its pieces
-    w.da_part = take((size_t)2 * s.B * s.H * sizeof(double));  // and the parts of dD behind them
+    w.da_part = take((size_t)2 * s.B * s.nc * s.H * sizeof(double));  // and the parts of dD behind them
     w.total = off;
     return w;
 }
@@ -550,7 +550,7 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
                                            anchor, st),
                    "backward anchors");
     double *da_part = reinterpret_cast<double *>(base + w.da_part);
-    double *dd_part = da_part + (size_t)s.B * s.H;
+    double *dd_part = da_part + (size_t)s.B * s.nc * s.H;
     BWD_LAUNCH(ssd::launch_bwd_ddt(s, el, dt, A, atf(w.e1), atf(w.u), atf(w.dd), anchor, ddt, da_part, dd_part, st,
                                    rows_in_scan ? atf(w.parts) : nullptr, s.N / 32, reset, sum_on_chip ? s.N / 32 : 0),
                "backward ddt");

@@ -303,11 +303,11 @@ __global__ __launch_bounds__(256) void bwd_anchor_kernel(const T *__restrict__ d
     }
 }
 
-// One wave per (b, h), one pass of the wave per chunk (chunks of at most 64 steps).  q is known at both ends of a
-// chunk (the anchors) and obeys q_t - q_{t+1} = u_t in between; the computed u do not sum exactly to the
-// difference of the anchors, and the mismatch is spread evenly over the chunk's steps:
+// One wave per (b, c, h): a chunk of at most 64 steps.  q is known at both ends of a chunk (the anchors) and obeys
+// q_t - q_{t+1} = u_t in between; the computed u do not sum exactly to the difference of the anchors, and the
+// mismatch is spread evenly over the chunk's steps:
 // q_t = anchor_c - sum_{v < t in the chunk} u_v - mismatch * (steps before t) / (steps of the chunk).
-// ddt_t = e1_t + A q_t and this sequence's parts of dA = sum dt_t q_t and of dD = sum dd_t.  Sums in float64.
+// ddt_t = e1_t + A q_t and this chunk's parts of dA = sum dt_t q_t and of dD = sum dd_t.  Sums in float64.
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, const float *__restrict__ A,
                                                       const float *__restrict__ e1, const float *__restrict__ u,
@@ -317,10 +317,11 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
                                                       const float *__restrict__ parts, int nparts,
                                                       const unsigned char *__restrict__ reset, int raw_anchors) {
     const int lane = threadIdx.x & 63;
-    const long long bh = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (bh >= (long long)s.B * s.H) return;
-    const int h = (int)(bh % s.H);
-    const long long b = bh / s.H;
+    const long long id = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (id >= (long long)s.B * s.nc * s.H) return;
+    const int h = (int)(id % s.H);
+    const int c = (int)((id / s.H) % s.nc);
+    const long long b = id / ((long long)s.H * s.nc);
     auto last_lane = [](double v) {
         return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), 63),
                                 __builtin_amdgcn_readlane(__double2loint(v), 63));
@@ -328,65 +329,150 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
     const double a = (double)A[h];
     // raw_anchors > 0: `anchor` holds that many pieces per (b, c, h) of the inner product of the two states at the
     // chunk's start, still without the first step's decay (zero where the sequence restarts there)
-    auto anchor_at = [&](int c) {
-        const size_t at = ((size_t)b * (s.nc + 1) + c) * s.H + h;
+    auto anchor_at = [&](int k) {
+        const size_t at = ((size_t)b * (s.nc + 1) + k) * s.H + h;
         if (raw_anchors == 0) return anchor[at];
         double v = 0.0;
-        for (int k = 0; k < raw_anchors; ++k) v += anchor[at * raw_anchors + k];
-        if (c < s.nc) {
-            const size_t t = (size_t)b * s.L + (size_t)c * s.Q;
+        for (int i = 0; i < raw_anchors; ++i) v += anchor[at * raw_anchors + i];
+        if (k < s.nc) {
+            const size_t t = (size_t)b * s.L + (size_t)k * s.Q;
             v *= (reset != nullptr && reset[t] != 0) ? 0.0 : exp((double)(float)dt[t * s.H + h] * a);
         }
         return v;
     };
-    double da = 0.0, sdd = 0.0;
-    double q1 = anchor_at(0);
-    for (int c = 0; c < s.nc; ++c) {
-        const double q0 = q1;
-        q1 = anchor_at(c + 1);
-        const int t0 = c * s.Q, len = min(s.Q, s.L - t0);
-        const bool ok = lane < len;
-        const size_t at = ((size_t)b * s.L + t0 + (ok ? lane : 0)) * s.H + h;
-        float e1v = 0.f, ddv = 0.f, dtv = 0.f, uf = 0.f;
-        if (ok) {
-            dtv = (float)dt[at];
-            if (parts != nullptr) {  // (e1, dd) pairs; u from the pieces of C . yC
-                const float2 pr = *reinterpret_cast<const float2 *>(e1 + 2 * at);
-                e1v = pr.x;
-                ddv = pr.y;
-                float sc = 0.f;
-                for (int k = 0; k < nparts; ++k) sc += parts[at * nparts + k];
-                uf = sc - dtv * e1v;
-            } else {
-                e1v = e1[at];
-                ddv = dd[at];
-                uf = u[at];
-            }
-        }
-        const double uv = (double)uf;
-        const double incl = wave_inclusive_scan(uv);
-        const double mismatch = q0 - last_lane(incl) - q1;
-        if (ok) {
-            const double q = q0 - (incl - uv) - mismatch * (double)lane / (double)len;
-            ddt[at] = (T)(float)((double)e1v + a * q);
-            da += (double)dtv * q;
-            sdd += (double)ddv;
+    const double q0 = anchor_at(c), q1 = anchor_at(c + 1);
+    const int t0 = c * s.Q, len = min(s.Q, s.L - t0);
+    const bool ok = lane < len;
+    const size_t at = ((size_t)b * s.L + t0 + (ok ? lane : 0)) * s.H + h;
+    float e1v = 0.f, ddv = 0.f, dtv = 0.f, uf = 0.f;
+    if (ok) {
+        dtv = (float)dt[at];
+        if (parts != nullptr) {  // (e1, dd) pairs; u from the pieces of C . yC
+            const float2 pr = *reinterpret_cast<const float2 *>(e1 + 2 * at);
+            e1v = pr.x;
+            ddv = pr.y;
+            float sc = 0.f;
+            for (int k = 0; k < nparts; ++k) sc += parts[at * nparts + k];
+            uf = sc - dtv * e1v;
+        } else {
+            e1v = e1[at];
+            ddv = dd[at];
+            uf = u[at];
         }
     }
-    const double tot = last_lane(wave_inclusive_scan(da)), totd = last_lane(wave_inclusive_scan(sdd));
+    const double uv = (double)uf;
+    const double incl = wave_inclusive_scan(uv);
+    const double mismatch = q0 - last_lane(incl) - q1;
+    double da = 0.0;
+    if (ok) {
+        const double q = q0 - (incl - uv) - mismatch * (double)lane / (double)len;
+        ddt[at] = (T)(float)((double)e1v + a * q);
+        da = (double)dtv * q;
+    }
+    const double tot = last_lane(wave_inclusive_scan(da)), totd = last_lane(wave_inclusive_scan((double)ddv));
     if (lane == 0) {
-        dA_part[bh] = tot;
-        dD_part[bh] = totd;
+        dA_part[id] = tot;
+        dD_part[id] = totd;
     }
 }
 
-// One workgroup per head: dA[h] = sum_b dA_part[b,h], dD[h] = sum_b dD_part[b,h] (float64 sums).
+// The same for chunks of 64 steps and NH = 4, 8 or 16 heads with one wave per (b, c) and all its heads: lane =
+// (step % TL) * NH + head with TL = 64 / NH, register r = step / TL, so that every load and store of the wave is one
+// contiguous run of 64 elements of a [B, L, H] array (a wave per head touches a cache line per lane instead).
+template <typename T, int NH>
+__global__ __launch_bounds__(256) void bwd_ddt_heads_kernel(const T *__restrict__ dt, const float *__restrict__ A,
+                                                            const float *__restrict__ e1, const float *__restrict__ u,
+                                                            const float *__restrict__ dd, const double *__restrict__ anchor,
+                                                            T *__restrict__ ddt, double *__restrict__ dA_part,
+                                                            double *__restrict__ dD_part, ScanShape s,
+                                                            const float *__restrict__ parts, int nparts,
+                                                            const unsigned char *__restrict__ reset, int raw_anchors) {
+    constexpr int TL = 64 / NH, R = 64 / TL;
+    const int lane = threadIdx.x & 63;
+    const long long id = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (id >= (long long)s.B * s.nc) return;
+    const int c = (int)(id % s.nc);
+    const long long b = id / s.nc;
+    const int h = lane % NH, tl = lane / NH;
+    const double a = (double)A[h];
+    auto anchor_at = [&](int k) {
+        const size_t at = ((size_t)b * (s.nc + 1) + k) * NH + h;
+        if (raw_anchors == 0) return anchor[at];
+        double v = 0.0;
+        for (int i = 0; i < raw_anchors; ++i) v += anchor[at * raw_anchors + i];
+        if (k < s.nc) {
+            const size_t t = (size_t)b * s.L + (size_t)k * 64;
+            v *= (reset != nullptr && reset[t] != 0) ? 0.0 : exp((double)(float)dt[t * NH + h] * a);
+        }
+        return v;
+    };
+    const double q0 = anchor_at(c), q1 = anchor_at(c + 1);
+    const int t0 = c * 64, len = min(64, s.L - t0);
+    const size_t row0 = ((size_t)b * s.L + t0) * NH;  // this chunk's first element of a [B, L, H] array
+    float e1v[R], ddv[R], dtv[R];
+    double uv[R], before[R];  // u_t and the sum of u over the chunk's earlier steps
+    double carry = 0.0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int t = r * TL + tl;
+        const size_t at = row0 + (size_t)r * 64 + lane;
+        e1v[r] = ddv[r] = dtv[r] = 0.f;
+        float uf = 0.f;
+        if (t < len) {
+            dtv[r] = (float)dt[at];
+            if (parts != nullptr) {
+                const float2 pr = *reinterpret_cast<const float2 *>(e1 + 2 * at);
+                e1v[r] = pr.x;
+                ddv[r] = pr.y;
+                float sc = 0.f;
+                for (int k = 0; k < nparts; ++k) sc += parts[at * nparts + k];
+                uf = sc - dtv[r] * e1v[r];
+            } else {
+                e1v[r] = e1[at];
+                ddv[r] = dd[at];
+                uf = u[at];
+            }
+        }
+        uv[r] = (double)uf;
+        double v = uv[r];  // inclusive sum over this register's steps of the same head (lanes NH apart)
+#pragma unroll
+        for (int d = NH; d < 64; d <<= 1) {
+            const double o = __shfl_up(v, d, 64);
+            if (lane >= d) v += o;
+        }
+        before[r] = carry + v - uv[r];
+        carry += __shfl(v, 64 - NH + h, 64);
+    }
+    const double mismatch = q0 - carry - q1;
+    double da = 0.0, sdd = 0.0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int t = r * TL + tl;
+        if (t < len) {
+            const double q = q0 - before[r] - mismatch * (double)t / (double)len;
+            ddt[row0 + (size_t)r * 64 + lane] = (T)(float)((double)e1v[r] + a * q);
+            da += (double)dtv[r] * q;
+            sdd += (double)ddv[r];
+        }
+    }
+#pragma unroll
+    for (int d = NH; d < 64; d <<= 1) {
+        da += __shfl_xor(da, d, 64);
+        sdd += __shfl_xor(sdd, d, 64);
+    }
+    if (tl == 0) {
+        dA_part[id * NH + h] = da;
+        dD_part[id * NH + h] = sdd;
+    }
+}
+
+// One workgroup per head: dA[h] = the sum over (b, c) of dA_part[b,c,h], dD[h] likewise (float64 sums).
 __global__ __launch_bounds__(256) void bwd_head_sums_kernel(const double *__restrict__ dA_part, const double *__restrict__ dD_part,
                                                             float *__restrict__ dA, float *__restrict__ dD, ScanShape s) {
     __shared__ double red[2][256];
     const int h = blockIdx.x;
     double sa = 0.0, sd = 0.0;
-    for (long long i = threadIdx.x; i < s.B; i += blockDim.x) {
+    for (long long i = threadIdx.x; i < (long long)s.B * s.nc; i += blockDim.x) {
         sa += dA_part[i * s.H + h];
         sd += dD_part[i * s.H + h];
     }
@@ -472,7 +558,20 @@ hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float
                  const double *anchor, void *ddt, double *dA_part, double *dD_part, const float *parts, int nparts,
                  const unsigned char *reset, int raw_anchors, hipStream_t st) {
     if (s.Q > 64) return hipErrorInvalidValue;  // one pass of the wave per chunk
-    const long long waves = (long long)s.B * s.H;
+    if (s.Q == 64 && (s.H == 4 || s.H == 8 || s.H == 16)) {
+        const long long chunks = (long long)s.B * s.nc;
+        const dim3 grid((unsigned)((chunks + 3) / 4)), block(256);
+#define SSD_DDT_HEADS(NH)                                                                                              \
+    bwd_ddt_heads_kernel<T, NH><<<grid, block, 0, st>>>(static_cast<const T *>(dt), A, e1, u, dd, anchor,               \
+                                                        static_cast<T *>(ddt), dA_part, dD_part, s, parts, nparts, reset, \
+                                                        raw_anchors)
+        if (s.H == 4) SSD_DDT_HEADS(4);
+        else if (s.H == 8) SSD_DDT_HEADS(8);
+        else SSD_DDT_HEADS(16);
+#undef SSD_DDT_HEADS
+        return hipGetLastError();
+    }
+    const long long waves = (long long)s.B * s.nc * s.H;
     bwd_ddt_kernel<T><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st>>>(static_cast<const T *>(dt), A, e1, u, dd, anchor,
                                                                               static_cast<T *>(ddt), dA_part, dD_part, s, parts,
                                                                               nparts, reset, raw_anchors);
