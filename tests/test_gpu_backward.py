@@ -201,6 +201,7 @@ def test_gradients_with_restarts_inside_the_sequence(dtype, seqlen):
     Workload("bwd_sums_two_groups", 64, 150, 16, 32, 32, 2, 128, dtype="bf16", init_std=0.5),
     Workload("bwd_sums_ragged", 96, 129, 8, 32, 64, 1, 64, dtype="bf16", init_std=0.5),
     Workload("bwd_sums_short", 100, 5, 8, 32, 64, 1, 64, dtype="bf16", init_std=0.5),
+    Workload("bwd_sums_slice_per_wave", 64, 150, 8, 32, 64, 1, 64, dtype="bf16", init_std=0.5),  # too few groups for two
 ], ids=lambda w: w.name)
 @pytest.mark.parametrize("with_D,with_init,with_dfinal", [(True, True, True), (False, False, False)])
 def test_head_sums_taken_on_chip(w, with_D, with_init, with_dfinal):

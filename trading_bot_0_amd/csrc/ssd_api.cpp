@@ -499,26 +499,35 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
                                atf(w.gfin), states, false, 0))
         return rc;
     if (sum_on_chip) {
-        ssd::ScanShape f = sTR;
-        f.mode = 1;
-        f.dt_len = s.L;
-        f.x_groups = s.G;
-        // dB = sum over heads of dt (x . g): the adjoint recurrence with the state transposed; tile states in `states`
-        BWD_LAUNCH(ssd::launch_transposed_scan(f, true, Cm, dt, A, dy, x, nullptr, dfin_t, reset, dB, atf(w.gfin_t), states,
-                                               nullptr, ssd::ScanAnchors{}, st),
-                   "transposed adjoint scan");
-        f = sT;
-        f.x_groups = s.G;
-        // dC = sum over heads of dy . h: the forward recurrence with the state transposed; it meets the adjoint's
-        // tile states on the way and leaves the pieces of the anchors
+        // dB = sum over heads of dt (x . g): the adjoint recurrence with the state transposed; dC = sum over heads
+        // of dy . h: the forward recurrence with the state transposed.  The one that runs first leaves its tile
+        // states (in `states`), the other meets them on the way and leaves the pieces of the anchors.
+        ssd::ScanShape fa = sTR, ff = sT;
+        fa.mode = 1;
+        fa.dt_len = s.L;
+        fa.x_groups = ff.x_groups = s.G;
         ssd::ScanAnchors an;
-        an.adj_tiles = states;
-        an.adj_final = atf(w.gfin_t);
-        an.dfinal = dfin_t;
+        an.other_tiles = states;
         an.out = reinterpret_cast<double *>(base + w.anchor);
-        BWD_LAUNCH(ssd::launch_transposed_scan(f, false, Bm, dt, A, x, dy, Cm, init_t, reset, dC, nullptr, nullptr,
-                                               atf(w.parts), an, st),
-                   "transposed forward scan");
+        if (ssd::transposed_scan_anchors_in_adjoint(sT)) {
+            BWD_LAUNCH(ssd::launch_transposed_scan(ff, false, Bm, dt, A, x, dy, Cm, init_t, reset, dC, atf(w.ffin_t), states,
+                                                   atf(w.parts), ssd::ScanAnchors{}, st),
+                       "transposed forward scan");
+            an.other_final = atf(w.ffin_t);
+            an.other_init = init_t;
+            BWD_LAUNCH(ssd::launch_transposed_scan(fa, true, Cm, dt, A, dy, x, nullptr, dfin_t, reset, dB, nullptr, nullptr,
+                                                   nullptr, an, st),
+                       "transposed adjoint scan");
+        } else {
+            BWD_LAUNCH(ssd::launch_transposed_scan(fa, true, Cm, dt, A, dy, x, nullptr, dfin_t, reset, dB, atf(w.gfin_t),
+                                                   states, nullptr, ssd::ScanAnchors{}, st),
+                       "transposed adjoint scan");
+            an.other_final = atf(w.gfin_t);
+            an.other_init = dfin_t;
+            BWD_LAUNCH(ssd::launch_transposed_scan(ff, false, Bm, dt, A, x, dy, Cm, init_t, reset, dC, nullptr, nullptr,
+                                                   atf(w.parts), an, st),
+                       "transposed forward scan");
+        }
         if (!rows_in_scan)
             BWD_LAUNCH(ssd::launch_bwd_rows_parts(s, fast_r ? 0 : Lp, el, x, dy, dt, D, atf(w.r_rev), atf(w.parts), s.N / 32, dx,
                                                   atf(w.e1), atf(w.dd), atf(w.u), st),

@@ -123,8 +123,9 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
 // workgroup is eight heads on one 32-column slice of x: every wave stages its own B and C tile, the x tile is
 // shared, and instead of writing y per head the waves add their tiles in LDS and the workgroup writes the sum
 // over its heads (dC, or dB with the heads' dt as weights) -- the per-head outputs never reach memory.  KIND 3
-// also writes, per head, the part of C_t . y_t that its slice holds, and (ScanAnchors) the inner products of the
-// state entering each tile with the adjoint scan's state at the same timestep, which the decay gradient hangs on.
+// also writes, per head, the part of C_t . y_t that its slice holds.  Whichever of the two runs second also takes
+// (ScanAnchors) the inner products of the state entering each of its tiles with the other scan's state at the same
+// timestep, which the decay gradient hangs on: KIND 3 and 7 hold that code.
 // KIND 5: the reversed-adjoint scan of the backward pass with the row products in its epilogue (headdim 32: a wave
 // holds a head's whole row).  With r_t the recurrence's output it writes dx_t = dt_t r_t + D x_t (x being the
 // scan's x operand, dy) instead of r, and per (b, t, h) the pair (aux_t . r_t, aux_t . x_t) -- aux is the forward's
@@ -132,6 +133,16 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
 // LDS of a workgroup of the transposed scans: a B and a C tile per wave (eight waves), the shared x tile and
 // second-operand tile, the per-wave tables, and a [Q][33] float tile per wave for the heads' outputs (summed in a
 // fixed order when the workgroup writes them out, so that results do not depend on timing).
+// KIND 6 and 7 are 3 and 4 for a 64-wide transposed state (dstate 64) with both 32-column slices of a head in one
+// wave: the head's masked, decayed score tile -- the part of a tile's work that does not shrink with the state's
+// width -- and its B and C tiles are then formed and staged once instead of once per slice.  Their LDS holds two x
+// tiles and two tiles of the second operand of C . y, all tiles 8 elements apart instead of 16 to make room, and a
+// float tile per wave of 32 rows only: the workgroup writes its sums out after every block of 32 rows.
+constexpr int wide_transposed_tile_elems(int Q) { return Q * 32 + 8; }
+constexpr size_t wide_transposed_scan_lds_bytes(int Q) {
+    return (size_t)(2 * 8 + 4) * wide_transposed_tile_elems(Q) * 2 + (size_t)8 * ((5 + Q / 32) * Q * 4 + 64) +
+           (size_t)8 * 32 * 65 * 4;
+}
 constexpr size_t transposed_scan_lds_bytes(int Q) {
     return (size_t)(2 * 8 + 2) * fused_scan_xtile_elems(Q) * 2 + (size_t)8 * ((5 + Q / 32) * Q * 4 + 64) +
            (size_t)8 * Q * 33 * 4;
@@ -144,7 +155,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     const float *init, const unsigned char *__restrict__ reset, TO *__restrict__ y, float *final_states,
     float *tile_states, float *seg_decay, const __bf16 *__restrict__ aux, ScanShape s, ScanAnchors an) {
     using T = __bf16;
-    constexpr bool ADJ = KIND == 1 || KIND == 4 || KIND == 5, STATES_ONLY = KIND == 2, TR = KIND == 3 || KIND == 4;
+    constexpr bool ADJ = KIND == 1 || KIND == 4 || KIND == 5 || KIND == 7, STATES_ONLY = KIND == 2;
+    constexpr bool TR = KIND == 3 || KIND == 4 || KIND == 6 || KIND == 7;
+    constexpr bool TR_FWD = KIND == 3 || KIND == 6, TR_ADJ = KIND == 4 || KIND == 7;
+    constexpr int SL = (KIND == 6 || KIND == 7) ? 2 : 1;  // 32-column slices of x (and of the state) per wave
     constexpr bool ROWS = KIND == 5;
     static_assert(!TR || (NK == 2 && WAVES == 8), "the transposed scans: 32-wide state, eight heads per workgroup");
     constexpr int N = 16 * NK, NB = NK / 2, Q = 32 * QB, nthr = 64 * WAVES;
@@ -160,8 +174,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     using XT = ChunkTile<32>;
     using BT = ChunkTile<N>;
     // static, so that LDS addresses are compile-time offsets
-    constexpr int XS = fused_scan_xtile_elems(Q);
-    __shared__ __attribute__((aligned(16))) unsigned char smem[TR ? transposed_scan_lds_bytes(Q) : fused_scan_lds_bytes(N, Q, WAVES)];
+    constexpr int XS = SL == 2 ? wide_transposed_tile_elems(Q) : fused_scan_xtile_elems(Q);
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SL == 2 ? wide_transposed_scan_lds_bytes(Q)
+                                                                        : TR ? transposed_scan_lds_bytes(Q)
+                                                                             : fused_scan_lds_bytes(N, Q, WAVES)];
     const int tid = threadIdx.x;
     const int lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -173,10 +189,12 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     T *Cs = TR ? tiles + (WAVES + wave) * XS : tiles + Q * N;
     T *xs_all = TR ? tiles + 2 * WAVES * XS : tiles + 2 * Q * N;
     T *xs = TR ? xs_all : xs_all + wave * XS;
-    T *aux_s = xs_all + XS;  // transposed only
-    float *wf0 = reinterpret_cast<float *>(TR ? xs_all + 2 * XS : xs_all + WAVES * XS);
+    T *aux_s = xs_all + SL * XS;  // transposed only (one tile per slice, behind the x tiles)
+    float *wf0 = reinterpret_cast<float *>(TR ? xs_all + 2 * SL * XS : xs_all + WAVES * XS);
     float *wf = wf0 + wave * ((5 + QB) * Q + 16);
-    float *red = wf0 + WAVES * ((5 + QB) * Q + 16);  // transposed only: [WAVES][Q][33], every head's output tile
+    // transposed only: every head's output tile, [WAVES][Q][33], or [WAVES][32][65] with two slices per wave
+    float *red = wf0 + WAVES * ((5 + QB) * Q + 16);
+    constexpr int RS = SL == 2 ? 65 : 33;
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
     float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [8..8+QB): log2-decay across block lb
 
@@ -192,14 +210,14 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     const int c_end = s.seg_tiles > 0 ? min(s.nc, c_first + s.seg_tiles) : s.nc;
     // transposed: the workgroup is heads h0 .. h0+7 (one per wave) on x slice pb; s.G == s.H there, and
     // s.x_groups says how many groups of heads x is given for
-    const int TW = TR ? (s.H / 8) * PBn : 1;  // transposed workgroups per batch row
+    const int TW = TR ? (s.H / 8) * (SL == 2 ? 1 : PBn) : 1;  // transposed workgroups per batch row
     const int b = TR ? logical / TW : logical / (s.G * UW);
     const int g = TR ? 0 : (logical / UW) % s.G;
     const int unit0 = TR ? 0 : (logical % UW) * WAVES;
     const int unit = unit0 + wave;
-    const int h0 = TR ? ((logical % TW) / PBn) * 8 : 0;
+    const int h0 = TR ? (SL == 2 ? logical % TW : (logical % TW) / PBn) * 8 : 0;
     const int h = TR ? h0 + wave : g * HG + unit / PBn;
-    const int pb = TR ? (logical % TW) % PBn : unit % PBn;
+    const int pb = TR ? (SL == 2 ? 0 : (logical % TW) % PBn) : unit % PBn;
     const int xcol0 = g * HG * s.P + unit0 * 32;  // first element of the workgroup's slice of an x row
     const int HP = s.H * s.P;
     // x rows: one per timestep, HP wide -- or, when x is shared by groups of heads (s.x_groups, with G == H so
@@ -214,7 +232,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     const T *xb = x + (size_t)b * trows * XLD + xcol;
     const T *Bb = Bm + ((size_t)b * trows * s.G + (TR ? h0 : g)) * N;  // transposed: eight heads' rows side by side
     const T *Cb = Cm + ((size_t)b * trows * s.G + (TR ? h0 : g)) * N;
-    const T *auxb = TR && aux ? aux + (size_t)b * trows * XLD + xcol : nullptr;
+    const T *auxb = TR_FWD && aux ? aux + (size_t)b * trows * XLD + xcol : nullptr;
     // mode 1 (the time-reversed adjoint recurrence): step t decays by the dt of step L - t of a dt tensor of
     // dt_len rows, steps outside it do not decay, and every step's input weighs one instead of dt
     const int dt_rows = ADJ ? s.dt_len : s.L;
@@ -231,7 +249,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // copy of the thread index that an empty asm hides from the compiler, so that it cannot hoist them out
     // of the tile loop again (hoisted, they held about a hundred registers through all phases and forced
     // spills whose reloads, each an s_waitcnt vmcnt(0), serialised the prefetch).
-    constexpr bool kRecomputeOffsets = QB > 2;
+    constexpr bool kRecomputeOffsets = QB > 2 || SL == 2;
     auto phase_tid = [&]() {
         int t = tid;
         if (kRecomputeOffsets) asm volatile("" : "+v"(t));
@@ -282,8 +300,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             return v;
         };
         if constexpr (TR) {
-            const int prow = tv / XPR, srow = tv / 4;
-            const unsigned pcol = (tv % XPR) * 8, scol = (tv % 4) * 8;
+            const int prow = tv / XPR, srow = tv / (4 * SL);
+            const unsigned pcol = (tv % XPR) * 8, scol = (tv % (4 * SL)) * 8;
             auto source = [&](int row, bool &ok) {  // the tensors' row of this tile's row `row`
                 const int src = ADJ ? s.L - 1 - t0 - row : t0 + row;
                 ok = ADJ ? (src >= 0 && src < trows) : row < rows;
@@ -299,9 +317,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             {
                 bool ok;
                 const int src = source(srow, ok);
-                ok = ok && tv < Q * 4;
+                ok = ok && tv < Q * 4 * SL;
                 xq[0] = ld16(xb + (size_t)src * XLD + scol, ok);
-                if (auxb != nullptr) auxq = ld16(auxb + (size_t)src * XLD + scol, ok);
+                if (TR_FWD && auxb != nullptr) auxq = ld16(auxb + (size_t)src * XLD + scol, ok);
             }
 #pragma unroll
             for (int e = 0; e < EPL; ++e) dq[e] = dt_bits(e, (tv & 63) * EPL + e < rows);
@@ -359,68 +377,84 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     };
 
     // ---- running state of this unit: st[nb][v] = H[p = r, n = 32 nb + 8 (v/4) + 4 half + v%4] ----
-    f32x16 st[NB];
-    {
-        const float *ib = init ? init + ((((size_t)b * S + seg) * s.H + h) * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5)
+    // (with two slices per wave: slice sl in st[sl * NB ..])
+    f32x16 st[SL * NB];
+#pragma unroll
+    for (int sl = 0; sl < SL; ++sl) {
+        const float *ib = init ? init + ((((size_t)b * S + seg) * s.H + h) * s.P + (pb + sl) * 32 + (lane0 & 31)) * N +
+                                     4 * (lane0 >> 5)
                                : nullptr;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
             for (int gq = 0; gq < 4; ++gq) {
                 const float4 v = ib ? *reinterpret_cast<const float4 *>(ib + 32 * nb + 8 * gq) : make_float4(0, 0, 0, 0);
-                st[nb][4 * gq + 0] = v.x;
-                st[nb][4 * gq + 1] = v.y;
-                st[nb][4 * gq + 2] = v.z;
-                st[nb][4 * gq + 3] = v.w;
+                st[sl * NB + nb][4 * gq + 0] = v.x;
+                st[sl * NB + nb][4 * gq + 1] = v.y;
+                st[sl * NB + nb][4 * gq + 2] = v.z;
+                st[sl * NB + nb][4 * gq + 3] = v.w;
             }
         }
     }
 
     // this lane's part of the unit's [32 columns, N] block of a [P,N] state
     auto store_state = [&](float *state_bh) {
-        float *fb = state_bh + (size_t)(pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
+        for (int sl = 0; sl < SL; ++sl) {
+            float *fb = state_bh + (size_t)((pb + sl) * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
 #pragma unroll
-            for (int gq = 0; gq < 4; ++gq)
-                *reinterpret_cast<float4 *>(fb + 32 * nb + 8 * gq) =
-                    make_float4(st[nb][4 * gq], st[nb][4 * gq + 1], st[nb][4 * gq + 2], st[nb][4 * gq + 3]);
+            for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq)
+                    *reinterpret_cast<float4 *>(fb + 32 * nb + 8 * gq) =
+                        make_float4(st[sl * NB + nb][4 * gq], st[sl * NB + nb][4 * gq + 1], st[sl * NB + nb][4 * gq + 2],
+                                    st[sl * NB + nb][4 * gq + 3]);
+            }
         }
     };
 
-    // KIND 3: this slice's part of <state, adjoint state> at the start of tile k (k = nc: the end of the sequence).
-    // The adjoint scan ran over the reversed sequence, so its tile nc - k begins where forward tile k does.
-    auto adjoint_state = [&](int k) -> const float * {
-        const float *g = k == 0 ? an.adj_final : k == s.nc ? an.dfinal : an.adj_tiles;
+    // The anchors (KIND 3 and 7): this slice's part of <this scan's state, the other scan's state> at the start of this
+    // scan's tile j (j = nc: its final state).  The other scan ran over the sequence in the opposite direction, so its
+    // tile nc - j begins where this one's tile j does; this scan's initial state meets the other's final state and
+    // the other way round.  The piece goes to out[b, k, h, slice] with k counted in forward time.
+    constexpr bool ANCH = KIND == 3 || KIND == 7;
+    auto adjoint_state = [&](int j) -> const float * {
+        const float *g = j == 0 ? an.other_final : j == s.nc ? an.other_init : an.other_tiles;
         if (g == nullptr) return nullptr;
-        const size_t bh = k == 0 || k == s.nc ? (size_t)b * s.H + h : ((size_t)b * s.nc + (s.nc - k)) * s.H + h;
+        const size_t bh = j == 0 || j == s.nc ? (size_t)b * s.H + h : ((size_t)b * s.nc + (s.nc - j)) * s.H + h;
         return g + (bh * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
     };
-    auto load_adjoint = [&](const float *g, float4 (&gq)[NB][4]) {
+    // one slice at a time, so that at most one slice of the other scan's state is held in registers
+    auto load_other = [&](const float *g, int sl, float4 (&gq)[NB][4]) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4)
-                gq[nb][q4] = g ? *reinterpret_cast<const float4 *>(g + 32 * nb + 8 * q4) : make_float4(0, 0, 0, 0);
+                gq[nb][q4] = g ? *reinterpret_cast<const float4 *>(g + sl * 32 * N + 32 * nb + 8 * q4) : make_float4(0, 0, 0, 0);
         }
     };
-    auto write_anchor = [&](int k, const float4 (&gq)[NB][4]) {
+    auto write_anchor = [&](int k, int sl, const float4 (&gq)[NB][4]) {
         double part = 0.0;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
+            const int sn = sl * NB + nb;
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4)
-                part += (double)st[nb][4 * q4] * gq[nb][q4].x + (double)st[nb][4 * q4 + 1] * gq[nb][q4].y +
-                        (double)st[nb][4 * q4 + 2] * gq[nb][q4].z + (double)st[nb][4 * q4 + 3] * gq[nb][q4].w;
+                part += (double)st[sn][4 * q4] * gq[nb][q4].x + (double)st[sn][4 * q4 + 1] * gq[nb][q4].y +
+                        (double)st[sn][4 * q4 + 2] * gq[nb][q4].z + (double)st[sn][4 * q4 + 3] * gq[nb][q4].w;
         }
         part = wave_inclusive_scan(part);
-        if (lane0 == 63) an.out[(((size_t)b * (s.nc + 1) + k) * s.H + h) * PBn + pb] = part;
+        if (lane0 == 63) an.out[(((size_t)b * (s.nc + 1) + (ADJ ? s.nc - k : k)) * s.H + h) * PBn + pb + sl] = part;
     };
-    if constexpr (KIND == 3) {
+    if constexpr (ANCH) {
         if (an.out != nullptr) {
-            float4 gq[NB][4];
-            load_adjoint(init ? adjoint_state(0) : nullptr, gq);  // no initial state: the first anchor is zero
-            write_anchor(0, gq);
+            const float *g0 = init ? adjoint_state(0) : nullptr;  // no initial state: a zero anchor
+#pragma unroll
+            for (int sl = 0; sl < SL; ++sl) {
+                float4 gq[NB][4];
+                load_other(g0, sl, gq);
+                write_anchor(0, sl, gq);
+            }
         }
     }
 
@@ -453,9 +487,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 *reinterpret_cast<uint2 *>(tb + WAVES * XS) = make_uint2(cq[u].x, cq[u].y);
                 *reinterpret_cast<uint2 *>(tb1 + WAVES * XS) = make_uint2(cq[u].z, cq[u].w);
             }
-            if (tw < Q * 4) {
-                XT::put16(xs_all, tw / 4, (tw % 4) * 8, xq[0]);
-                XT::put16(aux_s, tw / 4, (tw % 4) * 8, auxq);
+            if (tw < Q * 4 * SL) {
+                const int col = (tw % (4 * SL)) * 8;
+                XT::put16(xs_all + (col / 32) * XS, tw / (4 * SL), col % 32, xq[0]);
+                if (TR_FWD) XT::put16(aux_s + (col / 32) * XS, tw / (4 * SL), col % 32, auxq);
             }
         }
 #pragma unroll
@@ -540,17 +575,18 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         if constexpr (!STATES_ONLY) {
             const int lane = phase_tid() & 63;
             const int r = lane & 31, half = lane >> 5;
-            Frag<T> Hhi[NK], Hlo[NK];
+            Frag<T> Hhi[SL * NK], Hlo[SL * NK];
 #pragma unroll
-            for (int kk = 0; kk < NK; ++kk) {
+            for (int sk = 0; sk < SL * NK; ++sk) {  // slice sk / NK, K step sk % NK
+                const int kk = sk % NK, sn = (sk / NK) * NB + kk / 2;
                 FragBits fh, fl;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int v = 8 * (kk % 2) + 2 * i;
-                    split_pair(st[kk / 2][v], 1.f, st[kk / 2][v + 1], 1.f, fh.u[i], fl.u[i]);
+                    split_pair(st[sn][v], 1.f, st[sn][v + 1], 1.f, fh.u[i], fl.u[i]);
                 }
-                Hhi[kk] = fh.frag();
-                Hlo[kk] = fl.frag();
+                Hhi[sk] = fh.frag();
+                Hlo[sk] = fl.frag();
             }
             // masked, decayed scores of one s-block as hi/lo operands; fv = the block's four F vectors
             auto make_m = [&](const f32x16 &sc, const float4 (&fv)[4], bool masked, Frag<T>(&mh)[2], Frag<T>(&ml)[2]) {
@@ -582,7 +618,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 // KIND 5: this lane's pieces of the second operand's rows and the rows' dt, requested here and used in
                 // the epilogue (lane = (row l, half): elements 8 vg + 4 half .. + 3 of the head's row)
                 uint2 aq[4] = {make_uint2(0, 0), make_uint2(0, 0), make_uint2(0, 0), make_uint2(0, 0)};
-                float wt = 0.f;
+                float wt = 1.f;
                 if constexpr (ROWS) {
                     const int arow = s.L - 1 - (t0 + l);
                     if (l < rows && arow >= 0 && arow < trows) {
@@ -595,13 +631,18 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 Frag<T> Cf[NK];
 #pragma unroll
                 for (int kk = 0; kk < NK; ++kk) Cf[kk] = BT::split_frag(Cs, l, 16 * kk + 4 * half);
-                f32x16 acc = {0};
+                f32x16 accs[SL];  // one output tile per slice
 #pragma unroll
-                for (int kk = 0; kk < NK; ++kk) {
-                    acc = mma32(Hhi[kk], Cf[kk], acc);
-                    acc = mma32(Hlo[kk], Cf[kk], acc);
+                for (int sl = 0; sl < SL; ++sl) {
+                    accs[sl] = f32x16{0};
+#pragma unroll
+                    for (int kk = 0; kk < NK; ++kk) {
+                        accs[sl] = mma32(Hhi[sl * NK + kk], Cf[kk], accs[sl]);
+                        accs[sl] = mma32(Hlo[sl * NK + kk], Cf[kk], accs[sl]);
+                    }
+                    accs[sl] = accs[sl] * blk_s[lb];
                 }
-                acc = acc * blk_s[lb];
+                f32x16 &acc = accs[0];
                 const float *F_row = F_s + lb * Q;
                 // one s-block.  On the separable path the diagonal block is one more term of the sum that E[l]
                 // scales at the end; on the exact path the sum is scaled first and the block carries its full factors.
@@ -613,10 +654,13 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
 #pragma unroll
                     for (int kk = 0; kk < NK; ++kk) sc = mma32(Bf[kk], Cf[kk], sc);
                     // requested while the score MFMAs run
-                    Frag<T> xf[2];
+                    Frag<T> xf[SL][2];
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)  // K order of mh[j]: rows 32 sb + 16 j + 4 half + {0..3} and the same + 8
-                        xf[j] = XT::frag(xs, sb * 32 + 16 * j + 4 * half, 8, 0, lane);
+                    for (int sl = 0; sl < SL; ++sl) {
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)  // K order of mh[j]: rows 32 sb + 16 j + 4 half + {0..3} and the same + 8
+                            xf[sl][j] = XT::frag(xs + sl * XS, sb * 32 + 16 * j + 4 * half, 8, 0, lane);
+                    }
                     float4 fv[4];
                     if (!diag || fast) {
 #pragma unroll
@@ -626,7 +670,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     if (diag) {
                         El = E_s[l];
                         if (!fast) {
-                            acc = acc * El;
+#pragma unroll
+                            for (int sl = 0; sl < SL; ++sl) accs[sl] = accs[sl] * El;
                             const float al_hi = ah_s[l], al_lo = alo_s[l];
 #pragma unroll
                             for (int vg = 0; vg < 4; ++vg) {
@@ -645,11 +690,14 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     Frag<T> mh[2], ml[2];
                     make_m(sc, fv, diag, mh, ml);
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        acc = mma32(xf[j], mh[j], acc);
-                        acc = mma32(xf[j], ml[j], acc);
+                    for (int sl = 0; sl < SL; ++sl) {
+#pragma unroll
+                        for (int j = 0; j < 2; ++j) {
+                            accs[sl] = mma32(xf[sl][j], mh[j], accs[sl]);
+                            accs[sl] = mma32(xf[sl][j], ml[j], accs[sl]);
+                        }
+                        if (diag && fast) accs[sl] = accs[sl] * El;  // everything summed so far shares the factor E[l]
                     }
-                    if (diag && fast) acc = acc * El;  // everything summed so far shares the factor E[l]
                 };
                 // compile-time block index: every LDS address is a lane offset plus an immediate
 #pragma unroll
@@ -662,22 +710,49 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     const int le = phase_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
                     const int trow = ADJ ? s.L - 1 - (t0 + ll) : t0 + ll;
                     const bool live = ll < rows && trow >= 0 && trow < trows;
-                    float wt = 1.f;  // KIND 4: dB sums the heads' outputs weighted by their dt
-                    if (KIND == 4) wt = live ? (float)dt[((size_t)b * trows + trow) * s.H + h] : 0.f;
-                    float part = 0.f;  // KIND 3: this slice's part of C_t . y_t
+                    // adjoint: dB sums the heads' outputs weighted by their dt
+                    if (TR_ADJ) wt = live ? (float)dt[((size_t)b * trows + trow) * s.H + h] : 0.f;
 #pragma unroll
-                    for (int vg = 0; vg < 4; ++vg) {
-                        if (KIND == 3 && aux != nullptr) {
-                            const bf16x4 c4 = XT::row4(aux_s, ll, 8 * vg + 4 * he);
+                    for (int sl = 0; sl < SL; ++sl) {
+                        float part = 0.f;  // forward: this slice's part of C_t . y_t
+                        // where this lane's 16 elements of the head's tile go (two slices: tiles of 32 rows, side by side)
+                        float *rw = SL == 2 ? red + (wave * 32 + (le & 31)) * RS + sl * 32 : red + (wave * Q + ll) * RS;
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) part += acc[vg * 4 + i] * (float)c4[i];
+                        for (int vg = 0; vg < 4; ++vg) {
+                            if (TR_FWD && aux != nullptr) {
+                                const bf16x4 c4 = XT::row4(aux_s + sl * XS, ll, 8 * vg + 4 * he);
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) part += accs[sl][vg * 4 + i] * (float)c4[i];
+                            }
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) rw[8 * vg + 4 * he + i] = wt * accs[sl][vg * 4 + i];
                         }
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) red[(wave * Q + ll) * 33 + 8 * vg + 4 * he + i] = wt * acc[vg * 4 + i];
+                        if (TR_FWD && seg_decay != nullptr) {  // (seg_decay: the per-head parts [B, L, H, P/32])
+                            part += __shfl_xor(part, 32, 64);
+                            if (he == 0 && live) seg_decay[(((size_t)b * trows + trow) * s.H + h) * PBn + pb + sl] = part;
+                        }
                     }
-                    if (KIND == 3 && seg_decay != nullptr) {  // (seg_decay: the per-head parts [B, L, H, P/32])
-                        part += __shfl_xor(part, 32, 64);
-                        if (he == 0 && live) seg_decay[(((size_t)b * trows + trow) * s.H + h) * PBn + pb] = part;
+                    if constexpr (SL == 2) {
+                        // the sum over the workgroup's heads of these 32 rows, [32][64], goes to the group's rows of
+                        // the gradient: 4 elements per thread
+                        block_sync_lds();
+                        const int tq = phase_tid();
+                        const int row = tq >> 4, c4 = (tq & 15) * 4;
+                        float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
+#pragma unroll
+                        for (int wv = 0; wv < WAVES; ++wv) {  // heads in order
+                            const float *rr = red + (wv * 32 + row) * RS + c4;
+                            v0 += rr[0];
+                            v1 += rr[1];
+                            v2 += rr[2];
+                            v3 += rr[3];
+                        }
+                        const int lr = lb * 32 + row;
+                        const int orow = ADJ ? s.L - 1 - (t0 + lr) : t0 + lr;
+                        if (lr < rows && orow >= 0 && orow < trows)
+                            *reinterpret_cast<uint2 *>(y + ((size_t)b * trows + orow) * XLD + xcol + c4) =
+                                make_uint2(pack_bf16x2(v0, v1), pack_bf16x2(v2, v3));
+                        if (lb + 1 < QB) block_sync_lds();  // the next block of rows overwrites the tiles
                     }
                 } else if constexpr (ROWS) {
                     // epilogue: dx[t, h, p] = dt[t, h] * rT[p, l] + D[h] * x[t, h, p], and the row's two inner products
@@ -717,7 +792,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             }
         }
 
-        if constexpr (TR) {
+        if constexpr (TR && SL == 1) {
             // the sum over the workgroup's heads (a whole group: eight heads) of this tile's outputs, [Q][32], goes
             // to the group's rows of the gradient
             block_sync_lds();
@@ -744,14 +819,16 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         }
         // ---- phase 2: the state leaving this chunk ----
         if (!kEarlyPrefetch && c + 1 < c_end) prefetch(c + 1);
-        float4 gq[KIND == 3 ? NB : 1][4];  // the adjoint state where this tile ends, in flight during phase 2
-        if constexpr (KIND == 3) {
-            if (an.out != nullptr) load_adjoint(adjoint_state(c + 1), gq);
+        // the other scan's state where this tile ends: the first slice in flight during phase 2, the second (two
+        // slices per wave leave no registers to hold both) requested after it
+        float4 gq[ANCH ? NB : 1][4];
+        if constexpr (ANCH) {
+            if (an.out != nullptr) load_other(adjoint_state(c + 1), 0, gq);
         }
         seg_total *= a_end;
         const int lane = phase_tid() & 63, half = lane >> 5;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) st[nb] = st[nb] * a_end;
+        for (int sn = 0; sn < SL * NB; ++sn) st[sn] = st[sn] * a_end;
         // Offsets of this lane's transposing reads for K steps 0 and 1.  Both swizzles repeat every 32 rows, so
         // step i reads at the offset of step i%2 plus (i/2)*32 rows: immediates after unrolling.
         int xo[2][2], bo[2][2][NB];
@@ -774,7 +851,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             const int k0 = ks + 8 * half;
             const int par = (ks / 16) & 1, rb = (ks / 32) * 32;
             // x[l = k0..k0+7, p = r] and B[l = k0..k0+7, n = 32 nb + r]
-            const Frag<T> xr = join(XT::tr_read(xs + xo[par][0] + rb * 32), XT::tr_read(xs + xo[par][1] + rb * 32));
+            Frag<T> xr[SL];
+#pragma unroll
+            for (int sl = 0; sl < SL; ++sl)
+                xr[sl] = join(XT::tr_read(xs + sl * XS + xo[par][0] + rb * 32), XT::tr_read(xs + sl * XS + xo[par][1] + rb * 32));
             Frag<T> bf[NB];
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
@@ -782,19 +862,28 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             const float4 wa = *reinterpret_cast<const float4 *>(w_s + k0);
             const float4 wb = *reinterpret_cast<const float4 *>(w_s + k0 + 4);
             const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
-            FragBits xh, xl;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                split_pair((float)xr.v[2 * i], wv[2 * i], (float)xr.v[2 * i + 1], wv[2 * i + 1], xh.u[i], xl.u[i]);
-            const Frag<T> xhf = xh.frag(), xlf = xl.frag();
+            for (int sl = 0; sl < SL; ++sl) {
+                FragBits xh, xl;
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                st[nb] = mma32(bf[nb], xhf, st[nb]);
-                st[nb] = mma32(bf[nb], xlf, st[nb]);
+                for (int i = 0; i < 4; ++i)
+                    split_pair((float)xr[sl].v[2 * i], wv[2 * i], (float)xr[sl].v[2 * i + 1], wv[2 * i + 1], xh.u[i], xl.u[i]);
+                const Frag<T> xhf = xh.frag(), xlf = xl.frag();
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    st[sl * NB + nb] = mma32(bf[nb], xhf, st[sl * NB + nb]);
+                    st[sl * NB + nb] = mma32(bf[nb], xlf, st[sl * NB + nb]);
+                }
             }
         }
-        if constexpr (KIND == 3) {
-            if (an.out != nullptr) write_anchor(c + 1, gq);
+        if constexpr (ANCH) {
+            if (an.out != nullptr) {
+                write_anchor(c + 1, 0, gq);
+                if constexpr (SL == 2) {
+                    load_other(adjoint_state(c + 1), 1, gq);
+                    write_anchor(c + 1, 1, gq);
+                }
+            }
         }
     }
 
@@ -864,7 +953,9 @@ static hipError_t fused_launch_transposed(const ScanShape &s, const void *x, con
                                           const ScanAnchors &an, hipStream_t st) {
     if (s.N != 32 || s.G != s.H || s.x_groups <= 0 || s.H != 8 * s.x_groups || s.P % 32 != 0 || s.seg_tiles != 0)
         return hipErrorInvalidValue;
-    const int grid = s.B * (s.H / 8) * (s.P / 32);
+    constexpr bool kWide = KIND == 6 || KIND == 7;  // both slices of a 64-wide state in one wave
+    if (kWide && s.P != 64) return hipErrorInvalidValue;
+    const int grid = s.B * (s.H / 8) * (kWide ? 1 : s.P / 32);
     fused_scan_kernel<TO, 2, kOnePassTile / 32, 8, KIND><<<dim3(grid), dim3(512), 0, st>>>(
         static_cast<const __bf16 *>(x), static_cast<const __bf16 *>(dt), A, static_cast<const __bf16 *>(Bm),
         static_cast<const __bf16 *>(Cm), nullptr, init, reset, static_cast<TO *>(out), final_states, tile_states, parts,

@@ -111,14 +111,16 @@ hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, cons
 // [B,L,H,32] are per head.  out [B,L,x_groups,P] (bf16) = the sum over each group's heads of the per-head
 // outputs, weighted by the heads' dt when adjoint.  Forward in time it also writes parts [B,L,H,P/32]: per head
 // and 32-column slice, aux_t . y_t (aux [B,L,x_groups,P]).  tile_states / final_states as for the one-pass kernel.
-// With `an.out` given, the forward scan also writes, per (b, k, h) for k = 0 .. nc and per 32-column slice, the inner
-// product of its state at the start of tile k (k = nc: its final state) with the adjoint scan's state at the same
-// timestep -- adj_tiles[b, nc - k, h] for 0 < k < nc, adj_final for k = 0 (zero without an initial state), dfinal
-// for k = nc (zero when NULL): out [B, nc+1, H, P/32], float64.
+// With `an.out` given, the scan that runs second (transposed_scan_anchors_in_adjoint says which takes them) also
+// writes, per (b, k, h) for k = 0 .. nc in forward time and per 32-column slice, the inner product of the two scans'
+// states at the start of forward tile k (k = nc: the end of the sequence): its own state entering its tile j with
+// other_tiles[b, nc - j, h] for 0 < j < nc, its initial state with other_final (zero without an initial state), its
+// final state with other_init (zero when NULL).  out [B, nc+1, H, P/32], float64.
 struct ScanAnchors {
-    const float *adj_tiles = nullptr, *adj_final = nullptr, *dfinal = nullptr;
+    const float *other_tiles = nullptr, *other_final = nullptr, *other_init = nullptr;
     double *out = nullptr;
 };
+bool transposed_scan_anchors_in_adjoint(const ScanShape &sT);
 bool transposed_scan_supported(const ScanShape &sT, int x_groups);
 hipError_t launch_transposed_scan(const ScanShape &sT, bool adjoint, const void *x, const void *dt, const float *A,
                                   const void *Bm, const void *Cm, const void *aux, const float *init,
