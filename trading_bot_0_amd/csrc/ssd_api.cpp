@@ -149,7 +149,37 @@ struct BwdWorkspace {
         init_t, dfin_t, e1, dd, u, parts, anchor, da_part, total;
 };
 
-BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
+// Which kernels a backward pass of a given shape runs on (a function of shape and dtype only: the workspace is laid
+// out for it).
+struct BwdPlan {
+    bool fast_r;        // the adjoint scan on the one-pass kernel (else staged, with gathered operands)
+    bool fast_t;        // the two transposed scans on the one-pass kernel
+    bool sum_on_chip;   // ... on its transposed kinds, which sum dB and dC over a group's heads themselves
+    bool rows_in_scan;  // the adjoint scan with the row products in its epilogue (writes dx; no float r)
+};
+
+BwdPlan plan_bwd(const ssd::ScanShape &s, const ssd::ScanShape &sT, int dtype) {
+    const int inner = dtype == SSD_DTYPE_F32 ? SSD_DTYPE_F32 : SSD_DTYPE_BF16_Y32;  // the scans write float y
+    // The one-pass kernel reverses time itself (reads the forward tensors, writes its output in forward order), reads
+    // an x that a group's heads share in place and writes the state entering every 64-step tile, which is what the
+    // staged kernels leave in their state array.
+    auto one_pass = [&](const ssd::ScanShape &shape) {
+        const int waves = ssd::fused_scan_waves(shape, inner);
+        if (waves == 0 || shape.Q != 64) return false;
+        const int64_t groups = (int64_t)shape.B * shape.G * ((shape.H / shape.G) * (shape.P / 32) / waves);
+        return (waves == 8 && groups >= kOnePassMinWorkgroups) || (waves == 2 && groups >= 4 * kOnePassMinWorkgroups);
+    };
+    BwdPlan p;
+    // bf16, headdim 32, eight heads per group, enough workgroups
+    p.sum_on_chip = inner != SSD_DTYPE_F32 && ssd::transposed_scan_supported(sT, s.G) &&
+                    (int64_t)s.B * (s.H / 8) * (s.N / 32) >= kOnePassMinWorkgroups;
+    p.fast_r = one_pass(s);  // (the padded length does not enter)
+    p.fast_t = p.sum_on_chip || one_pass(sT);
+    p.rows_in_scan = p.sum_on_chip && p.fast_r && ssd::adjoint_rows_scan_supported(s);
+    return p;
+}
+
+BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes, const BwdPlan &plan) {
     BwdWorkspace w;
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -157,20 +187,21 @@ BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes) {
         off += align_up(bytes, 256);
         return at;
     };
+    auto take_if = [&](bool used, size_t bytes) { return take(used ? bytes : 0); };
     const size_t BL = (size_t)s.B * s.L, BLp = (size_t)s.B * s.nc * s.Q;  // true and padded rows
     const size_t HP = (size_t)s.H * s.P, HN = (size_t)s.H * s.N, GN = (size_t)s.G * s.N;
     const size_t st = (size_t)s.B * s.H * s.P * s.N * sizeof(float);
     w.scan_off = take(carve(s).total);
-    w.states2 = take((size_t)s.nc * st);
-    w.dy_rev = take(BLp * HP * elem_bytes);
-    w.x_rev = take(BLp * HP * elem_bytes);
-    w.c_rev_g = take(BLp * GN * elem_bytes);
-    w.b_rev_g = take(BLp * GN * elem_bytes);
-    w.c_rev_h = take(BLp * HN * elem_bytes);
-    w.b_fwd_h = take(BL * HN * elem_bytes);
-    w.r_rev = take(BLp * HP * sizeof(float));
-    w.yb_rev = take(BLp * HN * sizeof(float));
-    w.yc = take(BL * HN * sizeof(float));
+    w.states2 = take_if(!plan.sum_on_chip, (size_t)s.nc * st);
+    w.dy_rev = take_if(!plan.fast_r || !plan.fast_t, BLp * HP * elem_bytes);
+    w.x_rev = take_if(!plan.fast_t, BLp * HP * elem_bytes);
+    w.c_rev_g = take_if(!plan.fast_r, BLp * GN * elem_bytes);
+    w.b_rev_g = take_if(!plan.fast_r, BLp * GN * elem_bytes);
+    w.c_rev_h = take_if(!plan.fast_t, BLp * HN * elem_bytes);
+    w.b_fwd_h = take_if(!plan.fast_t, BL * HN * elem_bytes);
+    w.r_rev = take_if(!plan.rows_in_scan, BLp * HP * sizeof(float));
+    w.yb_rev = take_if(!plan.sum_on_chip, BLp * HN * sizeof(float));
+    w.yc = take_if(!plan.sum_on_chip, BL * HN * sizeof(float));
     w.gfin = take(st);
     w.gfin_t = take(st);
     w.ffin_t = take(st);
@@ -377,7 +408,7 @@ int ssd_chunk_scan_bwd_workspace_bytes(const ssd_dims *dims, int dtype, size_t *
     if (out_bytes == nullptr) return fail(SSD_ERR_INVALID, "ssd: out_bytes must not be NULL");
     ssd::ScanShape s, sT;
     if (int rc = make_bwd_shapes(dims, dtype, &s, &sT)) return rc;
-    *out_bytes = carve_bwd(s, dtype == SSD_DTYPE_F32 ? 4 : 2).total;
+    *out_bytes = carve_bwd(s, dtype == SSD_DTYPE_F32 ? 4 : 2, plan_bwd(s, sT, dtype)).total;
     return SSD_OK;
 }
 
@@ -406,7 +437,8 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     OPTIONAL_PTR(dinitial_states);
     if (dD != nullptr && D == nullptr) return fail(SSD_ERR_INVALID, "ssd: dD asked for without D");
     const int eb = dtype == SSD_DTYPE_F32 ? 4 : 2;
-    const BwdWorkspace w = carve_bwd(s, eb);
+    const BwdPlan plan = plan_bwd(s, sT, dtype);
+    const BwdWorkspace w = carve_bwd(s, eb, plan);
     if (workspace_bytes < w.total)
         return fail(SSD_ERR_WORKSPACE, "ssd: backward workspace has %zu bytes, %zu needed", workspace_bytes, w.total);
     char *base = static_cast<char *>(workspace);
@@ -431,23 +463,8 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     sR.L = Lp;
     sTR.L = Lp;
     float *states2 = atf(w.states2);
-    // Which scans take the one-pass kernel.  It reverses time itself (reads the forward tensors, writes its output
-    // in forward order), reads an x that a group's heads share in place and writes the state entering every
-    // 64-step tile, which is what the staged kernels leave in their state array.  The staged kernels get their
-    // operands gathered: time-reversed copies, and one copy of a group's B or C per head.
-    auto one_pass = [&](const ssd::ScanShape &shape) {
-        const int waves = ssd::fused_scan_waves(shape, inner);
-        if (waves == 0 || shape.Q != 64) return false;
-        const int64_t groups = (int64_t)shape.B * shape.G * ((shape.H / shape.G) * (shape.P / 32) / waves);
-        return (waves == 8 && groups >= kOnePassMinWorkgroups) || (waves == 2 && groups >= 4 * kOnePassMinWorkgroups);
-    };
-    // The transposed scans with the sum over a group's heads taken on chip (they write dB and dC themselves): bf16,
-    // headdim 32, eight heads per group, enough workgroups.
-    const bool sum_on_chip = inner != SSD_DTYPE_F32 && ssd::transposed_scan_supported(sT, s.G) &&
-                             (int64_t)s.B * (s.H / 8) * (s.N / 32) >= kOnePassMinWorkgroups;
-    const bool fast_r = one_pass(sR), fast_t = sum_on_chip || one_pass(sT);
-    // the adjoint scan with the row products in its epilogue (it writes dx; no float r, no row kernel)
-    const bool rows_in_scan = sum_on_chip && fast_r && ssd::adjoint_rows_scan_supported(sR);
+    // The staged kernels get their operands gathered: time-reversed copies, and one copy of a group's B or C per head.
+    const bool fast_r = plan.fast_r, fast_t = plan.fast_t, sum_on_chip = plan.sum_on_chip, rows_in_scan = plan.rows_in_scan;
     const void *c_heads = Cm, *b_heads = Bm;
     if (!fast_r || !fast_t)
         BWD_LAUNCH(ssd::launch_gather_rows(el, dy, at(w.dy_rev), s.B, s.L, Lp, s.H, s.P, 1, true, st), "gather dy");
