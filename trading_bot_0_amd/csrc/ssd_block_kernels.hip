@@ -47,7 +47,7 @@ template <> struct Pack8<float> {
 // wave mixes the two code paths.  History
 // before t = 0 comes from state_in [B, d_conv-1, C] (the last d_conv-1 input rows of the previous call) or is
 // zero; state_out receives the last d_conv-1 input rows.
-constexpr int kPreSteps = 8;
+constexpr int kPreSteps = 16;
 
 template <typename T, int DCONV>
 __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zxbcdt, const float *__restrict__ conv_w,
@@ -67,6 +67,14 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
         const int h0 = (int)(d % HP8) * 8;
         const long long bt = d / HP8;
         const T *src = zxbcdt + (size_t)bt * E + 2 * DI + 2 * GN;
+        if (s.H % 8 == 0) {  // eight heads are one aligned 16-byte (bf16) piece on both sides
+            const Pack8<T> v = Pack8<T>::load(src + h0);
+            float o[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = softplus(v.get(i) + dt_bias[h0 + i]);
+            Pack8<T>::store(dt + (size_t)bt * s.H + h0, o);
+            return;
+        }
         for (int h = h0; h < min(h0 + 8, s.H); ++h) dt[(size_t)bt * s.H + h] = (T)softplus((float)src[h] + dt_bias[h]);
         return;
     }
@@ -122,8 +130,16 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
         dst = Cm + ((size_t)b * s.L) * GN + (c0 - DI - GN);
         dst_stride = GN;
     }
-    for (int t = t0; t < t1; ++t) {
-        const Pack8<T> v = Pack8<T>::load(row0 + (size_t)t * E + DI + c0);
+    // all of the run's input rows are requested before the first is used
+    Pack8<T> in[kPreSteps];
+#pragma unroll
+    for (int j = 0; j < kPreSteps; ++j)
+        if (t0 + j < t1) in[j] = Pack8<T>::load(row0 + (size_t)(t0 + j) * E + DI + c0);
+#pragma unroll
+    for (int j = 0; j < kPreSteps; ++j) {
+        const int t = t0 + j;
+        if (t >= t1) break;
+        const Pack8<T> v = in[j];
         float acc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -159,23 +175,25 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
     }
 }
 
-// One wave per (b, t): out = rmsnorm(y * silu(z)) * weight over the H*P channels.
-template <typename T, typename TY>
+// LPR lanes per (b, t) row, 64 / LPR rows per wave: out = rmsnorm(y * silu(z)) * weight over the H*P channels.
+// LPR is the smallest of 16, 32, 64 whose lanes cover the row with at most MAXP pieces of 8 channels each, so that
+// narrow rows (256 channels are 32 pieces) leave no lane idle.
+template <typename T, typename TY, int LPR>
 __global__ __launch_bounds__(256) void block_post_kernel(const TY *__restrict__ y, const T *__restrict__ zxbcdt,
                                                          const float *__restrict__ norm_w, float eps,
                                                          T *__restrict__ out, BlockShape s) {
     const int DI = s.H * s.P, E = 2 * DI + 2 * s.G * s.N + s.H;
-    const int lane = threadIdx.x & 63;
-    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (row >= (long long)s.B * s.L) return;
-    const TY *yr = y + (size_t)row * DI;
-    const T *zr = zxbcdt + (size_t)row * E;
-    constexpr int MAXP = 4;  // pieces of 8 channels per lane kept in registers: covers H*P <= 2048
+    const int lane = threadIdx.x & (LPR - 1);
+    const long long row = ((long long)blockIdx.x * blockDim.x + threadIdx.x) / LPR;
+    const bool live = row < (long long)s.B * s.L;  // (whole waves stay for the lane exchanges)
+    const TY *yr = y + (size_t)(live ? row : 0) * DI;
+    const T *zr = zxbcdt + (size_t)(live ? row : 0) * E;
+    constexpr int MAXP = 4;  // pieces of 8 channels per lane kept in registers: 64 lanes cover H*P <= 2048
     float v[MAXP][8];
     float ss = 0.f;
 #pragma unroll
     for (int u = 0; u < MAXP; ++u) {
-        const int c0 = (u * 64 + lane) * 8;
+        const int c0 = (u * LPR + lane) * 8;
         if (c0 < DI) {
             const Pack8<TY> yv = Pack8<TY>::load(yr + c0);
             const Pack8<T> zv = Pack8<T>::load(zr + c0);
@@ -187,12 +205,12 @@ __global__ __launch_bounds__(256) void block_post_kernel(const TY *__restrict__ 
         }
     }
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
+    for (int m = LPR / 2; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
     const float scale = rsqrtf(ss / (float)DI + eps);
 #pragma unroll
     for (int u = 0; u < MAXP; ++u) {
-        const int c0 = (u * 64 + lane) * 8;
-        if (c0 < DI) {
+        const int c0 = (u * LPR + lane) * 8;
+        if (c0 < DI && live) {
             float o[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) o[i] = v[u][i] * scale * norm_w[c0 + i];
@@ -231,25 +249,32 @@ hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, 
                  : pre_dispatch<float>(s, zxbcdt, conv_w, conv_b, dt_bias, state_in, state_out, x, Bm, Cm, dt, st);
 }
 
-hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
-                             float eps, void *out, hipStream_t st) {
+template <typename T, typename TY>
+static hipError_t post_dispatch(const BlockShape &s, const void *y, const void *zxbcdt, const float *norm_w, float eps,
+                                void *out, hipStream_t st) {
     const long long rows = (long long)s.B * s.L;
-    const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-    switch (dtype) {
-        case 0:
-            block_post_kernel<float, float><<<grid, block, 0, st>>>(static_cast<const float *>(y), static_cast<const float *>(zxbcdt),
-                                                                    norm_w, eps, static_cast<float *>(out), s);
-            break;
-        case 1:
-            block_post_kernel<__bf16, __bf16><<<grid, block, 0, st>>>(static_cast<const __bf16 *>(y), static_cast<const __bf16 *>(zxbcdt),
-                                                                      norm_w, eps, static_cast<__bf16 *>(out), s);
-            break;
-        default:  // bf16 activations with the scan's float32 y
-            block_post_kernel<__bf16, float><<<grid, block, 0, st>>>(static_cast<const float *>(y), static_cast<const __bf16 *>(zxbcdt),
-                                                                     norm_w, eps, static_cast<__bf16 *>(out), s);
-            break;
+    const int pieces = s.H * s.P / 8;
+    const TY *yy = static_cast<const TY *>(y);
+    const T *zz = static_cast<const T *>(zxbcdt);
+    T *oo = static_cast<T *>(out);
+    // the fewest lanes per row that keep a lane's pieces within what the kernel holds in registers for 64 lanes (4)
+    if (pieces <= 16 * 4) {
+        block_post_kernel<T, TY, 16><<<dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st>>>(yy, zz, norm_w, eps, oo, s);
+    } else if (pieces <= 32 * 4) {
+        block_post_kernel<T, TY, 32><<<dim3((unsigned)((rows * 32 + 255) / 256)), dim3(256), 0, st>>>(yy, zz, norm_w, eps, oo, s);
+    } else {
+        block_post_kernel<T, TY, 64><<<dim3((unsigned)((rows * 64 + 255) / 256)), dim3(256), 0, st>>>(yy, zz, norm_w, eps, oo, s);
     }
     return hipGetLastError();
+}
+
+hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                             float eps, void *out, hipStream_t st) {
+    switch (dtype) {
+        case 0: return post_dispatch<float, float>(s, y, zxbcdt, norm_w, eps, out, st);
+        case 1: return post_dispatch<__bf16, __bf16>(s, y, zxbcdt, norm_w, eps, out, st);
+        default: return post_dispatch<__bf16, float>(s, y, zxbcdt, norm_w, eps, out, st);  // the scan's float32 y
+    }
 }
 
 }  // namespace ssd
