@@ -227,3 +227,32 @@ def test_restarts_on_the_one_pass_adjoint_scan():
                                       np64(sub(dev["C"])), np64(dev["D"]), None, np64(sub(dy)), None, reset=m[rows])
     for k_out, k_ref in (("dx", "dx"), ("ddt", "ddt"), ("dB", "dB"), ("dC", "dC"), ("dinitial_states", "dinit")):
         check(got[k_out][rows], ref[k_ref], torch.bfloat16, f"one-pass reset {k_out}")
+
+
+@pytest.mark.parametrize("batch", [3, 96])
+def test_backward_inside_a_captured_graph(batch):
+    """The backward pass allocates nothing and synchronises nothing either, so a training step that holds it can be
+    captured (trading_bots/src/torch/train/update.rs:206-330): the general path (3 sequences) and the path on the
+    one-pass kernel's kinds (96).  Replays are interleaved with eager work, inputs change in place between them, and
+    every replay is compared with an eager call on the same inputs."""
+    w = Workload("bwd_graph", batch, 200, 8, 32, 64, 1, 128, dtype="bf16", init_std=0.3)
+    dev = make_inputs(w, seed=5, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(9)
+    dy = torch.randn(dev["x"].shape, generator=g, device="cuda").to(torch.bfloat16)
+    call = lambda: ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], dy, chunk=w.chunk,
+                                           initial_states=dev["init"], need_dinitial_states=True)
+    call()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = call()
+    x_keep, dy_keep = dev["x"].clone(), dy.clone()
+    for i in range(3):
+        dev["x"].copy_(x_keep * 0.5 if i % 2 else x_keep)
+        dy.copy_(dy_keep if i % 2 else dy_keep * 2)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = call()
+        torch.cuda.synchronize()
+        for k in ("dx", "ddt", "dA", "dB", "dC", "dD", "dinitial_states"):
+            assert torch.equal(captured[k], eager[k]), f"replay {i}: {k}"
