@@ -224,6 +224,14 @@ int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt,
                       const float *conv_b, const float *dt_bias, const void *conv_state_in, void *conv_state_out,
                       void *x, void *Bm, void *Cm, void *dt, void *hip_stream);
 
+/* The block's two projections (the reference's equivalents are the linear layers around its temporal mixer,
+ * trading_bots/src/torch/model/blocks/gqa.rs:82-109): out [rows, out_features] = u [rows, in_features] .
+ * w [out_features, in_features]^T, bfloat16 in and out (dtype 1), float32 accumulation; rows = batch * seqlen.
+ * in_features must be 128 or 256 and out_features a multiple of 8 (SSD_ERR_UNSUPPORTED otherwise: use the
+ * caller's BLAS).  No bias. */
+int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, int dtype, const void *u, const void *w,
+                       void *out, void *hip_stream);
+
 /* out [B,L,H*P] = rmsnorm(y * silu(z)) * norm_w over the H*P channels of a timestep (z from zxbcdt). */
 int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,
                        const float *norm_w, float eps, void *out, void *hip_stream);

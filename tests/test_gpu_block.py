@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import mamba2_block_oracle as blk
-from trading_bot_0_amd import Mamba2Block, SsdError, block_post, block_pre
+from trading_bot_0_amd import Mamba2Block, SsdError, block_post, block_pre, block_proj
 
 from _util import np64, rel_err
 
@@ -80,6 +80,40 @@ def oracle_params(b):
     return dict(in_proj=np64(b.in_proj), conv_w=np64(b.conv_w), conv_b=np64(b.conv_b), dt_bias=np64(b.dt_bias),
                 A=np64(b.A), D=np64(b.D), norm_w=np64(b.norm_w), out_proj=np64(b.out_proj), H=b.H, P=b.P, N=b.N, G=b.G,
                 eps=b.eps)
+
+
+@pytest.mark.parametrize("rows,k,n", [(300, 256, 648), (256, 128, 32), (1, 128, 264), (4099, 256, 256), (2, 256, 8),
+                                      (2049, 256, 648), (70000, 128, 168)])
+def test_projection_against_float64(rows, k, n):
+    """out = u . w^T in bf16 with float32 accumulation: every element within one bf16 rounding of the float64
+    product of the same bf16 inputs (plus a floor for sums that cancel); ragged row counts, column blocks and
+    chunks."""
+    g = torch.Generator().manual_seed(rows + n)
+    u = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16)
+    out = block_proj(u.cuda(), w.cuda())
+    torch.cuda.synchronize()
+    assert out.shape == (rows, n) and out.dtype == torch.bfloat16
+    ref = u.double().numpy() @ w.double().numpy().T
+    o = out.float().cpu().numpy().astype(np.float64)
+    rms = np.sqrt(np.mean(ref * ref))
+    bad = np.abs(o - ref) > 2.0 ** -8 * np.abs(ref) + 1e-4 * rms
+    assert np.isfinite(o).all() and not bad.any(), f"{int(bad.sum())} elements off"
+
+
+def test_projection_keeps_leading_dimensions_and_refuses_other_shapes():
+    u = torch.randn(3, 50, 256).to(torch.bfloat16).cuda()
+    w = torch.randn(40, 256).to(torch.bfloat16).cuda()
+    out = block_proj(u, w)
+    assert out.shape == (3, 50, 40)
+    ref = u.double().cpu().numpy().reshape(150, 256) @ w.double().cpu().numpy().T
+    assert np.abs(out.float().cpu().numpy().reshape(150, 40) - ref).max() <= 2.0 ** -7 * np.abs(ref).max()
+    with pytest.raises(SsdError):
+        block_proj(torch.randn(8, 96).to(torch.bfloat16).cuda(), torch.randn(8, 96).to(torch.bfloat16).cuda())
+    with pytest.raises(SsdError):
+        block_proj(u, torch.randn(42, 256).to(torch.bfloat16).cuda())
+    with pytest.raises(ValueError):
+        block_proj(u.float(), w.float())
 
 
 def test_block_forward_float32_matches_the_oracle_block():

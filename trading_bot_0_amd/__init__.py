@@ -17,4 +17,4 @@ from .ssd import (  # noqa: F401
     workspace_bytes,
 )
 from .stream_state import SsdStreamState  # noqa: F401
-from .block import Mamba2Block, Mamba2StreamState, block_post, block_pre  # noqa: F401
+from .block import Mamba2Block, Mamba2StreamState, block_post, block_pre, block_proj  # noqa: F401

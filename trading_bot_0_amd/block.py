@@ -34,8 +34,10 @@ def _lib():
         P = c_void_p
         lib.ssd_block_pre_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_block_post_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, P]
+        lib.ssd_block_proj_fwd.argtypes = [c_int64, c_int64, c_int64, c_int, P, P, P, P]
         lib.ssd_block_pre_fwd.restype = c_int
         lib.ssd_block_post_fwd.restype = c_int
+        lib.ssd_block_proj_fwd.restype = c_int
         _bound = True
     return lib
 
@@ -97,6 +99,29 @@ def block_post(y, zxbcdt, norm_w, nheads, headdim, dstate, ngroups, eps=1e-5):
     dims = SsdBlockDims(Bsz, L, H, P, N, G, 4)
     ssd._check(lib, lib.ssd_block_post_fwd(byref(dims), code, y.data_ptr(), zxbcdt.data_ptr(), norm_w.data_ptr(),
                                            c_float(eps), out.data_ptr(), ssd._stream_ptr(zxbcdt)))
+    return out
+
+
+def block_proj_supported(u: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `block_proj` takes this product (else the caller's BLAS does it)."""
+    return (u.is_cuda and u.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and u.shape[-1] in (128, 256)
+            and weight.shape[0] % 8 == 0 and u.numel() > 0)
+
+
+def block_proj(u: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """u [..., in_features] (bf16) times weight [out_features, in_features]^T -> [..., out_features] (bf16), float32
+    accumulation: the block's in- and out-projection as one memory-bound kernel."""
+    lib = _lib()
+    if u.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError(f"block_proj takes bfloat16 tensors, got {u.dtype} and {weight.dtype}")
+    if weight.dim() != 2 or u.shape[-1] != weight.shape[1]:
+        raise ValueError(f"block_proj: u [..., {u.shape[-1]}] does not match weight {tuple(weight.shape)}")
+    if not u.is_contiguous() or not weight.is_contiguous():
+        raise ValueError("block_proj takes contiguous tensors")
+    rows = u.numel() // u.shape[-1]
+    out = torch.empty(u.shape[:-1] + (weight.shape[0],), dtype=torch.bfloat16, device=u.device)
+    ssd._check(lib, lib.ssd_block_proj_fwd(rows, u.shape[-1], weight.shape[0], ssd.SSD_DTYPE_BF16, u.data_ptr(),
+                                           weight.data_ptr(), out.data_ptr(), ssd._stream_ptr(u)))
     return out
 
 
@@ -163,8 +188,7 @@ class Mamba2Block:
             raise ValueError(f"block input must be [batch, seqlen, {self.d_model}], got {tuple(u.shape)}")
         if reset is not None and state is not None:
             raise ValueError("restarts inside the window and a carried conv state cannot be combined")
-        dt_ = u.dtype
-        zxbcdt = torch.matmul(u, self.in_proj.to(dt_).t()).contiguous()
+        zxbcdt = self._project(u, self.in_proj)
         if state is None:
             x, Bm, Cm, dt = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G)
             y, _ = ssd.ssd_chunk_scan(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk, return_final_states=False,
@@ -175,7 +199,16 @@ class Mamba2Block:
             state.conv = conv
             y = state.ssm.init_from_prefix(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk)
         yn = block_post(y, zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
-        return torch.matmul(yn, self.out_proj.to(dt_).t())
+        return self._project(yn, self.out_proj)
+
+    def _project(self, u: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        """u . weight^T in the activation dtype: the library's kernel where it takes the shape (bf16, in_features 128
+        or 256, a tall u), else the BLAS behind torch."""
+        w = weight.to(u.dtype)
+        u = u.contiguous()
+        if block_proj_supported(u, w) and u.numel() // u.shape[-1] >= 16384:
+            return block_proj(u, w.contiguous())
+        return torch.matmul(u, w.t()).contiguous()
 
     def step(self, u_t: torch.Tensor, state: Mamba2StreamState) -> torch.Tensor:
         """One timestep for every stream: u_t [B,d_model] -> [B,d_model]; advances `state` in place."""

@@ -721,6 +721,26 @@ int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt,
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block pre-scan launch");
 }
 
+int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, int dtype, const void *u, const void *w,
+                       void *out, void *hip_stream) {
+    if (dtype != SSD_DTYPE_BF16)
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: the block projection takes dtype 1 (bfloat16), got %d", dtype);
+    if (rows <= 0 || in_features <= 0 || out_features <= 0)
+        return fail(SSD_ERR_INVALID, "ssd: projection sizes must be positive, got %lld x %lld -> %lld", (long long)rows,
+                    (long long)in_features, (long long)out_features);
+    if (in_features > 0x7fffffff || out_features > 0x7fffffff ||
+        !ssd::block_proj_supported(rows, (int)in_features, (int)out_features))
+        return fail(SSD_ERR_UNSUPPORTED,
+                    "ssd: the block projection needs in_features 128 or 256 and out_features a multiple of 8, got "
+                    "%lld and %lld",
+                    (long long)in_features, (long long)out_features);
+    REQUIRE_PTR(u);
+    REQUIRE_PTR(w);
+    REQUIRE_PTR(out);
+    hipError_t e = ssd::launch_block_proj(rows, (int)in_features, (int)out_features, u, w, out, (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "block projection launch");
+}
+
 int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,
                        const float *norm_w, float eps, void *out, void *hip_stream) {
     ssd::BlockShape s;

@@ -1,0 +1,153 @@
+// The block's projections: out[m, n] = sum_k u[m, k] w[n, k] for a tall u (rows = batch * seqlen, 128 or 256
+// columns) and a small weight matrix, bf16 in and out, float32 accumulation (gfx950).
+//
+// With K of a few hundred the product is bound by memory, not by the matrix cores: u is read once, out written once
+// (0.95 GB for 524 288 rows, 256 -> 648).  A workgroup owns a block of at most 160 output columns and a range of
+// rows: it puts its rows of w into LDS once (84 KB), and from then on its eight waves run without a barrier -- each
+// takes tiles of 32 rows, loads its rows of u straight into MFMA operand fragments (u and w are both contiguous
+// along K, so a lane's eight K elements are one 16-byte load; the next tile's rows are in flight during this
+// tile's products), and walks the block's columns in chunks of 32 with the w fragments read from LDS.  The MFMA's first operand is w, so that a lane ends up with one row m and runs of
+// four consecutive columns n; two chunks are collected in an LDS tile of the wave's own and written out with
+// adjacent lanes on adjacent 16-byte pieces of a row (stores scattered over 32 rows straight from the
+// accumulators' layout run at a fraction of the memory system's rate).
+#include "ssd_device.h"
+
+namespace ssd {
+
+namespace {
+
+constexpr int kProjWaves = 8;         // waves per workgroup: two per SIMD, 256 registers each
+constexpr int kProjBlockCols = 160;   // most output columns per workgroup (their rows of w stay in LDS)
+constexpr int kProjChunk = 32;        // output columns per MFMA tile
+constexpr int kProjTiles = 8;         // tiles of 32 rows per wave
+
+template <int KS>  // K = 16 * KS
+__global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf16 *__restrict__ u,
+                                                                      const __bf16 *__restrict__ w,
+                                                                      __bf16 *__restrict__ out, long long M, int N,
+                                                                      int col_blocks, int block_cols) {
+    constexpr int K = 16 * KS, NTHR = 64 * kProjWaves;
+    constexpr int ROWB = K * 2 + 16;        // bytes of a staged row of w: 16 bytes of padding shift the banks
+    constexpr int kTileRowB = 64 * 2 + 16;  // a row of a wave's output tile: 64 columns and 16 bytes of padding
+    __shared__ __attribute__((aligned(16))) unsigned char wsm[kProjBlockCols * ROWB];
+    __shared__ __attribute__((aligned(16))) unsigned char otile[kProjWaves][32 * kTileRowB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Workgroups go to the eight XCDs in turn, each XCD with an L2 of its own: the column blocks of a range of rows
+    // are consecutive workgroups of ONE XCD, so that they run at the same time and all but the first find those
+    // rows of u in its L2.
+    const int xcd = blockIdx.x % 8, within = blockIdx.x / 8;
+    const int cb = within % col_blocks;
+    const long long rg = (long long)(within / col_blocks) * 8 + xcd;
+    const int n0 = cb * block_cols;                 // this workgroup's first column
+    const int ncols = min(block_cols, N - n0);      // a multiple of 8
+    const int chunks = (ncols + kProjChunk - 1) / kProjChunk;
+    const long long row0 = rg * kProjTiles * (32LL * kProjWaves);
+    if (row0 >= M) return;  // the grid is padded to whole rounds of XCDs
+
+    {   // rows n0 .. n0 + 32 * chunks - 1 of w, all requested before the first is written to LDS (rows past N repeat
+        // the last one; their columns are never stored)
+        constexpr int FILL = (kProjBlockCols * (K / 8) + NTHR - 1) / NTHR;
+        const int pieces = chunks * kProjChunk * (K / 8);
+        uint4 q[FILL];
+#pragma unroll
+        for (int i = 0; i < FILL; ++i) {
+            const int p = min(tid + i * NTHR, pieces - 1);
+            q[i] = *reinterpret_cast<const uint4 *>(w + (size_t)min(n0 + p / (K / 8), N - 1) * K + (p % (K / 8)) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < FILL; ++i) {
+            const int p = tid + i * NTHR;
+            if (p < pieces) *reinterpret_cast<uint4 *>(wsm + (p / (K / 8)) * ROWB + (p % (K / 8)) * 16) = q[i];
+        }
+    }
+    __syncthreads();
+
+    const int r = lane & 31, half = lane >> 5;
+    unsigned char *tile = otile[wave];
+    auto tile_row0 = [&](int t) { return row0 + (long long)t * (32 * kProjWaves) + wave * 32; };
+    // this lane's part of its row of u: K elements 16 ks + 8 half .. + 7 for every K step (rows past M repeat the
+    // last row; they are never stored)
+    auto load_rows = [&](int t, Frag<__bf16>(&uf)[KS]) {
+        const __bf16 *ur = u + (size_t)min(tile_row0(t) + r, M - 1) * K + 8 * half;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) uf[ks].v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(ur + 16 * ks));
+    };
+    auto tile_product = [&](int t, const Frag<__bf16>(&uf)[KS]) {
+        const long long m0 = tile_row0(t);
+        for (int c0 = 0; c0 < chunks; c0 += 2) {
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                const int c = c0 + sub;
+                if (c >= chunks) break;
+                const unsigned char *wb = wsm + (c * kProjChunk + r) * ROWB + half * 16;
+                f32x16 acc = {0}, acc_odd = {0};  // two chains of dependent MFMAs instead of one
+#pragma unroll
+                for (int ks = 0; ks < KS; ks += 2) {
+                    Frag<__bf16> wf0, wf1;
+                    wf0.v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(wb + ks * 32));
+                    wf1.v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(wb + ks * 32 + 32));
+                    acc = mma32(wf0, uf[ks], acc);
+                    acc_odd = mma32(wf1, uf[ks + 1], acc_odd);
+                }
+                acc = acc + acc_odd;
+                // acc[4 vg + i] = out[m, n0 + 32 c + 8 vg + 4 half + i]
+#pragma unroll
+                for (int vg = 0; vg < 4; ++vg)
+                    *reinterpret_cast<uint2 *>(tile + r * kTileRowB + (sub * 32 + 8 * vg + 4 * half) * 2) = make_uint2(
+                        pack_bf16x2(acc[4 * vg], acc[4 * vg + 1]), pack_bf16x2(acc[4 * vg + 2], acc[4 * vg + 3]));
+            }
+            // The tile was written by this wave's other lanes: LDS works a wave's requests off in order, so all that
+            // is needed is that the compiler keeps the order (a fence would also wait for the stores to memory).
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int pass = 0; pass < 4; ++pass) {
+                const int row = pass * 8 + (lane >> 3), col = c0 * kProjChunk + (lane & 7) * 8;
+                const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kTileRowB + (lane & 7) * 16);
+                if (m0 + row < M && col < ncols)
+                    *reinterpret_cast<uint4 *>(out + (size_t)(m0 + row) * N + n0 + col) = v;
+            }
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+        }
+    };
+    // Two sets of row fragments: the next tile's rows are requested before this tile's products, because loads and
+    // stores complete in order per wave -- requested after, they would wait for this tile's stores to reach memory.
+    Frag<__bf16> ua[KS], ub[KS];
+    load_rows(0, ua);
+    for (int t = 0; t < kProjTiles; t += 2) {
+        if (tile_row0(t) >= M) break;
+        load_rows(t + 1, ub);
+        tile_product(t, ua);
+        if (tile_row0(t + 1) >= M) break;
+        if (t + 2 < kProjTiles) load_rows(t + 2, ua);
+        tile_product(t + 1, ub);
+    }
+}
+
+}  // namespace
+
+bool block_proj_supported(long long rows, int in_features, int out_features) {
+    return rows > 0 && (in_features == 128 || in_features == 256) && out_features > 0 && out_features % 8 == 0;
+}
+
+hipError_t launch_block_proj(long long rows, int in_features, int out_features, const void *u, const void *w, void *out,
+                             hipStream_t st) {
+    if (!block_proj_supported(rows, in_features, out_features)) return hipErrorInvalidValue;
+    // column blocks of equal size (a multiple of 8 columns), at most kProjBlockCols
+    const int col_blocks = (out_features + kProjBlockCols - 1) / kProjBlockCols;
+    const int block_cols = ((out_features + col_blocks - 1) / col_blocks + 7) / 8 * 8;
+    const long long rows_per_group = 32LL * kProjWaves * kProjTiles;
+    const long long groups = ((rows + rows_per_group - 1) / rows_per_group + 7) / 8 * 8 * col_blocks;
+    if (groups > 0x7fffffffLL || block_cols > kProjBlockCols) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)groups), block(64 * kProjWaves);
+    const __bf16 *uu = static_cast<const __bf16 *>(u), *ww = static_cast<const __bf16 *>(w);
+    __bf16 *oo = static_cast<__bf16 *>(out);
+    if (in_features == 128)
+        block_proj_kernel<8><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, col_blocks, block_cols);
+    else
+        block_proj_kernel<16><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, col_blocks, block_cols);
+    return hipGetLastError();
+}
+
+}  // namespace ssd

@@ -99,6 +99,11 @@ hipError_t launch_steps(const StepShape &s, int nsteps, int dtype, float *state,
 // dt = softplus(dt_raw + dt_bias); conv state [B, d_conv-1, H*P + 2*G*N] in the activation dtype (both optional).
 // post: out [B,L,H*P] = rmsnorm(y * silu(z)) * norm_w.  dtype 2 = bf16 activations with float32 y.
 bool block_supported(const BlockShape &s);
+// The block's projections in bf16: out [rows, out_features] = u [rows, in_features] . w [out_features, in_features]^T,
+// float32 accumulation.  in_features 128 or 256, out_features a multiple of 8.
+bool block_proj_supported(long long rows, int in_features, int out_features);
+hipError_t launch_block_proj(long long rows, int in_features, int out_features, const void *u, const void *w, void *out,
+                             hipStream_t stream);
 hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w,
                             const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
                             void *x, void *Bm, void *Cm, void *dt, hipStream_t stream);

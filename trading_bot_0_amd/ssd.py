@@ -44,6 +44,7 @@ EXPORTED_SYMBOLS = (
     "ssd_steps_fwd",
     "ssd_block_pre_fwd",
     "ssd_block_post_fwd",
+    "ssd_block_proj_fwd",
     "ssd_chunk_scan_bwd_workspace_bytes",
     "ssd_chunk_scan_bwd",
 )
