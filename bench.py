@@ -22,7 +22,8 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
   backward     the backward pass of the scan at the same shape: time per call, and its compulsory traffic
                (x, dt, B, C, dy read; dx, ddt, dB, dC written) against the HBM peak
   mamba2_block the block around the scan at the policy shape (d_model = nheads*headdim): whole block, and the
-               library's pre-scan and post-scan kernels alone with their GB/s
+               library's projection, pre-scan and post-scan kernels alone with their GB/s (the projections
+               also through the BLAS behind torch, for comparison)
   cpu_baseline the plain-C oracle (sequential recurrence, float32, OpenMP) timed on this
                box's host cores on a bounded batch slice of the same workload
 
@@ -362,9 +363,9 @@ def main():
             {"name": "mamba2_infer_step", "time_ms": t_step, "config": {"batch": 4, "seq_len": 1, "dtype": "BFloat16"}},
         ]
 
-    # ---- the Mamba-2 block around the scan (projections by torch's GEMM, the rest in the library) ----
+    # ---- the Mamba-2 block around the scan: its stages through their own entry points, and the whole block ----
     if not args.no_block:
-        from trading_bot_0_amd import Mamba2Block, block_post, block_pre
+        from trading_bot_0_amd import Mamba2Block, block_post, block_pre, block_proj
         bw = WORKLOADS["policy_bf16"]
         blk = Mamba2Block(d_model=bw.nheads * bw.headdim, nheads=bw.nheads, headdim=bw.headdim, dstate=bw.dstate,
                           ngroups=bw.ngroups, chunk=bw.chunk)
@@ -391,10 +392,23 @@ def main():
         t_pre = timed(lambda: block_pre(zx, blk.conv_w, blk.conv_b, blk.dt_bias, blk.H, blk.P, blk.N, blk.G))
         t_post = timed(lambda: block_post(ys_, zx, blk.norm_w, blk.H, blk.P, blk.N, blk.G))
         t_block = timed(lambda: blk.forward(u), n=10)
+        w_in, w_out = blk.in_proj.to(u.dtype).contiguous(), blk.out_proj.to(u.dtype).contiguous()
+        yn = block_post(ys_, zx, blk.norm_w, blk.H, blk.P, blk.N, blk.G)
+        rows = bw.batch * bw.seqlen
+        in_bytes = e * rows * (blk.d_model + w_in.shape[0])
+        out_bytes = e * rows * (blk.d_inner + blk.d_model)
+        t_in = timed(lambda: block_proj(u, w_in))
+        t_out = timed(lambda: block_proj(yn, w_out))
+        t_in_blas = timed(lambda: torch.matmul(u, w_in.t()))
+        t_out_blas = timed(lambda: torch.matmul(yn, w_out.t()))
         out["mamba2_block"] = {"d_model": blk.d_model, "ms": round(t_block, 4),
+                               "in_proj_ms": round(t_in, 4), "in_proj_GBps": round(in_bytes / t_in / 1e6, 1),
+                               "in_proj_blas_ms": round(t_in_blas, 4),
                                "pre_ms": round(t_pre, 4), "pre_GBps": round(pre_bytes / t_pre / 1e6, 1),
-                               "post_ms": round(t_post, 4), "post_GBps": round(post_bytes / t_post / 1e6, 1)}
-        del u, zx, xs_, bs_, cs_, ds_, ys_, blk
+                               "post_ms": round(t_post, 4), "post_GBps": round(post_bytes / t_post / 1e6, 1),
+                               "out_proj_ms": round(t_out, 4), "out_proj_GBps": round(out_bytes / t_out / 1e6, 1),
+                               "out_proj_blas_ms": round(t_out_blas, 4)}
+        del u, zx, xs_, bs_, cs_, ds_, ys_, yn, blk
 
     # ---- CPU baseline: the C oracle on a bounded batch slice ---------------------------------
     if not args.no_cpu_baseline:
