@@ -992,16 +992,19 @@ static hipError_t fused_dispatch_w(const ScanShape &s, int waves, const void *x,
         if (waves == 4)
             return fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
         return hipErrorInvalidValue;
+    } else {  // (an else, so that no eight-wave kernel is instantiated for the 128-wide state)
+        if (waves == 8)
+            return fused_launch<TO, NK, QB, 8>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
+        if (waves == 4)
+            return fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
+        // two waves: one head of 64 columns with its own B and C (the transposed scans of the backward pass);
+        // the staging offsets fit a 32-wide state only, and only the float-output library instantiates it
+        if constexpr (NK == 2 && sizeof(TO) == 4) {
+            if (waves == 2)
+                return fused_launch<TO, NK, QB, 2>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
+        }
+        return hipErrorInvalidValue;
     }
-    if (waves == 8) return fused_launch<TO, NK, QB, 8>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
-    if (waves == 4) return fused_launch<TO, NK, QB, 4>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
-    // two waves: one head of 64 columns with its own B and C (the transposed scans of the backward pass);
-    // the staging offsets fit a 32-wide state only, and only the float-output library instantiates it
-    if constexpr (NK == 2 && sizeof(TO) == 4) {
-        if (waves == 2)
-            return fused_launch<TO, NK, QB, 2>(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
-    }
-    return hipErrorInvalidValue;
 }
 
 template <typename TO>
