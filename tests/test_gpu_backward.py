@@ -256,3 +256,47 @@ def test_backward_inside_a_captured_graph(batch):
         torch.cuda.synchronize()
         for k in ("dx", "ddt", "dA", "dB", "dC", "dD", "dinitial_states"):
             assert torch.equal(captured[k], eager[k]), f"replay {i}: {k}"
+
+
+def test_calls_from_several_threads_on_their_own_streams():
+    """The library keeps no state between calls but a thread-local error string, so host threads may call it at the
+    same time (the reference's tests run multi-threaded in one process, trading_bots/src/torch/test_rng.rs:1-40): four
+    threads, each with its own stream, inputs and workspace, run forward and backward several times; every result
+    equals the single-threaded one bit for bit."""
+    import threading
+    w = Workload("threads", 6, 257, 8, 32, 64, 1, 128, dtype="bf16", init_std=0.3)
+    cases = []
+    for seed in range(4):
+        dev = make_inputs(w, seed=40 + seed, device="cuda")
+        dy = torch.randn(dev["x"].shape, generator=torch.Generator(device="cuda").manual_seed(seed), device="cuda").to(torch.bfloat16)
+        y, fin = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk, initial_states=dev["init"])
+        grads = ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], dy, chunk=w.chunk,
+                                        initial_states=dev["init"], need_dinitial_states=True)
+        cases.append((dev, dy, y, fin, grads))
+    torch.cuda.synchronize()
+    failures = []
+
+    def worker(i):
+        dev, dy, y_ref, fin_ref, g_ref = cases[i]
+        stream = torch.cuda.Stream()
+        try:
+            with torch.cuda.stream(stream):
+                for _ in range(5):
+                    y, fin = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                                            initial_states=dev["init"])
+                    g = ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], dy, chunk=w.chunk,
+                                                initial_states=dev["init"], need_dinitial_states=True)
+                    stream.synchronize()
+                    ok = torch.equal(y, y_ref) and torch.equal(fin, fin_ref) and all(
+                        torch.equal(g[k], g_ref[k]) for k in ("dx", "ddt", "dA", "dB", "dC", "dD", "dinitial_states"))
+                    if not ok:
+                        failures.append(i)
+        except Exception as e:  # noqa: BLE001 - reported below
+            failures.append((i, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures
