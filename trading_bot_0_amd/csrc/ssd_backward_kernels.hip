@@ -371,8 +371,9 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
     }
     const double tot = last_lane(wave_inclusive_scan(da)), totd = last_lane(wave_inclusive_scan((double)ddv));
     if (lane == 0) {
-        dA_part[id] = tot;
-        dD_part[id] = totd;
+        const size_t at_part = (size_t)h * ((size_t)s.B * s.nc) + (size_t)b * s.nc + c;  // [H, B*nc]: a head's parts together
+        dA_part[at_part] = tot;
+        dD_part[at_part] = totd;
     }
 }
 
@@ -461,20 +462,21 @@ __global__ __launch_bounds__(256) void bwd_ddt_heads_kernel(const T *__restrict_
         sdd += __shfl_xor(sdd, d, 64);
     }
     if (tl == 0) {
-        dA_part[id * NH + h] = da;
-        dD_part[id * NH + h] = sdd;
+        const size_t at_part = (size_t)h * ((size_t)s.B * s.nc) + id;  // [H, B*nc]: a head's parts together
+        dA_part[at_part] = da;
+        dD_part[at_part] = sdd;
     }
 }
 
-// One workgroup per head: dA[h] = the sum over (b, c) of dA_part[b,c,h], dD[h] likewise (float64 sums).
+// One workgroup per head: dA[h] = the sum over (b, c) of dA_part[h,b,c], dD[h] likewise (float64 sums).
 __global__ __launch_bounds__(256) void bwd_head_sums_kernel(const double *__restrict__ dA_part, const double *__restrict__ dD_part,
                                                             float *__restrict__ dA, float *__restrict__ dD, ScanShape s) {
     __shared__ double red[2][256];
     const int h = blockIdx.x;
     double sa = 0.0, sd = 0.0;
     for (long long i = threadIdx.x; i < (long long)s.B * s.nc; i += blockDim.x) {
-        sa += dA_part[i * s.H + h];
-        sd += dD_part[i * s.H + h];
+        sa += dA_part[(size_t)h * ((size_t)s.B * s.nc) + i];
+        sd += dD_part[(size_t)h * ((size_t)s.B * s.nc) + i];
     }
     red[0][threadIdx.x] = sa;
     red[1][threadIdx.x] = sd;
