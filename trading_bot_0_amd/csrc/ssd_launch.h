@@ -175,8 +175,9 @@ hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, con
                               const float *rev_prev, const float *rev_final, const float *init_t, const float *fwd_final,
                               const float *dfin_t, const unsigned char *reset, double *anchor, hipStream_t stream);
 // q_t between the anchors of its chunk (chunk <= 64 steps); ddt = e1 + A q; dA_part[h,b,c] = the chunk's sum of
-// dt q, dD_part[h,b,c] = its sum of dd.  With parts given ([B,L,H,nparts], the pieces of C . yC), e1 holds the pairs (e1, dd)
-// of the adjoint scan with row products and u = sum of the parts - dt e1 is formed here (u and dd unused).
+// dt q, dD_part[h,b,c] = its sum of dd.  With parts given ([B,L,H,nparts], the pieces of C . yC), e1 holds the
+// pairs (e1, dd) of the adjoint scan with row products and u = sum of the parts - dt e1 is formed here (u and dd
+// unused).
 // With raw_anchors > 0, anchor holds that many pieces per (b, c, h) ([B, nc+1, H, raw_anchors], as ScanAnchors
 // writes them) of the two states' inner product, and the first step's decay exp(dt A) -- zero where `reset` marks
 // the chunk's first step -- is applied here.
