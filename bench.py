@@ -16,7 +16,7 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
   stages       the staged kernels issued one by one through their own entry points, each with
                its algorithmic bytes, GB/s and (stages 2, 4) dense MFMA rate; measured in both cases
   stream_step  the single-timestep update at batch 4096: latency and GB/s; stream_steps_one_launch: the same
-               64 steps as one launch of the multi-step kernel
+               64 steps as one call of ssd_steps_fwd (which runs 16 steps or more on the one-pass scan)
   reference_suite  the reference's historical benchmark cases for this path (batch 4, seq_len 4096,
                BFloat16), for the SSD op alone, in the reference's result schema
   backward     the backward pass of the scan at the same shape: time per call, and its compulsory traffic

@@ -156,7 +156,8 @@ def oracle_steps(cpu, reset=None):
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("shape", [(5, 4, 16, 16, 1, 7), (3, 8, 32, 64, 1, 16), (2, 16, 64, 128, 2, 5),
-                                   (6, 6, 32, 32, 3, 1), (4, 8, 16, 128, 1, 9)])
+                                   (6, 6, 32, 32, 3, 1), (4, 8, 16, 128, 1, 9),
+                                   (4, 8, 32, 64, 1, 150), (2, 16, 64, 128, 2, 70)])   # long runs: on the one-pass scan
 def test_steps_in_one_launch_match_the_oracle(shape, dtype):
     from trading_bot_0_amd import ssd_steps
     Bsz, H, P, N, G, T = shape
@@ -205,6 +206,34 @@ def test_steps_equal_repeated_single_steps_and_reset_cleans_a_poisoned_row():
     assert torch.isfinite(y_one).all() and torch.isfinite(b.state).all()
     assert rel_err(y_one, y_ref.double().cpu().numpy()) <= 1e-5
     assert rel_err(b.state, a.state.double().cpu().numpy()) <= 1e-5
+
+
+def test_long_runs_of_steps_on_the_scan_kernel_keep_the_reset_semantics():
+    """64 steps of bf16 streams run on the one-pass scan (state in place as its initial and final state): a row
+    that restarts before the first step may hold anything, a row without restarts continues from its state, and
+    the results agree with single steps to the bf16 bar."""
+    w = Workload("long", 5, 64, 8, 32, 64, 1, 32, dtype="bf16", init_std=0.5)
+    dev = to_dev(make_inputs(w, seed=6))
+    a = SsdStreamState(dev["init"].clone(), True)
+    b = SsdStreamState(dev["init"].clone(), True)
+    reset = torch.zeros((w.batch, w.seqlen), dtype=torch.bool, device="cuda")
+    reset[1, 0] = True
+    reset[3, 17] = True
+    reset[4, 63] = True
+    b.state[1].fill_(float("nan"))
+    ys = []
+    for t in range(w.seqlen):
+        rows = reset[:, t]
+        if bool(rows.any()):
+            a.reset_rows(rows)
+        ys.append(a.step(dev["x"][:, t].contiguous(), dev["dt"][:, t].contiguous(), dev["A"],
+                         dev["B"][:, t].contiguous(), dev["C"][:, t].contiguous(), dev["D"], y_dtype=torch.float32))
+    y_one = b.steps(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], reset=reset, y_dtype=torch.float32)
+    torch.cuda.synchronize()
+    y_ref = torch.stack(ys, 1)
+    assert torch.isfinite(y_one).all() and torch.isfinite(b.state).all()
+    assert rel_err(y_one, y_ref.double().cpu().numpy()) <= TOL[torch.bfloat16]
+    assert rel_err(b.state, a.state.double().cpu().numpy()) <= TOL[torch.bfloat16]
 
 
 def test_steps_refuses_what_it_cannot_hold_in_registers():

@@ -379,11 +379,13 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // ---- running state of this unit: st[nb][v] = H[p = r, n = 32 nb + 8 (v/4) + 4 half + v%4] ----
     // (with two slices per wave: slice sl in st[sl * NB ..])
     f32x16 st[SL * NB];
+    // a restart before the first step: the initial state is not read at all (it may hold anything)
+    const bool fresh = !ADJ && rsb != nullptr && seg == 0 && rsb[0] != 0;
 #pragma unroll
     for (int sl = 0; sl < SL; ++sl) {
-        const float *ib = init ? init + ((((size_t)b * S + seg) * s.H + h) * s.P + (pb + sl) * 32 + (lane0 & 31)) * N +
-                                     4 * (lane0 >> 5)
-                               : nullptr;
+        const float *ib = init && !fresh ? init + ((((size_t)b * S + seg) * s.H + h) * s.P + (pb + sl) * 32 + (lane0 & 31)) * N +
+                                               4 * (lane0 >> 5)
+                                         : nullptr;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
