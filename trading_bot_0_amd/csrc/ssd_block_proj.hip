@@ -6,10 +6,11 @@
 // rows: it puts its rows of w into LDS once (84 KB), and from then on its eight waves run without a barrier -- each
 // takes tiles of 32 rows, loads its rows of u straight into MFMA operand fragments (u and w are both contiguous
 // along K, so a lane's eight K elements are one 16-byte load; the next tile's rows are in flight during this
-// tile's products), and walks the block's columns in chunks of 32 with the w fragments read from LDS.  The MFMA's first operand is w, so that a lane ends up with one row m and runs of
-// four consecutive columns n; two chunks are collected in an LDS tile of the wave's own and written out with
-// adjacent lanes on adjacent 16-byte pieces of a row (stores scattered over 32 rows straight from the
-// accumulators' layout run at a fraction of the memory system's rate).
+// tile's products), and walks the block's columns in chunks of 32 with the w fragments read from LDS.  The MFMA's
+// first operand is w, so that a lane ends up with one row m and runs of four consecutive columns n; two chunks are
+// collected in an LDS tile of the wave's own and written out with adjacent lanes on adjacent 16-byte pieces of a
+// row (stores scattered over 32 rows straight from the accumulators' layout run at a fraction of the memory
+// system's rate).
 #include "ssd_device.h"
 
 namespace ssd {
