@@ -206,4 +206,27 @@ inline DeviceBuffer ssd_step(StreamState &state, const TensorView &x, const Tens
     return y;
 }
 
+// y = ssd_steps(state, x, dt, A, B, C, D, reset): advances every stream by T timesteps in one call, in place
+// (x [B,T,H,P], dt [B,T,H], B, C [B,T,G,N]: the scan's layout; reset: device pointer to [B,T] bytes or NULL, a
+// non-zero byte empties that stream right before the step -- the rollout's advance -> reset slots -> forward,
+// train/rollout.rs:130-135,209-235); returns y [B,T,H,P] in x's type.
+inline DeviceBuffer ssd_steps(StreamState &state, const TensorView &x, const TensorView &dt, const TensorView &A,
+                              const TensorView &Bm, const TensorView &Cm, const TensorView *D,
+                              const uint8_t *reset = nullptr, hipStream_t stream = nullptr) {
+    if (x.rank != 4 || Bm.rank != 4) throw Error(SSD_ERR_INVALID, "SSD steps x must be [B,T,H,P] and B [B,T,G,N]");
+    const int64_t B = state.batch(), H = state.nheads(), P = state.headdim(), N = state.dstate(), T = x.shape[1],
+                  G = Bm.shape[2];
+    detail::require(x, "x", x.dtype, {B, T, H, P});
+    detail::require(dt, "dt", x.dtype, {B, T, H});
+    detail::require(A, "A", DType::F32, {H});
+    detail::require(Bm, "B", x.dtype, {B, T, G, N});
+    detail::require(Cm, "C", x.dtype, {B, T, G, N});
+    if (D) detail::require(*D, "D", DType::F32, {H});
+    const ssd_step_dims dims = {B, H, P, N, G};
+    DeviceBuffer y((size_t)x.numel() * element_size(x.dtype));
+    check(ssd_steps_fwd(&dims, T, (int)x.dtype, state.data(), reset, x.ptr, dt.ptr, static_cast<const float *>(A.ptr), Bm.ptr,
+                        Cm.ptr, D ? static_cast<const float *>(D->ptr) : nullptr, y.data(), stream));
+    return y;
+}
+
 }  // namespace ssd_hip

@@ -1,5 +1,5 @@
 // C++ host-side check of libssd_hip through include/ssd_hip.hpp: the calls a compiled host program makes
-// (forward, streaming continuation, error paths), each checked against the plain-C oracle
+// (forward, streaming continuation step by step and as one call, error paths), each checked against the plain-C oracle
 // (oracle/ssd_oracle.c, linked from oracle/libssd_oracle.so).  Run by tests/test_gpu_host_cpp.py on the GPU.
 #include <cmath>
 #include <cstdio>
@@ -168,6 +168,42 @@ void forward_case(const Problem &p, const char *name) {
     const double wst = worst(std::vector<double>(st.begin(), st.end()), fin, tol, false);
     std::snprintf(what, sizeof(what), "%s: prefix + %d steps == full scan: y %.3f, state %.3f of the allowance", name, (int)tail, ws, wst);
     expect(ws <= 1.0 && wst <= 1.0, what);
+
+    // the same continuation as one call over a longer tail (bf16 runs of 16 steps or more go to the scan kernel)
+    {
+        const int64_t tail2 = 24, pre2 = p.L - tail2;
+        std::vector<double> qx(p.B * pre2 * p.H * p.P), qdt(p.B * pre2 * p.H), qB(p.B * pre2 * p.G * p.N), qC(qB.size());
+        std::vector<double> tx(p.B * tail2 * p.H * p.P), tdt(p.B * tail2 * p.H), tB(p.B * tail2 * p.G * p.N), tC(tB.size()),
+            ty(tx.size());
+        for (int64_t b = 0; b < p.B; ++b) {
+            std::copy_n(&p.x[b * p.L * p.H * p.P], pre2 * p.H * p.P, &qx[b * pre2 * p.H * p.P]);
+            std::copy_n(&p.dt[b * p.L * p.H], pre2 * p.H, &qdt[b * pre2 * p.H]);
+            std::copy_n(&p.Bm[b * p.L * p.G * p.N], pre2 * p.G * p.N, &qB[b * pre2 * p.G * p.N]);
+            std::copy_n(&p.Cm[b * p.L * p.G * p.N], pre2 * p.G * p.N, &qC[b * pre2 * p.G * p.N]);
+            std::copy_n(&p.x[(b * p.L + pre2) * p.H * p.P], tail2 * p.H * p.P, &tx[b * tail2 * p.H * p.P]);
+            std::copy_n(&p.dt[(b * p.L + pre2) * p.H], tail2 * p.H, &tdt[b * tail2 * p.H]);
+            std::copy_n(&p.Bm[(b * p.L + pre2) * p.G * p.N], tail2 * p.G * p.N, &tB[b * tail2 * p.G * p.N]);
+            std::copy_n(&p.Cm[(b * p.L + pre2) * p.G * p.N], tail2 * p.G * p.N, &tC[b * tail2 * p.G * p.N]);
+            std::copy_n(&y[(b * p.L + pre2) * p.H * p.P], tail2 * p.H * p.P, &ty[b * tail2 * p.H * p.P]);
+        }
+        DeviceBuffer dqx = upload(qx, p.bf16), dqdt = upload(qdt, p.bf16), dqB = upload(qB, p.bf16), dqC = upload(qC, p.bf16);
+        ScanOutput head = ssd_chunk_scan(view(dqx.data(), t, {p.B, pre2, p.H, p.P}), view(dqdt.data(), t, {p.B, pre2, p.H}), vA,
+                                         view(dqB.data(), t, {p.B, pre2, p.G, p.N}), view(dqC.data(), t, {p.B, pre2, p.G, p.N}),
+                                         &vD, p.chunk, nullptr);
+        StreamState many(p.B, p.H, p.P, p.N);
+        many.adopt(head.final_states);
+        DeviceBuffer dtx = upload(tx, p.bf16), dtdt = upload(tdt, p.bf16), dtB = upload(tB, p.bf16), dtC = upload(tC, p.bf16);
+        DeviceBuffer ym = ssd_steps(many, view(dtx.data(), t, {p.B, tail2, p.H, p.P}), view(dtdt.data(), t, {p.B, tail2, p.H}), vA,
+                                    view(dtB.data(), t, {p.B, tail2, p.G, p.N}), view(dtC.data(), t, {p.B, tail2, p.G, p.N}), &vD);
+        check_hip(hipDeviceSynchronize(), "sync");
+        const double wm = worst(download(ym, ty.size(), p.bf16), ty, tol, p.bf16);
+        std::vector<float> sm(fin.size());
+        check_hip(hipMemcpy(sm.data(), many.data(), sm.size() * 4, hipMemcpyDeviceToHost), "state");
+        const double wms = worst(std::vector<double>(sm.begin(), sm.end()), fin, tol, false);
+        std::snprintf(what, sizeof(what), "%s: prefix + %d steps in one call == full scan: y %.3f, state %.3f of the allowance",
+                      name, (int)tail2, wm, wms);
+        expect(wm <= 1.0 && wms <= 1.0, what);
+    }
 
     // a reset stream row starts from the empty state again
     state.reset_row(1);
