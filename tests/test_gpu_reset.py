@@ -102,3 +102,25 @@ def test_large_batch_and_prepared_call_take_the_mask():
     assert_close(f1[:3], fr, torch.bfloat16, "large batch reset final")
     with pytest.raises(ValueError):
         ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=128, reset=m[:, :-1])
+
+
+@pytest.mark.parametrize("batch,seqlen,dtype", [(4, 300, "f32"), (4, 300, "bf16"), (128, 256, "bf16"), (48, 2048, "bf16")])
+def test_a_restart_before_the_first_step_never_reads_the_initial_state(batch, seqlen, dtype):
+    """Whatever a restarted row's initial state holds (NaN here) must not reach y, the final state or the other
+    rows: staged kernels (separate and combined state passes), the one-pass kernel, the one-pass kernel on
+    segments.  The result equals the one with that row's initial state zero, bit for bit."""
+    w = Workload("fresh", batch, seqlen, 8, 32, 64, 1, 128, dtype=dtype, init_std=0.5)
+    dev = make_inputs(w, seed=21, device="cuda")
+    m = torch.zeros((batch, seqlen), dtype=torch.uint8, device="cuda")
+    m[1, 0] = 1
+    m[2, 5] = 1
+    zero = dev["init"].clone()
+    zero[1] = 0
+    bad = dev["init"].clone()
+    bad[1] = float("nan")
+    ops = [ssd_chunk_scan] + ([ssd_chunk_scan_onepass] if dtype == "bf16" else [])
+    for op in ops:
+        y0, f0 = op(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk, initial_states=zero, reset=m)
+        y1, f1 = op(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk, initial_states=bad, reset=m)
+        assert not torch.isnan(y1.float()).any() and not torch.isnan(f1).any(), op.__name__
+        assert torch.equal(y0, y1) and torch.equal(f0, f1), op.__name__

@@ -126,14 +126,16 @@ int run_staged(const ssd::ScanShape &s, int dtype, const void *x, const void *dt
                float *final_states, float *dtcs, float *states, hipStream_t st, int dt_len = 0) {
     hipError_t e = ssd::launch_chunk_cumsum(s, dtype, dt, A, reset, dtcs, st, mode, dt_len);
     if (e != hipSuccess) return hip_fail(e, "chunk_cumsum launch");
+    ssd::ScanShape sp = s;  // for the kernels that read the initial state
+    if (mode == 0) sp.fresh = reset;
     if ((int64_t)s.B * s.H >= kFusedStatePassingMinSequences) {
         // enough (b,h) sequences to fill the chip: stages 2 and 3 in one pass, states carried on chip
-        e = ssd::launch_chunk_state_scan(s, dtype, x, Bm, dtcs, initial_states, states, final_states, st);
+        e = ssd::launch_chunk_state_scan(sp, dtype, x, Bm, dtcs, initial_states, states, final_states, st);
         if (e != hipSuccess) return hip_fail(e, "chunk_state_passing launch");
     } else {
         e = ssd::launch_chunk_state(s, dtype, x, Bm, dtcs, states, st);
         if (e != hipSuccess) return hip_fail(e, "chunk_state launch");
-        e = ssd::launch_state_passing(s, states, dtcs, initial_states, states, final_states, st);  // in place
+        e = ssd::launch_state_passing(sp, states, dtcs, initial_states, states, final_states, st);  // in place
         if (e != hipSuccess) return hip_fail(e, "state_passing launch");
     }
     e = ssd::launch_chunk_scan(s, dtype, x, Bm, Cm, dtcs, states, D, y, st);

@@ -189,7 +189,7 @@ __global__ __launch_bounds__(64 * PB * ((NK + 1) / 2)) void chunk_state_kernel(
             if (t.c == 0) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-                if (init) {
+                if (init && !(s.fresh != nullptr && s.fresh[(size_t)t.b * s.L] != 0)) {  // (not after a restart at step 0)
                     const float *ib = init + ((size_t)t.b * s.H + t.h) * s.P * N + blk;
                     for_rows([&](int v, int o) { acc[v] = ib[o]; });
                 }

@@ -16,15 +16,17 @@ constexpr int kSegmentTargetGroups = 192;  // workgroups to aim for (256 CUs; th
 
 // enter[b,0] = init (or zero); enter[b,s+1] = decay[b,s] * enter[b,s] + local[b,s], written over local in place
 __global__ __launch_bounds__(256) void segment_states_kernel(float *states, const float *__restrict__ decay,
-                                                             const float *__restrict__ init, int S, int H, int pn4,
-                                                             long long total) {
+                                                             const float *__restrict__ init,
+                                                             const unsigned char *__restrict__ reset, int L, int S, int H,
+                                                             int pn4, long long total) {
     const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= total) return;
     const int idx = (int)(gid % pn4);
     const long long bh = gid / pn4;
     const int h = (int)(bh % H);
     const long long b = bh / H;
-    float4 cur = init ? reinterpret_cast<const float4 *>(init)[bh * pn4 + idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    const bool fresh = reset != nullptr && reset[b * L] != 0;  // restarts before its first step: init is not read
+    float4 cur = init && !fresh ? reinterpret_cast<const float4 *>(init)[bh * pn4 + idx] : make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s = 0; s < S; ++s) {
         float4 *slot = reinterpret_cast<float4 *>(states) + ((b * S + s) * H + h) * (long long)pn4 + idx;
         const float4 loc = *slot;
@@ -111,8 +113,8 @@ hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segmen
     if (e != hipSuccess) return e;
     const int pn4 = s.P * s.N / 4;
     const long long total = (long long)s.B * s.H * pn4;
-    segment_states_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(seg_states, seg_decay, init, segments, s.H,
-                                                                                     pn4, total);
+    segment_states_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(seg_states, seg_decay, init, reset, s.L, segments,
+                                                                                     s.H, pn4, total);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     ScanShape f = s;

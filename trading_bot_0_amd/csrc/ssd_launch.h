@@ -20,6 +20,9 @@ struct ScanShape {
     // The one-pass kernel only: the sequence cut into segments of seg_tiles tiles of 64 steps (0 = not cut) that
     // different workgroups walk; initial states are then given per segment, [B, segments, H, P, N].
     int seg_tiles = 0;
+    // The staged kernels that read the initial state only: the restart mask [B, L] (or NULL).  A sequence that
+    // restarts before its first step does not read its initial state at all, whatever that holds.
+    const unsigned char *fresh = nullptr;
 };
 
 struct StepShape {

@@ -109,7 +109,8 @@ __global__ __launch_bounds__(256) void state_passing_kernel(const float *states,
     float4 *dst = reinterpret_cast<float4 *>(prev) + ((size_t)b * s.nc * s.H + h) * pn4 + idx;
     const float *a_end = dtcs + ((size_t)bh * s.nc) * 4 * s.Q + (s.Q - 1);  // alpha_hi at the chunk end
     const size_t a_stride = (size_t)4 * s.Q;
-    float4 st = init ? reinterpret_cast<const float4 *>(init)[(size_t)bh * pn4 + idx] : make_float4(0, 0, 0, 0);
+    const bool fresh = s.fresh != nullptr && s.fresh[(size_t)b * s.L] != 0;  // restarts before its first step
+    float4 st = init && !fresh ? reinterpret_cast<const float4 *>(init)[(size_t)bh * pn4 + idx] : make_float4(0, 0, 0, 0);
     int c = 0;
     for (; c + kPassUnroll <= s.nc; c += kPassUnroll) {
         float4 sv[kPassUnroll];
