@@ -213,6 +213,10 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
  * scan's float32 y as the input of post); parameters are float32. */
 typedef struct {
     int64_t batch, seqlen, nheads, headdim, dstate, ngroups, d_conv;
+    /* elements from one timestep's row of zxbcdt to the next: 0 = E (dense), else at least E and a whole number of
+     * 16-byte pieces.  Rows a multiple of 128 bytes apart (704 for E = 648 in bf16) keep every row's lines of the
+     * memory system whole, which the in-projection's stores gain most from. */
+    int64_t zxbcdt_ld;
 } ssd_block_dims;
 
 /* x [B,L,H,P], Bm, Cm [B,L,G,N] = silu(causal depthwise conv1d of width d_conv (2..4) over the x | B | C
@@ -230,9 +234,10 @@ int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt,
  * trading_bots/src/torch/model/blocks/gqa.rs:82-109): out [rows, out_features] = u [rows, in_features] .
  * w [out_features, in_features]^T, bfloat16 in and out (dtype 1), float32 accumulation; rows = batch * seqlen.
  * in_features must be 128 or 256 and out_features a multiple of 8 (SSD_ERR_UNSUPPORTED otherwise: use the
- * caller's BLAS).  No bias. */
-int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, int dtype, const void *u, const void *w,
-                       void *out, void *hip_stream);
+ * caller's BLAS).  out_ld = elements from one row of out to the next (0 = out_features; else at least that and a
+ * multiple of 8): the padding columns are not written.  No bias. */
+int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, int64_t out_ld, int dtype, const void *u,
+                       const void *w, void *out, void *hip_stream);
 
 /* out [B,L,H*P] = rmsnorm(y * silu(z)) * norm_w over the H*P channels of a timestep (z from zxbcdt). */
 int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,

@@ -101,6 +101,60 @@ def test_projection_against_float64(rows, k, n):
     assert np.isfinite(o).all() and not bad.any(), f"{int(bad.sum())} elements off"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 8, 32, 64, 1, 4), (3, 7, 8, 16, 16, 2, 3), (4, 1, 8, 32, 64, 1, 4)])
+def test_stages_take_padded_rows(shape, dtype):
+    """zxbcdt as the first E columns of a buffer with longer rows (what the in-projection writes when asked for rows
+    of whole 128-byte lines): pre and post give the dense tensor's results bit for bit, whatever the padding holds."""
+    Bsz, L, H, P, N, G, K = shape
+    p = params(H, P, N, G, K)
+    E = 2 * H * P + 2 * G * N + H
+    g = torch.Generator().manual_seed(5)
+    z = torch.randn(Bsz, L, E, generator=g).to(dtype).cuda()
+    buf = torch.full((Bsz, L, (E + 63) // 64 * 64 + 64), float("nan"), dtype=dtype, device="cuda")
+    buf[..., :E] = z
+    zp = buf[..., :E]
+    assert not zp.is_contiguous() or L * Bsz == 1
+    st = (torch.randn(Bsz, K - 1, H * P + 2 * G * N, generator=g)).to(dtype).cuda()
+    dense = block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=st, return_conv_state=True)
+    padded = block_pre(zp, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=st, return_conv_state=True)
+    assert all(torch.equal(a, b) for a, b in zip(dense, padded))
+    y = (torch.randn(Bsz, L, H, P, generator=g) * 3).to(dtype).cuda()
+    assert torch.equal(block_post(y, z, p["norm_w"], H, P, N, G), block_post(y, zp, p["norm_w"], H, P, N, G))
+    with pytest.raises(ValueError):       # a view that does not start on a 16-byte piece
+        block_pre(buf[:, :, 1:E + 1], p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G)
+    with pytest.raises(ValueError):       # elements of a row not adjacent
+        block_pre(buf[:, :, :2 * E:2], p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G)
+
+
+@pytest.mark.parametrize("rows,k,n", [(300, 256, 648), (4099, 256, 256), (2049, 128, 168), (33, 256, 8), (5000, 256, 768)])
+def test_projection_into_padded_rows(rows, k, n):
+    """pad_rows: the same numbers as the dense call, bit for bit, in rows a multiple of 64 elements apart; columns
+    past out_features are not written."""
+    g = torch.Generator().manual_seed(rows + n)
+    u = torch.randn(rows, k, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16).cuda()
+    dense = block_proj(u, w)
+    padded = block_proj(u, w, pad_rows=True)
+    assert padded.shape == (rows, n) and padded.stride(0) == (n + 63) // 64 * 64 and padded.stride(1) == 1
+    assert torch.equal(dense, padded)
+    # through the C ABI into a poisoned buffer: the padding stays as it was
+    from ctypes import c_void_p
+    from trading_bot_0_amd import ssd
+    from trading_bot_0_amd.block import _lib
+    ld = (n + 63) // 64 * 64 + 64
+    buf = torch.full((rows, ld), -7.0, dtype=torch.bfloat16, device="cuda")
+    lib = _lib()
+    ssd._check(lib, lib.ssd_block_proj_fwd(rows, k, n, ld, ssd.SSD_DTYPE_BF16, u.data_ptr(), w.data_ptr(), buf.data_ptr(),
+                                           ssd._stream_ptr(u)))
+    torch.cuda.synchronize()
+    assert torch.equal(buf[:, :n], dense) and bool((buf[:, n:] == -7.0).all())
+    for bad_ld in ((n - 8, n + 4) if n > 8 else (n + 4, n + 9)):   # (0 would mean dense)
+        with pytest.raises(SsdError):
+            ssd._check(lib, lib.ssd_block_proj_fwd(rows, k, n, bad_ld, ssd.SSD_DTYPE_BF16, u.data_ptr(), w.data_ptr(),
+                                                   buf.data_ptr(), ssd._stream_ptr(u)))
+
+
 def test_projection_keeps_leading_dimensions_and_refuses_other_shapes():
     u = torch.randn(3, 50, 256).to(torch.bfloat16).cuda()
     w = torch.randn(40, 256).to(torch.bfloat16).cuda()

@@ -21,7 +21,7 @@ from .stream_state import SsdStreamState
 
 
 class SsdBlockDims(Structure):
-    _fields_ = [(n, c_int64) for n in ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "d_conv")]
+    _fields_ = [(n, c_int64) for n in ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "d_conv", "zxbcdt_ld")]
 
 
 _bound = False
@@ -34,7 +34,7 @@ def _lib():
         P = c_void_p
         lib.ssd_block_pre_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_block_post_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, P]
-        lib.ssd_block_proj_fwd.argtypes = [c_int64, c_int64, c_int64, c_int, P, P, P, P]
+        lib.ssd_block_proj_fwd.argtypes = [c_int64, c_int64, c_int64, c_int64, c_int, P, P, P, P]
         lib.ssd_block_pre_fwd.restype = c_int
         lib.ssd_block_post_fwd.restype = c_int
         lib.ssd_block_proj_fwd.restype = c_int
@@ -46,9 +46,24 @@ def in_proj_width(nheads, headdim, dstate, ngroups) -> int:
     return 2 * nheads * headdim + 2 * ngroups * dstate + nheads
 
 
+def _row_stride(zxbcdt) -> int:
+    """The row stride of zxbcdt [B,L,E]: dense, or the first E columns of a buffer with padded rows (what
+    `block_proj(..., pad_rows=True)` returns)."""
+    Bsz, L, E = zxbcdt.shape
+    ld = zxbcdt.stride(1) if L > 1 else (zxbcdt.stride(0) if Bsz > 1 else E)
+    if zxbcdt.is_contiguous():
+        return E
+    if zxbcdt.stride(2) != 1 or ld < E or (L > 1 and Bsz > 1 and zxbcdt.stride(0) != L * ld):
+        raise ValueError(f"zxbcdt must be contiguous or have evenly padded rows, got strides {zxbcdt.stride()}")
+    if zxbcdt.data_ptr() % 16:
+        raise ValueError("zxbcdt must be 16-byte aligned")
+    return ld
+
+
 def block_pre(zxbcdt, conv_w, conv_b, dt_bias, nheads, headdim, dstate, ngroups, conv_state=None,
               return_conv_state=False):
-    """zxbcdt [B,L,E] -> (x [B,L,H,P], Bm, Cm [B,L,G,N], dt [B,L,H][, conv state [B,d_conv-1,C]])."""
+    """zxbcdt [B,L,E] (rows dense or evenly padded) -> (x [B,L,H,P], Bm, Cm [B,L,G,N], dt [B,L,H][, conv state
+    [B,d_conv-1,C]])."""
     lib = _lib()
     if zxbcdt.dim() != 3:
         raise ValueError(f"block input must be rank-3 [batch, seqlen, channels], got {tuple(zxbcdt.shape)}")
@@ -59,7 +74,9 @@ def block_pre(zxbcdt, conv_w, conv_b, dt_bias, nheads, headdim, dstate, ngroups,
         raise ValueError(f"block input must have {in_proj_width(H, P, N, G)} channels, got {E}")
     dtype = zxbcdt.dtype
     code = ssd._dtype_code(zxbcdt)
-    ssd._require(zxbcdt, "zxbcdt", (Bsz, L, E), dtype)
+    if not zxbcdt.is_cuda:
+        raise ValueError("zxbcdt must be a GPU tensor")
+    ld = _row_stride(zxbcdt)
     if conv_w.dim() != 2 or conv_w.shape[0] != C:
         raise ValueError(f"conv_w must be [{C}, d_conv], got {tuple(conv_w.shape)}")
     d_conv = conv_w.shape[1]
@@ -74,7 +91,7 @@ def block_pre(zxbcdt, conv_w, conv_b, dt_bias, nheads, headdim, dstate, ngroups,
     Cm = torch.empty((Bsz, L, G, N), dtype=dtype, device=dev)
     dt = torch.empty((Bsz, L, H), dtype=dtype, device=dev)
     new_state = torch.empty((Bsz, d_conv - 1, C), dtype=dtype, device=dev) if return_conv_state else None
-    dims = SsdBlockDims(Bsz, L, H, P, N, G, d_conv)
+    dims = SsdBlockDims(Bsz, L, H, P, N, G, d_conv, ld)
     ssd._check(lib, lib.ssd_block_pre_fwd(byref(dims), code, zxbcdt.data_ptr(), conv_w.data_ptr(), conv_b.data_ptr(),
                                           dt_bias.data_ptr(), ssd._ptr(conv_state), ssd._ptr(new_state), x.data_ptr(),
                                           Bm.data_ptr(), Cm.data_ptr(), dt.data_ptr(), ssd._stream_ptr(zxbcdt)))
@@ -92,11 +109,13 @@ def block_post(y, zxbcdt, norm_w, nheads, headdim, dstate, ngroups, eps=1e-5):
         if not (dtype == torch.bfloat16 and y.dtype == torch.float32):
             raise ValueError(f"block y must be {dtype} (or float32 with bf16 activations), got {y.dtype}")
         code = ssd.SSD_DTYPE_BF16_Y32
-    ssd._require(zxbcdt, "zxbcdt", (Bsz, L, in_proj_width(H, P, N, G)), dtype)
+    if not zxbcdt.is_cuda or E != in_proj_width(H, P, N, G):
+        raise ValueError(f"zxbcdt must be a GPU tensor with {in_proj_width(H, P, N, G)} channels, got {tuple(zxbcdt.shape)}")
+    ld = _row_stride(zxbcdt)
     ssd._require(y, "y", (Bsz, L, H, P), y.dtype)
     ssd._require(norm_w, "norm_w", (H * P,), torch.float32)
     out = torch.empty((Bsz, L, H * P), dtype=dtype, device=zxbcdt.device)
-    dims = SsdBlockDims(Bsz, L, H, P, N, G, 4)
+    dims = SsdBlockDims(Bsz, L, H, P, N, G, 4, ld)
     ssd._check(lib, lib.ssd_block_post_fwd(byref(dims), code, y.data_ptr(), zxbcdt.data_ptr(), norm_w.data_ptr(),
                                            c_float(eps), out.data_ptr(), ssd._stream_ptr(zxbcdt)))
     return out
@@ -108,9 +127,11 @@ def block_proj_supported(u: torch.Tensor, weight: torch.Tensor) -> bool:
             and weight.shape[0] % 8 == 0 and u.numel() > 0)
 
 
-def block_proj(u: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def block_proj(u: torch.Tensor, weight: torch.Tensor, pad_rows: bool = False) -> torch.Tensor:
     """u [..., in_features] (bf16) times weight [out_features, in_features]^T -> [..., out_features] (bf16), float32
-    accumulation: the block's in- and out-projection as one memory-bound kernel."""
+    accumulation: the block's in- and out-projection as one memory-bound kernel.  With pad_rows the result is the
+    first out_features columns of a buffer whose rows are a multiple of 128 bytes apart (a non-contiguous view that
+    `block_pre` and `block_post` take): every line the kernel writes is then a whole one."""
     lib = _lib()
     if u.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise ValueError(f"block_proj takes bfloat16 tensors, got {u.dtype} and {weight.dtype}")
@@ -119,10 +140,12 @@ def block_proj(u: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     if not u.is_contiguous() or not weight.is_contiguous():
         raise ValueError("block_proj takes contiguous tensors")
     rows = u.numel() // u.shape[-1]
-    out = torch.empty(u.shape[:-1] + (weight.shape[0],), dtype=torch.bfloat16, device=u.device)
-    ssd._check(lib, lib.ssd_block_proj_fwd(rows, u.shape[-1], weight.shape[0], ssd.SSD_DTYPE_BF16, u.data_ptr(),
+    width = weight.shape[0]
+    ld = (width + 63) // 64 * 64 if pad_rows else width
+    out = torch.empty(u.shape[:-1] + (ld,), dtype=torch.bfloat16, device=u.device)
+    ssd._check(lib, lib.ssd_block_proj_fwd(rows, u.shape[-1], width, ld, ssd.SSD_DTYPE_BF16, u.data_ptr(),
                                            weight.data_ptr(), out.data_ptr(), ssd._stream_ptr(u)))
-    return out
+    return out[..., :width] if ld != width else out
 
 
 @dataclass
@@ -188,7 +211,7 @@ class Mamba2Block:
             raise ValueError(f"block input must be [batch, seqlen, {self.d_model}], got {tuple(u.shape)}")
         if reset is not None and state is not None:
             raise ValueError("restarts inside the window and a carried conv state cannot be combined")
-        zxbcdt = self._project(u, self.in_proj)
+        zxbcdt = self._project(u, self.in_proj, pad_rows=True)  # internal to the block: rows of whole lines
         if state is None:
             x, Bm, Cm, dt = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G)
             y, _ = ssd.ssd_chunk_scan(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk, return_final_states=False,
@@ -201,13 +224,13 @@ class Mamba2Block:
         yn = block_post(y, zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
         return self._project(yn, self.out_proj)
 
-    def _project(self, u: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    def _project(self, u: torch.Tensor, weight: torch.Tensor, pad_rows: bool = False) -> torch.Tensor:
         """u . weight^T in the activation dtype: the library's kernel where it takes the shape (bf16, in_features 128
         or 256, a tall u), else the BLAS behind torch."""
         w = weight.to(u.dtype)
         u = u.contiguous()
         if block_proj_supported(u, w) and u.numel() // u.shape[-1] >= 16384:
-            return block_proj(u, w.contiguous())
+            return block_proj(u, w.contiguous(), pad_rows=pad_rows)
         return torch.matmul(u, w.t()).contiguous()
 
     def step(self, u_t: torch.Tensor, state: Mamba2StreamState) -> torch.Tensor:

@@ -702,13 +702,18 @@ static int make_block_shape(const ssd_block_dims *d, int dtype, ssd::BlockShape 
                     (long long)d->seqlen);
     if (int rc = check_state_dims(d->nheads, d->headdim, d->dstate, d->ngroups)) return rc;
     const int64_t E = 2 * d->nheads * d->headdim + 2 * d->ngroups * d->dstate + d->nheads;
-    if (d->batch * d->seqlen > 0x7fffffff || d->batch * d->seqlen * E / 8 > 0x7fffffffffLL)
+    if (d->batch * d->seqlen > 0x7fffffff || d->zxbcdt_ld > 0x7fffffff ||
+        d->batch * d->seqlen * (d->zxbcdt_ld > E ? d->zxbcdt_ld : E) / 8 > 0x7fffffffffLL)
         return fail(SSD_ERR_UNSUPPORTED, "ssd: batch*seqlen exceeds 2^31-1");
     if (E % (dtype == SSD_DTYPE_F32 ? 4 : 8) != 0)
         return fail(SSD_ERR_UNSUPPORTED, "ssd: the %lld channels of a timestep must be a whole number of 16-byte "
                                          "pieces (nheads a multiple of %d)", (long long)E, dtype == SSD_DTYPE_F32 ? 4 : 8);
+    const int64_t ld = d->zxbcdt_ld == 0 ? E : d->zxbcdt_ld;
+    if (ld < E || ld > 0x7fffffff || ld % (dtype == SSD_DTYPE_F32 ? 4 : 8) != 0)
+        return fail(SSD_ERR_INVALID, "ssd: zxbcdt_ld must be 0 or at least the %lld channels of a timestep and a whole "
+                                     "number of 16-byte pieces, got %lld", (long long)E, (long long)d->zxbcdt_ld);
     ssd::BlockShape s{(int)d->batch, (int)d->seqlen, (int)d->nheads, (int)d->headdim, (int)d->dstate,
-                      (int)d->ngroups, (int)d->d_conv};
+                      (int)d->ngroups, (int)d->d_conv, (int)ld};
     if (!ssd::block_supported(s))
         return fail(SSD_ERR_UNSUPPORTED, "ssd: block stages need d_conv 2..4 (got %lld) and nheads*headdim <= 2048",
                     (long long)d->d_conv);
@@ -738,8 +743,8 @@ int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt,
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block pre-scan launch");
 }
 
-int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, int dtype, const void *u, const void *w,
-                       void *out, void *hip_stream) {
+int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, int64_t out_ld, int dtype, const void *u,
+                       const void *w, void *out, void *hip_stream) {
     if (dtype != SSD_DTYPE_BF16)
         return fail(SSD_ERR_UNSUPPORTED, "ssd: the block projection takes dtype 1 (bfloat16), got %d", dtype);
     if (rows <= 0 || in_features <= 0 || out_features <= 0)
@@ -751,10 +756,15 @@ int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, 
                     "ssd: the block projection needs in_features 128 or 256 and out_features a multiple of 8, got "
                     "%lld and %lld",
                     (long long)in_features, (long long)out_features);
+    if (out_ld == 0) out_ld = out_features;
+    if (out_ld < out_features || out_ld > 0x7fffffff || out_ld % 8 != 0)
+        return fail(SSD_ERR_INVALID, "ssd: out_ld must be 0 or at least out_features (%lld) and a multiple of 8, got %lld",
+                    (long long)out_features, (long long)out_ld);
     REQUIRE_PTR(u);
     REQUIRE_PTR(w);
     REQUIRE_PTR(out);
-    hipError_t e = ssd::launch_block_proj(rows, (int)in_features, (int)out_features, u, w, out, (hipStream_t)hip_stream);
+    hipError_t e = ssd::launch_block_proj(rows, (int)in_features, (int)out_features, (int)out_ld, u, w, out,
+                                          (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block projection launch");
 }
 

@@ -4,7 +4,8 @@
 //   post  gated RMSNorm: out = rmsnorm(y * silu(z)) * weight
 // The projections on either side are plain GEMMs and stay with the caller's BLAS.
 //
-// Input layout (per timestep, E = 2*H*P + 2*G*N + H channels): [ z | x | B | C | dt_raw ].
+// Input layout (per timestep, E = 2*H*P + 2*G*N + H channels): [ z | x | B | C | dt_raw ], rows s.ld elements
+// apart (ld >= E: a padded row keeps every row's 128-byte lines whole).
 #include "ssd_device.h"
 
 namespace ssd {
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
                                                         const T *__restrict__ state_in, T *__restrict__ state_out,
                                                         T *__restrict__ x, T *__restrict__ Bm, T *__restrict__ Cm,
                                                         T *__restrict__ dt, BlockShape s) {
-    const int DI = s.H * s.P, GN = s.G * s.N, C = DI + 2 * GN, E = 2 * DI + 2 * GN + s.H;
+    const int DI = s.H * s.P, GN = s.G * s.N, C = DI + 2 * GN;
     const int CP = C / 8, HP8 = (s.H + 7) / 8;
     const int runs = (s.L + kPreSteps - 1) / kPreSteps;
     const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
         if (d >= (long long)s.B * s.L * HP8) return;
         const int h0 = (int)(d % HP8) * 8;
         const long long bt = d / HP8;
-        const T *src = zxbcdt + (size_t)bt * E + 2 * DI + 2 * GN;
+        const T *src = zxbcdt + (size_t)bt * s.ld + 2 * DI + 2 * GN;
         if (s.H % 8 == 0) {  // eight heads are one aligned 16-byte (bf16) piece on both sides
             const Pack8<T> v = Pack8<T>::load(src + h0);
             float o[8];
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
     const long long br = gid / CP;
     const int t0 = (int)(br % runs) * kPreSteps, b = (int)(br / runs);
     const int t1 = min(t0 + kPreSteps, s.L);
-    const T *row0 = zxbcdt + ((size_t)b * s.L) * E;  // this batch row's first timestep
+    const T *row0 = zxbcdt + ((size_t)b * s.L) * s.ld;  // this batch row's first timestep
     const int c0 = piece * 8;  // channel within [x | B | C]
     float w[8][DCONV], bias[8];
     {   // the taps of 8 consecutive channels are 8*DCONV consecutive floats
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
 #pragma unroll
         for (int i = 0; i < 8; ++i) win[k][i] = 0.f;
         if (ts >= 0) {
-            const Pack8<T> v = Pack8<T>::load(row0 + (size_t)ts * E + DI + c0);
+            const Pack8<T> v = Pack8<T>::load(row0 + (size_t)ts * s.ld + DI + c0);
 #pragma unroll
             for (int i = 0; i < 8; ++i) win[k][i] = v.get(i);
         } else if (state_in != nullptr) {
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
     Pack8<T> in[kPreSteps];
 #pragma unroll
     for (int j = 0; j < kPreSteps; ++j)
-        if (t0 + j < t1) in[j] = Pack8<T>::load(row0 + (size_t)(t0 + j) * E + DI + c0);
+        if (t0 + j < t1) in[j] = Pack8<T>::load(row0 + (size_t)(t0 + j) * s.ld + DI + c0);
 #pragma unroll
     for (int j = 0; j < kPreSteps; ++j) {
         const int t = t0 + j;
@@ -182,12 +183,12 @@ template <typename T, typename TY, int LPR>
 __global__ __launch_bounds__(256) void block_post_kernel(const TY *__restrict__ y, const T *__restrict__ zxbcdt,
                                                          const float *__restrict__ norm_w, float eps,
                                                          T *__restrict__ out, BlockShape s) {
-    const int DI = s.H * s.P, E = 2 * DI + 2 * s.G * s.N + s.H;
+    const int DI = s.H * s.P;
     const int lane = threadIdx.x & (LPR - 1);
     const long long row = ((long long)blockIdx.x * blockDim.x + threadIdx.x) / LPR;
     const bool live = row < (long long)s.B * s.L;  // (whole waves stay for the lane exchanges)
     const TY *yr = y + (size_t)(live ? row : 0) * DI;
-    const T *zr = zxbcdt + (size_t)(live ? row : 0) * E;
+    const T *zr = zxbcdt + (size_t)(live ? row : 0) * s.ld;
     constexpr int MAXP = 4;  // pieces of 8 channels per lane kept in registers: 64 lanes cover H*P <= 2048
     float v[MAXP][8];
     float ss = 0.f;

@@ -26,7 +26,7 @@ template <int KS>  // K = 16 * KS
 __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf16 *__restrict__ u,
                                                                       const __bf16 *__restrict__ w,
                                                                       __bf16 *__restrict__ out, long long M, int N,
-                                                                      int col_blocks, int block_cols) {
+                                                                      int ldo, int col_blocks, int block_cols) {
     constexpr int K = 16 * KS, NTHR = 64 * kProjWaves;
     constexpr int ROWB = K * 2 + 16;        // bytes of a staged row of w: 16 bytes of padding shift the banks
     constexpr int kTileRowB = 64 * 2 + 16;  // a row of a wave's output tile: 64 columns and 16 bytes of padding
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
     const int cb = within % col_blocks;
     const long long rg = (long long)(within / col_blocks) * 8 + xcd;
     const int n0 = cb * block_cols;                 // this workgroup's first column
-    const int ncols = min(block_cols, N - n0);      // a multiple of 8
+    const int ncols = cb == col_blocks - 1 ? N - n0 : block_cols;  // a multiple of 8; the last block takes the rest
     const int chunks = (ncols + kProjChunk - 1) / kProjChunk;
     const long long row0 = rg * kProjTiles * (32LL * kProjWaves);
     if (row0 >= M) return;  // the grid is padded to whole rounds of XCDs
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
                 const int row = pass * 8 + (lane >> 3), col = c0 * kProjChunk + (lane & 7) * 8;
                 const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kTileRowB + (lane & 7) * 16);
                 if (m0 + row < M && col < ncols)
-                    *reinterpret_cast<uint4 *>(out + (size_t)(m0 + row) * N + n0 + col) = v;
+                    *reinterpret_cast<uint4 *>(out + (size_t)(m0 + row) * ldo + n0 + col) = v;
             }
             asm volatile("" ::: "memory");
             __builtin_amdgcn_wave_barrier();
@@ -132,22 +132,40 @@ bool block_proj_supported(long long rows, int in_features, int out_features) {
     return rows > 0 && (in_features == 128 || in_features == 256) && out_features > 0 && out_features % 8 == 0;
 }
 
-hipError_t launch_block_proj(long long rows, int in_features, int out_features, const void *u, const void *w, void *out,
-                             hipStream_t st) {
-    if (!block_proj_supported(rows, in_features, out_features)) return hipErrorInvalidValue;
-    // column blocks of equal size (a multiple of 8 columns), at most kProjBlockCols
-    const int col_blocks = (out_features + kProjBlockCols - 1) / kProjBlockCols;
-    const int block_cols = ((out_features + col_blocks - 1) / col_blocks + 7) / 8 * 8;
+// Column blocks: equal blocks of at most kProjBlockCols columns (a multiple of 8) -- or, where that takes no more
+// workgroups, blocks of 128 with the last one taking the rest (up to kProjBlockCols): every block then starts on a
+// multiple of 64 columns, so that with rows a multiple of 128 bytes apart every 128-byte piece a wave writes is one
+// whole line of the memory system (648 columns: 4 x 128 + 136 instead of 4 x 136 + 104, 21 column chunks instead of 25).
+static void proj_col_blocks(int out_features, int *col_blocks, int *block_cols) {
+    const int equal = (out_features + kProjBlockCols - 1) / kProjBlockCols;
+    const int by128 = out_features <= kProjBlockCols ? 1 : (out_features - kProjBlockCols + 127) / 128 + 1;
+    if (by128 == equal) {
+        *col_blocks = by128;
+        *block_cols = by128 == 1 ? (out_features + 7) / 8 * 8 : 128;
+    } else {
+        *col_blocks = equal;
+        *block_cols = ((out_features + equal - 1) / equal + 7) / 8 * 8;
+    }
+}
+
+hipError_t launch_block_proj(long long rows, int in_features, int out_features, int out_ld, const void *u, const void *w,
+                             void *out, hipStream_t st) {
+    if (!block_proj_supported(rows, in_features, out_features) || out_ld < out_features || out_ld % 8 != 0)
+        return hipErrorInvalidValue;
+    int col_blocks, block_cols;
+    proj_col_blocks(out_features, &col_blocks, &block_cols);
     const long long rows_per_group = 32LL * kProjWaves * kProjTiles;
     const long long groups = ((rows + rows_per_group - 1) / rows_per_group + 7) / 8 * 8 * col_blocks;
-    if (groups > 0x7fffffffLL || block_cols > kProjBlockCols) return hipErrorInvalidValue;
+    if (groups > 0x7fffffffLL || out_features - (col_blocks - 1) * block_cols > kProjBlockCols ||
+        out_features - (col_blocks - 1) * block_cols <= 0)
+        return hipErrorInvalidValue;
     const dim3 grid((unsigned)groups), block(64 * kProjWaves);
     const __bf16 *uu = static_cast<const __bf16 *>(u), *ww = static_cast<const __bf16 *>(w);
     __bf16 *oo = static_cast<__bf16 *>(out);
     if (in_features == 128)
-        block_proj_kernel<8><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, col_blocks, block_cols);
+        block_proj_kernel<8><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, out_ld, col_blocks, block_cols);
     else
-        block_proj_kernel<16><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, col_blocks, block_cols);
+        block_proj_kernel<16><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, out_ld, col_blocks, block_cols);
     return hipGetLastError();
 }
 

@@ -31,6 +31,7 @@ struct StepShape {
 
 struct BlockShape {  // a Mamba-2 block around the scan: conv width d_conv over the x | B | C channels
     int B, L, H, P, N, G, d_conv;
+    int ld;  // elements from one timestep's row of zxbcdt to the next (at least its channel count)
 };
 
 constexpr size_t kLdsLimitBytes = 160 * 1024;  // LDS per workgroup on gfx950
@@ -105,8 +106,8 @@ bool block_supported(const BlockShape &s);
 // The block's projections in bf16: out [rows, out_features] = u [rows, in_features] . w [out_features, in_features]^T,
 // float32 accumulation.  in_features 128 or 256, out_features a multiple of 8.
 bool block_proj_supported(long long rows, int in_features, int out_features);
-hipError_t launch_block_proj(long long rows, int in_features, int out_features, const void *u, const void *w, void *out,
-                             hipStream_t stream);
+hipError_t launch_block_proj(long long rows, int in_features, int out_features, int out_ld, const void *u, const void *w,
+                             void *out, hipStream_t st);
 hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w,
                             const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
                             void *x, void *Bm, void *Cm, void *dt, hipStream_t stream);
