@@ -33,7 +33,9 @@ def draw(case):
     return w, mask, rows, bool(rng.random() < 0.5)
 
 
-@pytest.mark.parametrize("case", range(24))
+# (case 76: float32, a timestep that decays the state by 2^-64 inside a block of heavy-tailed x -- the shape on which
+# separable decay factors across such a block cost float mode 30 ulps on the largest outputs)
+@pytest.mark.parametrize("case", list(range(24)) + [76])
 def test_random_shape(case):
     w, mask, rows, with_dfinal = draw(case)
     cpu = make_inputs(w, seed=case)

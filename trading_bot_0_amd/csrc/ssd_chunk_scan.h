@@ -190,7 +190,12 @@ __global__ __launch_bounds__(64 * QB, (is_bf16<T> && PB == 1 && NK <= 4 && QB >=
         const float El = exp2_hw(fminf(alpha_diff(al_hi, al_lo, rf_hi, rf_lo), 0.f));
         // non-negative floats order like their bit patterns: a scalar compare
         const float span = fmaxf(alpha_diff(rf_hi, rf_lo, ah_s[32 * lb + 31], alo_s[32 * lb + 31]), 0.f);
-        const bool fast = __builtin_amdgcn_readfirstlane(__float_as_int(span)) <= __float_as_int(120.f);
+        // The separable factors E[l] F[s] are exp2 of two arguments as large as the span, each rounded to float: their
+        // product carries a relative error of about 2^-24 * span * ln 2, nothing next to bf16 operands (2^-17), but in
+        // float mode a span of 64 would cost 30 ulps on the largest outputs.  Float mode therefore separates only
+        // blocks that hardly decay; its MFMAs leave the VALU idle enough for the exact path's exp2 per element.
+        constexpr float kSeparableSpan = is_bf16<T> ? 120.f : 4.f;
+        const bool fast = __builtin_amdgcn_readfirstlane(__float_as_int(span)) <= __float_as_int(kSeparableSpan);
         f32x16 accY[PB];
         // state readout, brought to the column block's first row (alpha <= 0)
         {
