@@ -157,7 +157,8 @@ def oracle_steps(cpu, reset=None):
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("shape", [(5, 4, 16, 16, 1, 7), (3, 8, 32, 64, 1, 16), (2, 16, 64, 128, 2, 5),
                                    (6, 6, 32, 32, 3, 1), (4, 8, 16, 128, 1, 9),
-                                   (4, 8, 32, 64, 1, 150), (2, 16, 64, 128, 2, 70)])   # long runs: on the one-pass scan
+                                   (4, 8, 32, 64, 1, 150), (2, 16, 64, 128, 2, 70),    # long runs: on the one-pass scan
+                                   (33, 2, 32, 32, 1, 16), (2, 1, 64, 32, 1, 65)])     # long runs of two units: not on it
 def test_steps_in_one_launch_match_the_oracle(shape, dtype):
     from trading_bot_0_amd import ssd_steps
     Bsz, H, P, N, G, T = shape

@@ -679,7 +679,9 @@ int ssd_steps_fwd(const ssd_step_dims *dims, int64_t nsteps, int dtype, float *s
     if (nsteps >= kStepsAsScanMin && dtype != SSD_DTYPE_F32) {
         const ssd_dims d = {dims->batch, nsteps, dims->nheads, dims->headdim, dims->dstate, dims->ngroups, kBackwardChunk};
         ssd::ScanShape sc;
-        if (make_shape(&d, dtype, &sc) == SSD_OK && ssd::fused_scan_waves(sc, dtype) != 0) {
+        // (asked for the bf16-y instance whatever y's type is: the two output types must take the same path, so
+        // that the bf16 y stays the float32 y rounded once; one instance exists for float y only)
+        if (make_shape(&d, dtype, &sc) == SSD_OK && ssd::fused_scan_waves(sc, SSD_DTYPE_BF16) != 0) {
             hipError_t e = ssd::launch_fused_scan(sc, dtype, x, dt, A, Bm, Cm, D, state, reset, y, state,
                                                   (hipStream_t)hip_stream);
             return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch (steps)");
