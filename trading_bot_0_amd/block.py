@@ -51,12 +51,12 @@ def _row_stride(zxbcdt) -> int:
     `block_proj(..., pad_rows=True)` returns)."""
     Bsz, L, E = zxbcdt.shape
     ld = zxbcdt.stride(1) if L > 1 else (zxbcdt.stride(0) if Bsz > 1 else E)
+    if zxbcdt.data_ptr() % 16:
+        raise ValueError("zxbcdt must be 16-byte aligned")
     if zxbcdt.is_contiguous():
         return E
     if zxbcdt.stride(2) != 1 or ld < E or (L > 1 and Bsz > 1 and zxbcdt.stride(0) != L * ld):
         raise ValueError(f"zxbcdt must be contiguous or have evenly padded rows, got strides {zxbcdt.stride()}")
-    if zxbcdt.data_ptr() % 16:
-        raise ValueError("zxbcdt must be 16-byte aligned")
     return ld
 
 
