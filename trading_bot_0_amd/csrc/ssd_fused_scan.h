@@ -256,9 +256,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         return t;
     };
     // When the next tile's inputs are requested: after phase 1 (they are then in flight during phase 2 only, but
-    // hold no registers through phase 1), or, for the two-wave workgroups, whose per-head B and C rows are short
-    // and slow to arrive, before phase 1.
-    constexpr bool kEarlyPrefetch = WAVES == 2;
+    // hold no registers through phase 1), or before phase 1 -- for the two-wave workgroups, whose per-head B and C
+    // rows are short and slow to arrive, and for the eight-wave forward, where it costs 6 registers and measures 2 %
+    // faster with bf16 y, 8 % with float y (217 against 222 us and 245 against 268 us at batch 256, 2048 steps, 8 heads
+    // of 32, state 64).  The four-wave forward with a 128-wide state is 5 % slower with it and keeps the late request.
+    constexpr bool kEarlyPrefetch = WAVES == 2 || (KIND == 0 && WAVES == 8);
     // (transposed: UX passes of the eight heads' B and C rows, one piece of the shared x tile and of the second
     // operand's tile)
     uint4 bq[TR ? UX : UBC], cq[TR ? UX : UBC], xq[TR ? 1 : UX], auxq = make_uint4(0, 0, 0, 0);
@@ -904,8 +906,6 @@ template <typename TO, int NK, int QB, int WAVES>
 static hipError_t fused_launch(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
                                const void *Cm, const float *D, const float *init, const unsigned char *reset, void *y,
                                float *final_states, float *tile_states, hipStream_t st) {
-    // (requesting the next tile's inputs at the top of the tile instead of after phase 1 measured the same,
-    // 217.6 us against 218.8 us, for 26 more live registers)
     const int units = (s.H / s.G) * (s.P / 32);
     const int segments = s.seg_tiles > 0 ? (s.nc + s.seg_tiles - 1) / s.seg_tiles : 1;
     const int grid = s.B * s.G * (units / WAVES) * segments;
