@@ -260,7 +260,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // rows are short and slow to arrive, and for the eight-wave forward, where it costs 6 registers and measures 2 %
     // faster with bf16 y, 8 % with float y (217 against 222 us and 245 against 268 us at batch 256, 2048 steps, 8 heads
     // of 32, state 64).  The four-wave forward with a 128-wide state is 5 % slower with it and keeps the late request.
-    constexpr bool kEarlyPrefetch = WAVES == 2 || (KIND == 0 && WAVES == 8);
+    // Of the backward pass's kinds, 5 and 6 take it without spilling (the pass 1.10 against 1.12 ms); 7 would spill.
+    constexpr bool kEarlyPrefetch = WAVES == 2 || (WAVES == 8 && (KIND == 0 || KIND == 5 || KIND == 6));
     // (transposed: UX passes of the eight heads' B and C rows, one piece of the shared x tile and of the second
     // operand's tile)
     uint4 bq[TR ? UX : UBC], cq[TR ? UX : UBC], xq[TR ? 1 : UX], auxq = make_uint4(0, 0, 0, 0);
