@@ -19,6 +19,8 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
                64 steps as one call of ssd_steps_fwd (which runs 16 steps or more on the one-pass scan)
   reference_suite  the reference's historical benchmark cases for this path (batch 4, seq_len 4096,
                BFloat16), for the SSD op alone, in the reference's result schema
+  forward_float32  the same workload with float32 inputs (the other parity mode): staged kernels on float MFMAs,
+               time per call and dense flops against the 157.3 TFLOP/s float MFMA peak, which binds it
   backward     the backward pass of the scan at the same shape: time per call, and its compulsory traffic
                (x, dt, B, C, dy read; dx, ddt, dB, dC written) against the HBM peak
   mamba2_block the block around the scan at the policy shape (d_model = nheads*headdim): whole block, and the
@@ -48,6 +50,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # calibration factor 1.00); counters cannot be read from inside this script, so the figure is carried here
 MEASURED_TRAFFIC_BYTES = {("policy_bf16", 256, "onepass_scan"): 490.8e6}
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_F32_PEAK_TFLOPS = 157.3
 
 
 def parse_args():
@@ -62,6 +65,7 @@ def parse_args():
     ap.add_argument("--no-reference-suite", action="store_true")
     ap.add_argument("--no-block", action="store_true")
     ap.add_argument("--no-backward", action="store_true")
+    ap.add_argument("--no-float32", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise kernel over 256 MiB in / 256 MiB out three times, the known-size "
@@ -248,6 +252,24 @@ def main():
     }
     if onepass or segments > 1:
         out["onepass_scan"] = onepass_info
+
+    # ---- the same workload in float32 mode (the north star's other parity mode): bound by the float MFMAs ----
+    if not args.no_float32 and w.dtype == "bf16":
+        x32, dt32, B32, C32 = x.float(), dt.float(), Bm.float(), Cm.float()
+        try:
+            f32_call = ssd.PreparedChunkScan(x32, dt32, A, B32, C32, D, chunk=w.chunk, initial_states=init)
+        except ssd.SsdError:
+            f32_call = None   # float tiles of this shape do not fit the LDS
+        if f32_call is not None:
+            for _ in range(3):
+                f32_call()
+            t32 = wall_time_steps(f32_call, 20, torch)
+            fl = sum(sf[k] for k in ("chunk_state", "chunk_scan"))   # dense MFMA flops of the op
+            out["forward_float32"] = {"ms": round(t32 * 1e3, 4), "path": "staged", "bound": "mfma (float32)",
+                                      "dense_TFLOPs": round(fl / t32 / 1e12, 1), "peak_TFLOPs": MFMA_F32_PEAK_TFLOPS,
+                                      "mfma_frac": round(fl / t32 / 1e12 / MFMA_F32_PEAK_TFLOPS, 4),
+                                      "units_per_s": round(w.batch * w.seqlen / t32, 1)}
+        del x32, dt32, B32, C32, f32_call
 
     # ---- the backward pass at the benchmark shape ------------------------------------------------------
     if not args.no_backward:
