@@ -221,3 +221,36 @@ def test_block_stage_errors():
     assert ei.value.code == 2
     with pytest.raises(ValueError, match="conv_state"):
         block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], 8, 32, 64, 1, conv_state=torch.zeros(2, 2, 384).cuda())
+
+
+def test_block_stages_inside_a_captured_graph():
+    """The library's three block kernels (projection into padded rows, pre, post) captured in one graph: replays,
+    with the input changed in place and eager work in between, equal the eager calls bit for bit."""
+    H, P, N, G, K = 8, 32, 64, 1, 4
+    p = params(H, P, N, G, K)
+    E = 2 * H * P + 2 * G * N + H
+    g = torch.Generator().manual_seed(9)
+    u = torch.randn(4, 300, 256, generator=g).to(torch.bfloat16).cuda()
+    w_in = (torch.randn(E, 256, generator=g) / 16).to(torch.bfloat16).cuda()
+    y = torch.randn(4, 300, H, P, generator=g).to(torch.bfloat16).cuda()
+
+    def chain():
+        zx = block_proj(u, w_in, pad_rows=True)
+        outs = block_pre(zx, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G)
+        return outs + (block_post(y, zx, p["norm_w"], H, P, N, G),)
+
+    chain()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = chain()
+    u_keep = u.clone()
+    for i in range(4):
+        for t in captured:
+            t.fill_(float("nan"))
+        u.copy_(u_keep * 0.5 if i % 2 else u_keep)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = chain()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(captured, eager)), f"replay {i}"

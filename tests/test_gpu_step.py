@@ -246,3 +246,55 @@ def test_steps_refuses_what_it_cannot_hold_in_registers():
     assert ei.value.code == 2
     with pytest.raises(ValueError):
         ssd_steps(dev["init"].clone(), dev["x"][:, 0], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"])
+
+
+def test_step_and_steps_inside_a_captured_graph():
+    """An inference loop is the natural thing to capture (the reference captures its update,
+    trading_bots/src/torch/train/update.rs:206-330): one captured graph holds a single step, a short run of steps
+    (state in registers) and a long one (on the scan), all advancing the same state in place.  Replays are
+    interleaved with eager work and every one is checked against the same calls made eagerly, bit for bit."""
+    from trading_bot_0_amd import ssd_steps
+    Bsz, H, P, N, G = 6, 8, 32, 64, 1
+    w = Workload("steps_graph", Bsz, 1 + 5 + 40, H, P, N, G, 64, dtype="bf16", init_std=0.7)
+    dev = make_inputs(w, seed=31, device="cuda")
+    x, dt, Bm, Cm = dev["x"], dev["dt"], dev["B"], dev["C"]
+    reset = torch.zeros((Bsz, 40), dtype=torch.uint8, device="cuda")
+    reset[2, 0] = 1
+    reset[4, 17] = 1
+
+    # contiguous tensors of their own, at fixed addresses
+    parts = [t.contiguous() for t in (x[:, 0], dt[:, 0], Bm[:, 0], Cm[:, 0], x[:, 1:6], dt[:, 1:6], Bm[:, 1:6], Cm[:, 1:6],
+                                      x[:, 6:], dt[:, 6:], Bm[:, 6:], Cm[:, 6:])]
+    x0, d0, b0, c0, x5, d5, b5, c5, x40, d40, b40, c40 = parts
+
+    def calls(state, y1, y5, y40):
+        ssd_step(state, x0, d0, dev["A"], b0, c0, dev["D"], out=y1)
+        ssd_steps(state, x5, d5, dev["A"], b5, c5, dev["D"], out=y5)
+        ssd_steps(state, x40, d40, dev["A"], b40, c40, dev["D"], reset=reset, out=y40)
+
+    def outputs():
+        return (torch.empty((Bsz, H, P), dtype=torch.bfloat16, device="cuda"),
+                torch.empty((Bsz, 5, H, P), dtype=torch.bfloat16, device="cuda"),
+                torch.empty((Bsz, 40, H, P), dtype=torch.bfloat16, device="cuda"))
+
+    state = dev["init"].clone()
+    ys = outputs()
+    calls(state.clone(), *outputs())            # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        calls(state, *ys)
+    eager_state = dev["init"].clone()
+    state.copy_(dev["init"])
+    x40_keep = x40.clone()
+    for i in range(4):                          # the state carries over from replay to replay, as in a rollout
+        for y in ys:
+            y.fill_(float("nan"))
+        x40.copy_(x40_keep * 0.5 if i % 2 else x40_keep)   # change a captured input in place
+        graph.replay()
+        torch.cuda.synchronize()
+        ye = outputs()
+        calls(eager_state, *ye)
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(ys, ye)), f"replay {i}: y"
+        assert torch.equal(state, eager_state), f"replay {i}: state"
