@@ -206,6 +206,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     const int S = s.seg_tiles > 0 ? (s.nc + s.seg_tiles - 1) / s.seg_tiles : 1;
     const int slot = xcd_remap(blockIdx.x, gridDim.x);
     const int seg = slot % S, logical = slot / S;
+    // states only: nothing comes after the last segment, so what it adds to the state is not needed (the final
+    // state comes from the forward over that segment) -- its workgroups leave at once
+    if (STATES_ONLY && S > 1 && seg == S - 1) return;
     const int c_first = seg * (s.seg_tiles > 0 ? s.seg_tiles : s.nc);
     const int c_end = s.seg_tiles > 0 ? min(s.nc, c_first + s.seg_tiles) : s.nc;
     // transposed: the workgroup is heads h0 .. h0+7 (one per wave) on x slice pb; s.G == s.H there, and

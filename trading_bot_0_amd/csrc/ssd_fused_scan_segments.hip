@@ -15,6 +15,7 @@ constexpr int kSegmentMinTiles = 4;        // shorter segments are mostly prolog
 constexpr int kSegmentTargetGroups = 192;  // workgroups to aim for (256 CUs; the last quarter gains little)
 
 // enter[b,0] = init (or zero); enter[b,s+1] = decay[b,s] * enter[b,s] + local[b,s], written over local in place
+// (local and decay of the last segment are not read: the states-only pass does not compute them)
 __global__ __launch_bounds__(256) void segment_states_kernel(float *states, const float *__restrict__ decay,
                                                              const float *__restrict__ init,
                                                              const unsigned char *__restrict__ reset, int L, int S, int H,
@@ -29,6 +30,10 @@ __global__ __launch_bounds__(256) void segment_states_kernel(float *states, cons
     float4 cur = init && !fresh ? reinterpret_cast<const float4 *>(init)[bh * pn4 + idx] : make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s = 0; s < S; ++s) {
         float4 *slot = reinterpret_cast<float4 *>(states) + ((b * S + s) * H + h) * (long long)pn4 + idx;
+        if (s + 1 == S) {
+            *slot = cur;
+            break;
+        }
         const float4 loc = *slot;
         const float a = decay[(b * S + s) * H + h];
         *slot = cur;
