@@ -826,6 +826,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             }
         }
         // ---- phase 2: the state leaving this chunk ----
+        // (the forward's last tile of a segment other than the last, or of a call that asks for no final state: nobody
+        // reads the state it leaves)
+        if (KIND == 0 && c + 1 == c_end && !(final_states != nullptr && seg == S - 1)) break;
         if (!kEarlyPrefetch && c + 1 < c_end) prefetch(c + 1);
         // the other scan's state where this tile ends: the first slice in flight during phase 2, the second (two
         // slices per wave leave no registers to hold both) requested after it
