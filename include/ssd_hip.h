@@ -230,6 +230,16 @@ int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt,
                       const float *conv_b, const float *dt_bias, const void *conv_state_in, void *conv_state_out,
                       void *x, void *Bm, void *Cm, void *dt, void *hip_stream);
 
+/* ssd_block_pre_fwd with episode boundaries inside the window: reset [B,L] bytes or NULL (the mask
+ * ssd_chunk_scan_reset_fwd takes); a non-zero reset[b,t] cuts the filter's history before timestep t -- the inputs
+ * of earlier timesteps (and conv_state_in) count as zeros from t on, in the outputs and in conv_state_out -- so that
+ * a replayed window with reset slots (trading_bots/src/torch/train/rollout.rs:130-135) equals the rollout that
+ * zeroed the conv state between steps (trading_bots/src/torch/model/stream/state.rs:10-21).  ssd_block_pre_fwd is
+ * this function with reset = NULL. */
+int ssd_block_pre_reset_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt, const float *conv_w,
+                            const float *conv_b, const float *dt_bias, const void *conv_state_in, void *conv_state_out,
+                            const uint8_t *reset, void *x, void *Bm, void *Cm, void *dt, void *hip_stream);
+
 /* The block's two projections (the reference's equivalents are the linear layers around its temporal mixer,
  * trading_bots/src/torch/model/blocks/gqa.rs:82-109): out [rows, out_features] = u [rows, in_features] .
  * w [out_features, in_features]^T, bfloat16 in and out (dtype 1), float32 accumulation; rows = batch * seqlen.

@@ -22,8 +22,10 @@ def split_widths(H, P, N, G):
     return DI, GN, DI + 2 * GN, 2 * DI + 2 * GN + H
 
 
-def block_pre(zxbcdt, conv_w, conv_b, dt_bias, H, P, N, G, conv_state=None):
-    """zxbcdt [B,L,E] laid out [z | x | B | C | dt_raw] -> x, Bm, Cm, dt, new conv state [B,d_conv-1,C]."""
+def block_pre(zxbcdt, conv_w, conv_b, dt_bias, H, P, N, G, conv_state=None, reset=None):
+    """zxbcdt [B,L,E] laid out [z | x | B | C | dt_raw] -> x, Bm, Cm, dt, new conv state [B,d_conv-1,C].
+    reset [B,L] (non-zero = an episode boundary before that timestep): from t on, inputs of timesteps before t
+    (and the conv state) count as zeros."""
     zxbcdt = np.asarray(zxbcdt, np.float64)
     Bsz, L, E = zxbcdt.shape
     DI, GN, C, E_ = split_widths(H, P, N, G)
@@ -33,14 +35,29 @@ def block_pre(zxbcdt, conv_w, conv_b, dt_bias, H, P, N, G, conv_state=None):
     hist = np.zeros((Bsz, K - 1, C)) if conv_state is None else np.asarray(conv_state, np.float64)
     full = np.concatenate([hist, xbc], 1)                       # [B, K-1+L, C]
     out = np.zeros((Bsz, L, C))
-    for k in range(K):                                           # tap K-1 multiplies the current timestep
-        out += full[:, k:k + L, :] * np.asarray(conv_w, np.float64)[None, None, :, k]
+    cw = np.asarray(conv_w, np.float64)
+    if reset is None:
+        for k in range(K):                                       # tap K-1 multiplies the current timestep
+            out += full[:, k:k + L, :] * cw[None, None, :, k]
+        new_state = full[:, L:, :]
+    else:
+        # last[b,t] = the latest restart at or before t (far in the past: none): a tap at timestep s < last[b,t] is cut
+        rs = np.asarray(reset) != 0
+        last = np.where(rs, np.arange(L)[None, :], -(10 ** 9))
+        last = np.maximum.accumulate(last, axis=1)
+        for k in range(K):
+            src = np.arange(L) - (K - 1) + k                     # timestep of tap k at every t (negative: the state)
+            live = src[None, :] >= last                          # [B, L]
+            out += full[:, k:k + L, :] * cw[None, None, :, k] * live[:, :, None]
+        # the state after the window: the last K-1 timesteps, those before the window's last restart zeroed
+        tail = np.arange(L - (K - 1), L)
+        new_state = full[:, L:, :] * (tail[None, :] >= last[:, -1:])[:, :, None]
     out = silu(out + np.asarray(conv_b, np.float64))
     dt = softplus(zxbcdt[:, :, DI + C:] + np.asarray(dt_bias, np.float64))
     x = out[:, :, :DI].reshape(Bsz, L, H, P)
     Bm = out[:, :, DI:DI + GN].reshape(Bsz, L, G, N)
     Cm = out[:, :, DI + GN:].reshape(Bsz, L, G, N)
-    return x, Bm, Cm, dt, full[:, L:, :]
+    return x, Bm, Cm, dt, new_state
 
 
 def block_post(y, zxbcdt, norm_w, eps):
@@ -59,7 +76,7 @@ def block_forward(u, p, conv_state=None, ssm_state=None, reset=None):
     u = np.asarray(u, np.float64)
     zxbcdt = u @ p["in_proj"].T
     x, Bm, Cm, dt, conv = block_pre(zxbcdt, p["conv_w"], p["conv_b"], p["dt_bias"], p["H"], p["P"], p["N"], p["G"],
-                                    conv_state)
+                                    conv_state, reset)
     y, final = orc.ssd_sequential(x, dt, p["A"], Bm, Cm, p["D"], ssm_state, reset=reset)
     yn = block_post(y, zxbcdt, p["norm_w"], p["eps"])
     return yn @ p["out_proj"].T, conv, final

@@ -32,6 +32,93 @@ def test_header_symbols_are_exported(lib):
         assert getattr(lib, n) is not None
 
 
+# ---- the Rust binding (bindings/rust/ssd.rs) against the header: there is no Rust toolchain here, so the extern
+# block is checked as text: same functions, same number of parameters, same pointer constness, same pointee /
+# integer kinds, same field lists of the three structs.
+
+C_KINDS = {"void": "void", "float": "f32", "double": "f64", "char": "char", "uint8_t": "u8", "int": "int",
+           "int64_t": "i64", "size_t": "usize", "ssd_dims": "dims", "ssd_step_dims": "step_dims",
+           "ssd_block_dims": "block_dims"}
+RUST_KINDS = {"c_void": "void", "f32": "f32", "f64": "f64", "c_char": "char", "u8": "u8", "c_int": "int", "i64": "i64",
+              "usize": "usize", "SsdDims": "dims", "SsdStepDims": "step_dims", "SsdBlockDims": "block_dims"}
+
+
+def c_type_kind(decl, with_name=True):
+    """'const float *A' -> ('ptr_const', 'f32'); 'size_t workspace_bytes' -> ('value', 'usize')."""
+    decl = decl.strip()
+    if "*" in decl:
+        base = decl[:decl.index("*")].split()
+        const = "const" in base
+        base = [t for t in base if t not in ("const", "struct")]
+        assert len(base) == 1, decl
+        return ("ptr_const" if const else "ptr_mut", C_KINDS[base[0]])
+    toks = [t for t in decl.split() if t != "const"]
+    if with_name:
+        toks = toks[:-1]
+    assert len(toks) == 1, decl
+    return ("value", C_KINDS[toks[0]])
+
+
+def rust_type_kind(ty):
+    ty = ty.strip()
+    m = re.fullmatch(r"\*(const|mut)\s+(\w+)", ty)
+    if m:
+        return ("ptr_const" if m.group(1) == "const" else "ptr_mut", RUST_KINDS[m.group(2)])
+    return ("value", RUST_KINDS[ty])
+
+
+def header_prototypes():
+    text = (REPO / "include" / "ssd_hip.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    protos = {}
+    for ret, name, args in re.findall(r"^\s*([\w\s\*]+?)\b(ssd_\w+)\s*\(([^)]*)\)\s*;", text, flags=re.M):
+        params = [] if args.strip() in ("", "void") else [c_type_kind(a) for a in args.split(",")]
+        protos[name] = (c_type_kind(ret, with_name=False), params)
+    return protos
+
+
+def rust_prototypes():
+    text = (REPO / "bindings" / "rust" / "ssd.rs").read_text()
+    text = re.sub(r"//[^\n]*", "", text)
+    block = re.search(r'extern\s+"C"\s*\{(.*?)\n\}', text, flags=re.S).group(1)
+    protos = {}
+    for name, args, ret in re.findall(r"fn\s+(\w+)\s*\(([^)]*)\)\s*->\s*([^;]+);", block):
+        params = []
+        for a in args.split(","):
+            if a.strip():
+                params.append(rust_type_kind(a.split(":", 1)[1]))
+        protos[name] = (rust_type_kind(ret), params)
+    return protos
+
+
+def test_rust_binding_matches_the_header():
+    c, r = header_prototypes(), rust_prototypes()
+    assert sorted(c) == sorted(ssd.EXPORTED_SYMBOLS)          # the parser sees every declaration
+    assert sorted(r) == sorted(c), f"missing in ssd.rs: {sorted(set(c) - set(r))}, unknown: {sorted(set(r) - set(c))}"
+    for name in c:
+        assert r[name][0] == c[name][0], f"{name}: return type {r[name][0]} vs {c[name][0]}"
+        assert len(r[name][1]) == len(c[name][1]), f"{name}: {len(r[name][1])} parameters in ssd.rs, {len(c[name][1])} in the header"
+        for i, (a, b) in enumerate(zip(r[name][1], c[name][1])):
+            assert a == b, f"{name}: parameter {i} is {a} in ssd.rs, {b} in the header"
+
+
+def test_rust_structs_match_the_header():
+    htext = re.sub(r"/\*.*?\*/", "", (REPO / "include" / "ssd_hip.h").read_text(), flags=re.S)
+    rtext = re.sub(r"//[^\n]*", "", (REPO / "bindings" / "rust" / "ssd.rs").read_text())
+    for cname, rname in (("ssd_dims", "SsdDims"), ("ssd_step_dims", "SsdStepDims"), ("ssd_block_dims", "SsdBlockDims")):
+        body = re.search(r"typedef struct[^{]*\{([^}]*)\}\s*" + cname + r"\s*;", htext, flags=re.S).group(1)
+        cfields = []
+        for stmt in body.split(";"):
+            stmt = stmt.strip()
+            if stmt:
+                assert stmt.startswith("int64_t"), stmt
+                cfields += [f.strip() for f in stmt[len("int64_t"):].split(",")]
+        m = re.search(r"#\[repr\(C\)\]\s*(?:#\[[^\]]*\]\s*)*pub struct " + rname + r"\s*\{([^}]*)\}", rtext, flags=re.S)
+        assert m, f"{rname} must be #[repr(C)]"
+        rfields = re.findall(r"pub\s+(\w+)\s*:\s*i64", m.group(1))
+        assert rfields == cfields, f"{rname}: {rfields} vs {cfields}"
+
+
 def test_version_and_empty_error_slot(lib):
     assert lib.ssd_version() >= 100
     assert ssd.last_error(lib) is None
@@ -100,6 +187,25 @@ def test_null_misaligned_and_dtype(lib):
     assert "dtype" in ssd.last_error(lib)
     assert lib.ssd_step_fwd(byref(sd), 1, None, FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, None) == 1
     assert "state must not be NULL" in ssd.last_error(lib)
+
+
+def test_backward_rejects_null_dims(lib):
+    out = c_size_t(0)
+    assert lib.ssd_chunk_scan_bwd_workspace_bytes(None, 1, byref(out)) == 1
+    assert "dims must not be NULL" in ssd.last_error(lib)
+    args = [FAKE] * 5 + [None, None, None, FAKE, None] + [FAKE] * 5 + [None, None, FAKE]
+    assert lib.ssd_chunk_scan_bwd(None, 1, *args, 1 << 30, None) == 1
+    assert "dims must not be NULL" in ssd.last_error(lib)
+
+
+def test_stage1_lds_bound_on_nheads(lib):
+    """Stage 1 transposes a [chunk, nheads] tile of dt through LDS: (H*(Q+1)+Q)*4 bytes must fit 160 KiB."""
+    out = c_size_t(0)
+    ok = dims(nheads=152, chunk=256, headdim=32, dstate=32)       # 152*257*4 + 1024 = 157 280 bytes
+    assert lib.ssd_workspace_bytes(byref(ok), byref(out)) == 0
+    bad = dims(nheads=160, chunk=256, headdim=32, dstate=32)      # 165 504 bytes
+    assert lib.ssd_workspace_bytes(byref(bad), byref(out)) == 2
+    assert "stage 1" in ssd.last_error(lib)
 
 
 def test_error_slot_is_thread_local(lib):

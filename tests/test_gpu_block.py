@@ -211,6 +211,93 @@ def test_block_streams_prefix_then_steps_equals_the_window():
     assert torch.equal(o1[1], o2[1])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(3, 50, 8, 32, 64, 1, 4), (2, 19, 8, 16, 16, 2, 3), (2, 33, 8, 32, 32, 1, 2), (3, 2, 8, 32, 64, 1, 4)])
+def test_pre_scan_stage_with_restarts(shape, dtype):
+    """Episode boundaries inside the window cut the conv's history: against the oracle (pinned by running the
+    episodes as separate windows), with restarts on both sides of the kernel's runs of 16 timesteps, back to back,
+    at the first and at the last timestep."""
+    Bsz, L, H, P, N, G, K = shape
+    p = params(H, P, N, G, K)
+    E = 2 * H * P + 2 * G * N + H
+    g = torch.Generator().manual_seed(11)
+    z = torch.randn(Bsz, L, E, generator=g).to(dtype).cuda()
+    st = (torch.randn(Bsz, K - 1, H * P + 2 * G * N, generator=g)).to(dtype).cuda()
+    reset = torch.zeros(Bsz, L, dtype=torch.uint8)
+    for t in (0, 5, 6, 15, 16, 17, 31, 33, L - 1):
+        if 0 <= t < L:
+            reset[t % Bsz, t] = 1
+    reset[0, L - 1] = 1
+    for state in (None, st):
+        got = block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=state, return_conv_state=True,
+                        reset=reset.cuda())
+        ref = blk.block_pre(np64(z), np64(p["conv_w"]), np64(p["conv_b"]), np64(p["dt_bias"]), H, P, N, G,
+                            None if state is None else np64(state), reset.numpy())
+        for name, a, b in zip(("x", "B", "C", "dt"), got[:4], ref[:4]):
+            close(a, b, dtype, f"pre {name} with restarts")
+        assert torch.equal(got[4].float().cpu(), torch.from_numpy(ref[4]).float()), "conv state after restarts"
+    # an all-zero mask is no mask
+    a = block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=st, return_conv_state=True)
+    b_ = block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=st, return_conv_state=True,
+                   reset=torch.zeros(Bsz, L, dtype=torch.bool).cuda())
+    assert all(torch.equal(u, v) for u, v in zip(a, b_))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("K", [2, 3, 4])
+def test_conv_state_updated_in_place_for_one_timestep(K, dtype):
+    """seqlen 1 with conv_state_in == conv_state_out (what a streaming step does): the new state is the old one
+    shifted by one row plus the new input row, as with separate buffers, for every filter width."""
+    Bsz, H, P, N, G = 5, 8, 32, 64, 1
+    p = params(H, P, N, G, K)
+    E = 2 * H * P + 2 * G * N + H
+    g = torch.Generator().manual_seed(12 + K)
+    st0 = torch.randn(Bsz, K - 1, H * P + 2 * G * N, generator=g).to(dtype).cuda()
+    separate, inplace = st0.clone(), st0.clone()
+    for step in range(K + 1):
+        z = torch.randn(Bsz, 1, E, generator=g).to(dtype).cuda()
+        out_a = block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=separate, return_conv_state=True)
+        out_b = block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=inplace, conv_state_out=inplace)
+        torch.cuda.synchronize()
+        assert out_b[4] is inplace
+        assert all(torch.equal(u, v) for u, v in zip(out_a, out_b)), f"step {step}"
+        ref_state = torch.cat([separate[:, 1:], z[:, :, H * P:H * P + separate.shape[2]]], 1)
+        assert torch.equal(out_a[4], ref_state)
+        separate = out_a[4]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_window_with_restarts_equals_the_stream_that_was_reset(dtype):
+    """A replayed window with episode boundaries gives what the rollout produced: stepping the block bar by bar and
+    zeroing a stream's conv and SSM state (reset_rows) before the bars the mask marks."""
+    b = Mamba2Block(d_model=64, nheads=8, headdim=32, dstate=64, ngroups=1, seed=7)
+    Bsz, L = 3, 40
+    u = torch.randn(Bsz, L, 64, generator=torch.Generator().manual_seed(8)).to(dtype).cuda()
+    reset = torch.zeros(Bsz, L, dtype=torch.bool)
+    reset[0, [3, 4, 20]] = True
+    reset[1, 0] = True
+    reset[2, [17, L - 1]] = True
+    window = b.forward(u, reset=reset.cuda())
+    st = b.new_state(Bsz, dtype=dtype)
+    outs = []
+    for t in range(L):
+        rows = torch.nonzero(reset[:, t]).flatten().cuda()
+        if rows.numel():
+            st.reset_rows(rows)
+        outs.append(b.step(u[:, t].contiguous(), st).unsqueeze(1))
+    stepped = torch.cat(outs, 1)
+    torch.cuda.synchronize()
+    ref, _, _ = blk.block_forward(np64(u), oracle_params(b), reset=reset.numpy())
+    if dtype == torch.float32:
+        assert rel_err(window, ref) <= 1e-3 and rel_err(stepped, ref) <= 1e-3
+        assert rel_err(window, np64(stepped)) <= 1e-3
+    else:
+        assert rel_err(window, ref) <= 1e-1 and rel_err(stepped, ref) <= 1e-1
+        # without the cut the three bars after each restart would see the previous episode: far outside rounding
+        leaky = b.forward(u)
+        assert rel_err(window, np64(stepped)) < 0.25 * rel_err(leaky, np64(stepped))
+
+
 def test_block_stage_errors():
     p = params(8, 32, 64, 1, 4)
     z = torch.randn(2, 4, 2 * 256 + 128 + 8).cuda()

@@ -51,6 +51,34 @@ def test_conv_state_continues_the_sequence_also_for_windows_shorter_than_the_sta
     np.testing.assert_array_equal(state, full[4])
 
 
+def test_restarts_cut_the_conv_history_like_separate_windows():
+    """A window with restarts equals its episodes run as separate windows, each from a zero conv state (the first
+    from the carried state), and the state it leaves is the last episode's."""
+    p = params()
+    L = 23
+    z = RNG.standard_normal((3, L, E))
+    st = RNG.standard_normal((3, K - 1, C))
+    reset = np.zeros((3, L), np.uint8)
+    reset[0, [5, 6, 14]] = 1          # back-to-back restarts
+    reset[1, [0, L - 1]] = 1          # the first step (drops the carried state) and the last (a one-step episode)
+    got = blk.block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, st, reset)
+    for b in range(3):
+        cuts = [0] + [int(t) for t in np.nonzero(reset[b])[0] if t > 0] + [L]
+        state = None if reset[b, 0] else st[b:b + 1]
+        pieces = []
+        for a, e in zip(cuts[:-1], cuts[1:]):
+            pieces.append(blk.block_pre(z[b:b + 1, a:e], p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, state))
+            state = None
+        for i in range(4):
+            np.testing.assert_allclose(got[i][b:b + 1], np.concatenate([q[i] for q in pieces], 1), rtol=1e-12, atol=1e-13)
+        np.testing.assert_array_equal(got[4][b:b + 1], pieces[-1][4])
+    # no restarts: the mask changes nothing
+    plain = blk.block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, st)
+    same = blk.block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, st, np.zeros((3, L), np.uint8))
+    for a, b_ in zip(plain, same):
+        np.testing.assert_array_equal(a, b_)
+
+
 def test_gated_rmsnorm_row_by_row():
     y = RNG.standard_normal((2, 5, H, P))
     z = RNG.standard_normal((2, 5, E))

@@ -35,6 +35,8 @@ def _lib():
         lib.ssd_block_pre_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_block_post_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, P]
         lib.ssd_block_proj_fwd.argtypes = [c_int64, c_int64, c_int64, c_int64, c_int, P, P, P, P]
+        lib.ssd_block_pre_reset_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P, P]
+        lib.ssd_block_pre_reset_fwd.restype = c_int
         lib.ssd_block_pre_fwd.restype = c_int
         lib.ssd_block_post_fwd.restype = c_int
         lib.ssd_block_proj_fwd.restype = c_int
@@ -61,9 +63,10 @@ def _row_stride(zxbcdt) -> int:
 
 
 def block_pre(zxbcdt, conv_w, conv_b, dt_bias, nheads, headdim, dstate, ngroups, conv_state=None,
-              return_conv_state=False):
+              return_conv_state=False, reset=None, conv_state_out=None):
     """zxbcdt [B,L,E] (rows dense or evenly padded) -> (x [B,L,H,P], Bm, Cm [B,L,G,N], dt [B,L,H][, conv state
-    [B,d_conv-1,C]])."""
+    [B,d_conv-1,C]]).  `reset` [B,L] (uint8 or bool): a non-zero entry cuts the filter's history before that
+    timestep.  `conv_state_out`: where to write the new conv state (may be `conv_state` itself for seqlen 1)."""
     lib = _lib()
     if zxbcdt.dim() != 3:
         raise ValueError(f"block input must be rank-3 [batch, seqlen, channels], got {tuple(zxbcdt.shape)}")
@@ -90,11 +93,21 @@ def block_pre(zxbcdt, conv_w, conv_b, dt_bias, nheads, headdim, dstate, ngroups,
     Bm = torch.empty((Bsz, L, G, N), dtype=dtype, device=dev)
     Cm = torch.empty((Bsz, L, G, N), dtype=dtype, device=dev)
     dt = torch.empty((Bsz, L, H), dtype=dtype, device=dev)
-    new_state = torch.empty((Bsz, d_conv - 1, C), dtype=dtype, device=dev) if return_conv_state else None
+    new_state = None
+    if conv_state_out is not None:
+        ssd._require(conv_state_out, "conv_state_out", (Bsz, d_conv - 1, C), dtype)
+        new_state, return_conv_state = conv_state_out, True
+    elif return_conv_state:
+        new_state = torch.empty((Bsz, d_conv - 1, C), dtype=dtype, device=dev)
+    if reset is not None:
+        if reset.dtype == torch.bool:
+            reset = reset.view(torch.uint8)
+        ssd._require(reset, "reset", (Bsz, L), torch.uint8)
     dims = SsdBlockDims(Bsz, L, H, P, N, G, d_conv, ld)
-    ssd._check(lib, lib.ssd_block_pre_fwd(byref(dims), code, zxbcdt.data_ptr(), conv_w.data_ptr(), conv_b.data_ptr(),
-                                          dt_bias.data_ptr(), ssd._ptr(conv_state), ssd._ptr(new_state), x.data_ptr(),
-                                          Bm.data_ptr(), Cm.data_ptr(), dt.data_ptr(), ssd._stream_ptr(zxbcdt)))
+    ssd._check(lib, lib.ssd_block_pre_reset_fwd(byref(dims), code, zxbcdt.data_ptr(), conv_w.data_ptr(),
+                                                conv_b.data_ptr(), dt_bias.data_ptr(), ssd._ptr(conv_state),
+                                                ssd._ptr(new_state), ssd._ptr(reset), x.data_ptr(), Bm.data_ptr(),
+                                                Cm.data_ptr(), dt.data_ptr(), ssd._stream_ptr(zxbcdt)))
     return (x, Bm, Cm, dt, new_state) if return_conv_state else (x, Bm, Cm, dt)
 
 
@@ -206,14 +219,17 @@ class Mamba2Block:
     def forward(self, u: torch.Tensor, state: Optional[Mamba2StreamState] = None,
                 reset: Optional[torch.Tensor] = None) -> torch.Tensor:
         """u [B,L,d_model] -> [B,L,d_model].  With `state`, continues from it and leaves it at the end of the
-        window (a prefix scan; then `step` per bar)."""
+        window (a prefix scan; then `step` per bar).  `reset` [B,L]: episode boundaries inside the window -- a
+        non-zero entry restarts both the SSM state and the conv's history before that timestep, exactly what
+        `Mamba2StreamState.reset_rows` does between two steps of a stream."""
         if u.dim() != 3 or u.shape[2] != self.d_model:
             raise ValueError(f"block input must be [batch, seqlen, {self.d_model}], got {tuple(u.shape)}")
         if reset is not None and state is not None:
             raise ValueError("restarts inside the window and a carried conv state cannot be combined")
         zxbcdt = self._project(u, self.in_proj, pad_rows=True)  # internal to the block: rows of whole lines
         if state is None:
-            x, Bm, Cm, dt = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G)
+            x, Bm, Cm, dt = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G,
+                                      reset=reset)
             y, _ = ssd.ssd_chunk_scan(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk, return_final_states=False,
                                       reset=reset)
         else:
@@ -239,9 +255,8 @@ class Mamba2Block:
             raise ValueError(f"block step input must be [batch, {self.d_model}], got {tuple(u_t.shape)}")
         dt_ = u_t.dtype
         zxbcdt = torch.matmul(u_t, self.in_proj.to(dt_).t()).unsqueeze(1).contiguous()
-        x, Bm, Cm, dt, conv = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N,
-                                        self.G, conv_state=state.conv, return_conv_state=True)
-        state.conv = conv
+        x, Bm, Cm, dt, _ = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N,
+                                     self.G, conv_state=state.conv, conv_state_out=state.conv)  # in place
         y = state.ssm.step(x[:, 0], dt[:, 0], self.A, Bm[:, 0], Cm[:, 0], self.D)
         yn = block_post(y.unsqueeze(1), zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
         return torch.matmul(yn[:, 0], self.out_proj.to(dt_).t())

@@ -86,6 +86,9 @@ int make_shape(const ssd_dims *d, int dtype, ssd::ScanShape *out) {
         return fail(SSD_ERR_UNSUPPORTED,
                     "ssd: headdim %lld / dstate %lld / chunk %lld needs more than 160 KiB of LDS in %s mode",
                     (long long)d->headdim, (long long)d->dstate, (long long)d->chunk, eb == 2 ? "bf16" : "float32");
+    if (ssd::chunk_cumsum_lds_bytes(s) > ssd::kLdsLimitBytes)
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: nheads %lld with chunk %lld needs more than 160 KiB of LDS in stage 1",
+                    (long long)d->nheads, (long long)d->chunk);
     *out = s;
     return SSD_OK;
 }
@@ -224,6 +227,7 @@ constexpr int64_t kBackwardChunk = 64;
 // The backward pass runs the forward's stage kernels on the transposed state ([N,P] per head, B and C per head),
 // so the transposed shape must be one they take as well.
 int make_bwd_shapes(const ssd_dims *dims, int dtype, ssd::ScanShape *s, ssd::ScanShape *sT) {
+    if (dims == nullptr) return fail(SSD_ERR_INVALID, "ssd: dims must not be NULL");
     if (dtype != SSD_DTYPE_F32 && dtype != SSD_DTYPE_BF16)
         return fail(SSD_ERR_INVALID, "ssd: the backward pass takes dtype 0 (float32) or 1 (bfloat16), got %d", dtype);
     // The pass tiles time by at most kBackwardChunk steps whatever chunk the caller names (it owns its workspace
@@ -338,29 +342,15 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
                                     workspace, workspace_bytes, hip_stream);
 }
 
-int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
-                             const void *Bm, const void *Cm, const float *D, const float *initial_states,
-                             const uint8_t *reset, void *y, float *final_states, void *workspace,
-                             size_t workspace_bytes, void *hip_stream) {
-    ssd::ScanShape s;
-    if (int rc = make_shape(dims, dtype, &s)) return rc;
-    REQUIRE_PTR(x);
-    REQUIRE_PTR(dt);
-    REQUIRE_PTR(A);
-    REQUIRE_PTR(Bm);
-    REQUIRE_PTR(Cm);
-    REQUIRE_PTR(y);
-    REQUIRE_PTR(workspace);
-    OPTIONAL_PTR(D);
-    OPTIONAL_PTR(initial_states);
-    OPTIONAL_PTR(final_states);
+// The forward proper, arguments checked: the way the plan says for this shape, with `workspace` (carve(s).total bytes,
+// or anything at all when scan_scratch_bytes says the shape needs none) as scratch.
+static int scan_forward(const ssd::ScanShape &s, int dtype, const void *x, const void *dt, const float *A, const void *Bm,
+                        const void *Cm, const float *D, const float *initial_states, const uint8_t *reset, void *y,
+                        float *final_states, void *workspace, hipStream_t st) {
     const Workspace w = carve(s);
-    if (workspace_bytes < w.total)
-        return fail(SSD_ERR_WORKSPACE, "ssd: workspace has %zu bytes, %zu needed", workspace_bytes, w.total);
     char *base = static_cast<char *>(workspace);
     float *dtcs = reinterpret_cast<float *>(base + w.dtcs_off);
     float *states = reinterpret_cast<float *>(base + w.st_off);
-    hipStream_t st = (hipStream_t)hip_stream;
     // One batch of sequences, the way the plan says.  The workspace is carved for the whole batch and so holds any
     // part of it.
     auto forward = [&](const ssd::ScanShape &part, const void *px, const void *pdt, const void *pb, const void *pc,
@@ -404,6 +394,33 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
                        reinterpret_cast<float *>(const_cast<char *>(off(final_states, main_rows * row_st * 4))));
     }
     return forward(s, x, dt, Bm, Cm, initial_states, reset, y, final_states);
+}
+
+
+#define SSD_SCAN_POINTER_CHECKS \
+    REQUIRE_PTR(x);             \
+    REQUIRE_PTR(dt);            \
+    REQUIRE_PTR(A);             \
+    REQUIRE_PTR(Bm);            \
+    REQUIRE_PTR(Cm);            \
+    REQUIRE_PTR(y);             \
+    OPTIONAL_PTR(D);            \
+    OPTIONAL_PTR(initial_states); \
+    OPTIONAL_PTR(final_states)
+
+int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
+                             const void *Bm, const void *Cm, const float *D, const float *initial_states,
+                             const uint8_t *reset, void *y, float *final_states, void *workspace,
+                             size_t workspace_bytes, void *hip_stream) {
+    ssd::ScanShape s;
+    if (int rc = make_shape(dims, dtype, &s)) return rc;
+    SSD_SCAN_POINTER_CHECKS;
+    REQUIRE_PTR(workspace);
+    const Workspace w = carve(s);
+    if (workspace_bytes < w.total)
+        return fail(SSD_ERR_WORKSPACE, "ssd: workspace has %zu bytes, %zu needed", workspace_bytes, w.total);
+    return scan_forward(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states, workspace,
+                        (hipStream_t)hip_stream);
 }
 
 int ssd_chunk_scan_bwd_workspace_bytes(const ssd_dims *dims, int dtype, size_t *out_bytes) {
@@ -621,7 +638,7 @@ int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, c
     OPTIONAL_PTR(final_states);
     if (ssd::fused_scan_waves(s, dtype) == 0)
         return fail(SSD_ERR_UNSUPPORTED,
-                    "ssd: the one-pass scan needs bf16 inputs, headdim a multiple of 32, dstate 32 or 64 and "
+                    "ssd: the one-pass scan needs bf16 inputs, headdim a multiple of 32, dstate 32, 64 or 128 and "
                     "(nheads/ngroups)*(headdim/32) a multiple of 4");
     hipError_t e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states,
                                           (hipStream_t)hip_stream);
@@ -726,6 +743,13 @@ static int make_block_shape(const ssd_block_dims *d, int dtype, ssd::BlockShape 
 int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt, const float *conv_w,
                       const float *conv_b, const float *dt_bias, const void *conv_state_in, void *conv_state_out,
                       void *x, void *Bm, void *Cm, void *dt, void *hip_stream) {
+    return ssd_block_pre_reset_fwd(dims, dtype, zxbcdt, conv_w, conv_b, dt_bias, conv_state_in, conv_state_out, nullptr, x,
+                                   Bm, Cm, dt, hip_stream);
+}
+
+int ssd_block_pre_reset_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt, const float *conv_w,
+                            const float *conv_b, const float *dt_bias, const void *conv_state_in, void *conv_state_out,
+                            const uint8_t *reset, void *x, void *Bm, void *Cm, void *dt, void *hip_stream) {
     ssd::BlockShape s;
     if (int rc = make_block_shape(dims, dtype, &s)) return rc;
     REQUIRE_PTR(zxbcdt);
@@ -741,7 +765,7 @@ int ssd_block_pre_fwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt,
     if (conv_state_in != nullptr && conv_state_in == conv_state_out && s.L > 1)
         return fail(SSD_ERR_INVALID, "ssd: conv_state_in and conv_state_out may alias only for seqlen 1");
     hipError_t e = ssd::launch_block_pre(s, dtype == SSD_DTYPE_F32 ? 0 : 1, zxbcdt, conv_w, conv_b, dt_bias,
-                                         conv_state_in, conv_state_out, x, Bm, Cm, dt, (hipStream_t)hip_stream);
+                                         conv_state_in, conv_state_out, reset, x, Bm, Cm, dt, (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block pre-scan launch");
 }
 

@@ -47,13 +47,16 @@ template <> struct Pack8<float> {
 // per run.  The dt channels are done by the threads after those, one (timestep, 8 heads) each, so that no
 // wave mixes the two code paths.  History
 // before t = 0 comes from state_in [B, d_conv-1, C] (the last d_conv-1 input rows of the previous call) or is
-// zero; state_out receives the last d_conv-1 input rows.
+// zero; state_out receives the last d_conv-1 input rows.  reset [B, L] bytes or NULL: a non-zero reset[b,t] cuts
+// the filter's history before timestep t (an episode boundary: the rows before t count as zeros from t on, in the
+// outputs and in state_out), which is what zeroing the conv state between two calls does at a window boundary.
 constexpr int kPreSteps = 16;
 
 template <typename T, int DCONV>
 __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zxbcdt, const float *__restrict__ conv_w,
                                                         const float *__restrict__ conv_b, const float *__restrict__ dt_bias,
-                                                        const T *__restrict__ state_in, T *__restrict__ state_out,
+                                                        const T *state_in, T *state_out,
+                                                        const unsigned char *__restrict__ reset,
                                                         T *__restrict__ x, T *__restrict__ Bm, T *__restrict__ Cm,
                                                         T *__restrict__ dt, BlockShape s) {
     const int DI = s.H * s.P, GN = s.G * s.N, C = DI + 2 * GN;
@@ -119,6 +122,20 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
             for (int i = 0; i < 8; ++i) win[k][i] = v.get(i);
         }
     }
+    const unsigned char *rs = reset ? reset + (size_t)b * s.L : nullptr;
+    if (rs != nullptr) {
+        // a restart at one of the d_conv-2 timesteps before this run cuts the window rows before it
+        bool cut = false;
+#pragma unroll
+        for (int k = DCONV - 2; k >= 1; --k) {  // window row k is timestep t0 - (DCONV-1) + k
+            const int ts = t0 - (DCONV - 1) + k;
+            cut = cut || (ts >= 0 && rs[ts] != 0);
+            if (cut) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) win[k - 1][i] = 0.f;
+            }
+        }
+    }
     T *dst;
     int dst_stride;
     if (c0 < DI) {
@@ -141,6 +158,13 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
         const int t = t0 + j;
         if (t >= t1) break;
         const Pack8<T> v = in[j];
+        if (rs != nullptr && rs[t] != 0) {
+#pragma unroll
+            for (int k = 0; k < DCONV - 1; ++k) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) win[k][i] = 0.f;
+            }
+        }
         float acc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -151,28 +175,19 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
             acc[i] = silu(a);
         }
         Pack8<T>::store(dst + (size_t)t * dst_stride, acc);
-        // streaming state: the last d_conv-1 input rows
-        if (state_out != nullptr && t >= s.L - (DCONV - 1))
-            Pack8<T>::store(state_out + ((size_t)b * (DCONV - 1) + (t - (s.L - (DCONV - 1)))) * C + c0, win[DCONV - 1]);
 #pragma unroll
         for (int k = 0; k < DCONV - 1; ++k) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) win[k][i] = win[k + 1][i];
         }
     }
-    if (state_out != nullptr && s.L < DCONV - 1 && t0 == 0) {
-        // fewer new rows than the state holds: rows 0 .. d_conv-2-L of the new state are the old state's tail
-        for (int j = 0; j < (DCONV - 1) - s.L; ++j) {
-            float o[8];
+    // Streaming state: the d_conv-1 input rows before timestep L.  After the run that ends the sequence the window
+    // registers hold exactly those rows -- rows of this call, or, where the call brought fewer than d_conv-1 new
+    // rows, the tail of state_in, which was loaded before anything was stored: state_in and state_out may be the
+    // same memory whenever one thread both reads and writes a channel piece's state (seqlen <= kPreSteps).
+    if (state_out != nullptr && t1 == s.L) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = 0.f;
-            if (state_in != nullptr) {
-                const Pack8<T> v = Pack8<T>::load(state_in + ((size_t)b * (DCONV - 1) + j + s.L) * C + c0);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) o[i] = v.get(i);
-            }
-            Pack8<T>::store(state_out + ((size_t)b * (DCONV - 1) + j) * C + c0, o);
-        }
+        for (int k = 0; k < DCONV - 1; ++k) Pack8<T>::store(state_out + ((size_t)b * (DCONV - 1) + k) * C + c0, win[k]);
     }
 }
 
@@ -226,8 +241,8 @@ bool block_supported(const BlockShape &s) {
 
 template <typename T>
 static hipError_t pre_dispatch(const BlockShape &s, const void *zxbcdt, const float *conv_w, const float *conv_b,
-                               const float *dt_bias, const void *state_in, void *state_out, void *x, void *Bm,
-                               void *Cm, void *dt, hipStream_t st) {
+                               const float *dt_bias, const void *state_in, void *state_out,
+                               const unsigned char *reset, void *x, void *Bm, void *Cm, void *dt, hipStream_t st) {
     const long long total = (long long)s.B * ((s.L + kPreSteps - 1) / kPreSteps) * ((s.H * s.P + 2 * s.G * s.N) / 8) +
                             (long long)s.B * s.L * ((s.H + 7) / 8);
     const dim3 grid((unsigned)((total + 255) / 256)), block(256);
@@ -235,9 +250,9 @@ static hipError_t pre_dispatch(const BlockShape &s, const void *zxbcdt, const fl
     T *so = static_cast<T *>(state_out), *xx = static_cast<T *>(x), *bb = static_cast<T *>(Bm), *cc = static_cast<T *>(Cm),
       *dd = static_cast<T *>(dt);
     switch (s.d_conv) {
-        case 2: block_pre_kernel<T, 2><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, xx, bb, cc, dd, s); break;
-        case 3: block_pre_kernel<T, 3><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, xx, bb, cc, dd, s); break;
-        case 4: block_pre_kernel<T, 4><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, xx, bb, cc, dd, s); break;
+        case 2: block_pre_kernel<T, 2><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, reset, xx, bb, cc, dd, s); break;
+        case 3: block_pre_kernel<T, 3><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, reset, xx, bb, cc, dd, s); break;
+        case 4: block_pre_kernel<T, 4><<<grid, block, 0, st>>>(in, conv_w, conv_b, dt_bias, si, so, reset, xx, bb, cc, dd, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -245,9 +260,9 @@ static hipError_t pre_dispatch(const BlockShape &s, const void *zxbcdt, const fl
 
 hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w,
                             const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
-                            void *x, void *Bm, void *Cm, void *dt, hipStream_t st) {
-    return dtype ? pre_dispatch<__bf16>(s, zxbcdt, conv_w, conv_b, dt_bias, state_in, state_out, x, Bm, Cm, dt, st)
-                 : pre_dispatch<float>(s, zxbcdt, conv_w, conv_b, dt_bias, state_in, state_out, x, Bm, Cm, dt, st);
+                            const unsigned char *reset, void *x, void *Bm, void *Cm, void *dt, hipStream_t st) {
+    return dtype ? pre_dispatch<__bf16>(s, zxbcdt, conv_w, conv_b, dt_bias, state_in, state_out, reset, x, Bm, Cm, dt, st)
+                 : pre_dispatch<float>(s, zxbcdt, conv_w, conv_b, dt_bias, state_in, state_out, reset, x, Bm, Cm, dt, st);
 }
 
 template <typename T, typename TY>

@@ -13,6 +13,7 @@
 // same for column r.  Accumulator register v of that lane is element
 // (row 8*(v/4) + 4*half + v%4, column r).
 #pragma once
+#include <atomic>
 #include <type_traits>
 
 #include "ssd_launch.h"
@@ -378,24 +379,92 @@ __device__ inline Tile decode_tile(int logical, const ScanShape &s) {
 }
 
 
+// ------------------------------------------------------------------------------------------
+// Per-(kernel, device, launch configuration) facts the launchers need on every call -- the resident workgroups
+// per CU, whether the kernel's dynamic LDS limit has been raised -- are asked of the runtime once and kept in a
+// small table.  The entry points are re-entrant, so the table is lock-free: a slot is claimed by a compare-and-swap
+// on the kernel's address, filled, then published with a release store; a reader that finds a slot claimed but not
+// yet published (or the table full) asks the runtime itself.  One table per translation unit.
+// ------------------------------------------------------------------------------------------
+struct LaunchFacts {
+    static constexpr int kSlots = 256;
+    struct Slot {
+        std::atomic<uintptr_t> kernel{0};
+        std::atomic<uint64_t> config{0};
+        std::atomic<int> value{0};
+        std::atomic<int> ready{0};
+    };
+    Slot slots[kSlots];
+    // value kept for (kernel, config), or -1
+    int find(const void *kernel, uint64_t config) const {
+        const uintptr_t k = reinterpret_cast<uintptr_t>(kernel);
+        for (int i = 0, at = (int)((k >> 4) % kSlots); i < kSlots; ++i, at = (at + 1) % kSlots) {
+            const uintptr_t have = slots[at].kernel.load(std::memory_order_acquire);
+            if (have == 0) return -1;
+            if (have == k && slots[at].ready.load(std::memory_order_acquire) &&
+                slots[at].config.load(std::memory_order_relaxed) == config)
+                return slots[at].value.load(std::memory_order_relaxed);
+        }
+        return -1;
+    }
+    void keep(const void *kernel, uint64_t config, int value) {
+        const uintptr_t k = reinterpret_cast<uintptr_t>(kernel);
+        for (int i = 0, at = (int)((k >> 4) % kSlots); i < kSlots; ++i, at = (at + 1) % kSlots) {
+            uintptr_t empty = 0;
+            if (slots[at].kernel.compare_exchange_strong(empty, k, std::memory_order_acq_rel)) {
+                slots[at].config.store(config, std::memory_order_relaxed);
+                slots[at].value.store(value, std::memory_order_relaxed);
+                slots[at].ready.store(1, std::memory_order_release);
+                return;
+            }
+        }
+    }
+};
+static inline LaunchFacts &launch_facts() {
+    static LaunchFacts facts;
+    return facts;
+}
+static inline uint64_t launch_config_key(int kind, int dev, int block, size_t lds) {
+    return ((uint64_t)kind << 60) | ((uint64_t)(dev & 0xff) << 48) | ((uint64_t)(block & 0xffff) << 32) | (uint64_t)(lds & 0xffffffffu);
+}
+static inline hipError_t device_cu_count(int dev, int *cus) {
+    static std::atomic<int> known[64];
+    if (dev >= 0 && dev < 64) {
+        const int have = known[dev].load(std::memory_order_relaxed);
+        if (have > 0) {
+            *cus = have;
+            return hipSuccess;
+        }
+    }
+    hipError_t e = hipDeviceGetAttribute(cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess && dev >= 0 && dev < 64) known[dev].store(*cus, std::memory_order_relaxed);
+    return e;
+}
+
 // Workgroups of a persistent kernel: as many as stay resident on the current device, in whole
 // multiples of the 8 XCDs, never more than there are tiles.
 template <typename K>
 static inline hipError_t persistent_grid(K kernel, int block, size_t lds, int tiles, int *grid) {
-    int dev = 0, cus = 0, per_cu = 0;
+    int dev = 0, cus = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    e = device_cu_count(dev, &cus);
     if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, lds);
-    if (e != hipSuccess) return e;
-    // The occupancy query counts a workgroup whose LDS fills the CU to the last byte; measured, that
-    // one does not become resident, and a persistent grid larger than residency runs a second round.
-    if (lds > 0) {
-        const int by_lds = (int)(kLdsLimitBytes / (lds + 1024));
-        if (per_cu > by_lds) per_cu = by_lds;
+    const void *kp = reinterpret_cast<const void *>(kernel);
+    const uint64_t key = launch_config_key(1, dev, block, lds);
+    int per_cu = launch_facts().find(kp, key);
+    if (per_cu < 0) {
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, lds);
+        if (e != hipSuccess) return e;
+        // The occupancy query counts a workgroup whose LDS fills the CU to the last byte; measured, that
+        // one does not become resident, and a persistent grid larger than residency runs a second round.
+        if (lds > 0) {
+            const int by_lds = (int)(kLdsLimitBytes / (lds + 1024));
+            if (per_cu > by_lds) per_cu = by_lds;
+        }
+        if (per_cu < 1) per_cu = 1;
+        launch_facts().keep(kp, key, per_cu);
     }
-    if (per_cu < 1) per_cu = 1;
     long long g = (long long)cus * per_cu;
     if (g > tiles) g = tiles;
     if (g >= 8) g -= g % 8;
@@ -403,10 +472,18 @@ static inline hipError_t persistent_grid(K kernel, int block, size_t lds, int ti
     return hipSuccess;
 }
 
+// Raises a kernel's dynamic LDS limit to `bytes` (needed above 64 KiB), once per kernel, device and size.
 template <typename K> static inline hipError_t allow_lds(K kernel, size_t bytes) {
     if (bytes <= 64 * 1024) return hipSuccess;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const void *kp = reinterpret_cast<const void *>(kernel);
+    const uint64_t key = launch_config_key(2, dev, 0, bytes);
+    if (launch_facts().find(kp, key) == 1) return hipSuccess;
+    e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) launch_facts().keep(kp, key, 1);
+    return e;
 }
 
 }  // namespace ssd

@@ -37,6 +37,8 @@ struct BlockShape {  // a Mamba-2 block around the scan: conv width d_conv over 
 constexpr size_t kLdsLimitBytes = 160 * 1024;  // LDS per workgroup on gfx950
 
 // Dynamic LDS the stage-2 / stage-4 workgroup needs (elem_bytes = 2 for bf16, 4 for float).
+// (stage 1 transposes a [chunk, nheads] tile of dt through LDS)
+inline size_t chunk_cumsum_lds_bytes(const ScanShape &s) { return ((size_t)s.H * (s.Q + 1) + s.Q) * sizeof(float); }
 size_t chunk_state_lds_bytes(const ScanShape &s, int elem_bytes);
 size_t chunk_scan_lds_bytes(const ScanShape &s, int elem_bytes);
 
@@ -100,7 +102,8 @@ hipError_t launch_steps(const StepShape &s, int nsteps, int dtype, float *state,
 
 // The memory-bound stages of a Mamba-2 block around the scan.  zxbcdt [B,L,E], E = 2*H*P + 2*G*N + H, laid out
 // per timestep as [ z | x | B | C | dt_raw ].  pre: conv1d + bias + SiLU over x|B|C into the scan's tensors and
-// dt = softplus(dt_raw + dt_bias); conv state [B, d_conv-1, H*P + 2*G*N] in the activation dtype (both optional).
+// dt = softplus(dt_raw + dt_bias); conv state [B, d_conv-1, H*P + 2*G*N] in the activation dtype (both optional);
+// reset [B,L] bytes or NULL: a non-zero entry cuts the filter's history before that timestep.
 // post: out [B,L,H*P] = rmsnorm(y * silu(z)) * norm_w.  dtype 2 = bf16 activations with float32 y.
 bool block_supported(const BlockShape &s);
 // The block's projections in bf16: out [rows, out_features] = u [rows, in_features] . w [out_features, in_features]^T,
@@ -110,7 +113,7 @@ hipError_t launch_block_proj(long long rows, int in_features, int out_features, 
                              void *out, hipStream_t st);
 hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w,
                             const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
-                            void *x, void *Bm, void *Cm, void *dt, hipStream_t stream);
+                            const unsigned char *reset, void *x, void *Bm, void *Cm, void *dt, hipStream_t stream);
 hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                              float eps, void *out, hipStream_t stream);
 

@@ -286,13 +286,17 @@ template <typename T>
 static hipError_t cumsum_dispatch(const ScanShape &s, const void *dt, const float *A, const unsigned char *reset,
                                   float *dtcs, hipStream_t st, int mode, int dt_len) {
     const dim3 grid(s.B * s.nc), block(256);
-    const size_t lds = ((size_t)s.H * (s.Q + 1) + s.Q) * sizeof(float);
+    const size_t lds = chunk_cumsum_lds_bytes(s);
     const T *d = static_cast<const T *>(dt);
+    hipError_t e;
     if (s.Q <= 64) {
+        if ((e = allow_lds(chunk_cumsum_kernel<T, 1>, lds)) != hipSuccess) return e;
         chunk_cumsum_kernel<T, 1><<<grid, block, lds, st>>>(d, A, reset, dtcs, s, mode, dt_len);
     } else if (s.Q == 128) {
+        if ((e = allow_lds(chunk_cumsum_kernel<T, 2>, lds)) != hipSuccess) return e;
         chunk_cumsum_kernel<T, 2><<<grid, block, lds, st>>>(d, A, reset, dtcs, s, mode, dt_len);
     } else {
+        if ((e = allow_lds(chunk_cumsum_kernel<T, 4>, lds)) != hipSuccess) return e;
         chunk_cumsum_kernel<T, 4><<<grid, block, lds, st>>>(d, A, reset, dtcs, s, mode, dt_len);
     }
     return hipGetLastError();

@@ -47,6 +47,7 @@ EXPORTED_SYMBOLS = (
     "ssd_block_proj_fwd",
     "ssd_chunk_scan_bwd_workspace_bytes",
     "ssd_chunk_scan_bwd",
+    "ssd_block_pre_reset_fwd",
 )
 
 
