@@ -20,6 +20,9 @@ pub const SSD_DTYPE_F32: c_int = 0;
 pub const SSD_DTYPE_BF16: c_int = 1;
 /// bf16 inputs, y written as f32 (same arithmetic, no output rounding)
 pub const SSD_DTYPE_BF16_Y32: c_int = 2;
+/// scratch that `ssd_chunk_scan_noalloc_fwd` can draw on (part of the library's device code)
+pub const SSD_STATIC_SCRATCH_BYTES: usize = 64 << 20;
+
 #[repr(C)]
 #[derive(Clone, Copy, Debug)]
 pub struct SsdDims {
@@ -78,6 +81,9 @@ extern "C" {
         a: *const f32, bm: *const c_void, cm: *const c_void, d: *const f32, initial_states: *const f32,
         reset: *const u8, y: *mut c_void, final_states: *mut f32, workspace: *mut c_void, workspace_bytes: usize,
         hip_stream: *mut c_void) -> c_int;
+    pub fn ssd_chunk_scan_noalloc_fwd(dims: *const SsdDims, dtype: c_int, x: *const c_void, dt: *const c_void,
+        a: *const f32, bm: *const c_void, cm: *const c_void, d: *const f32, initial_states: *const f32,
+        reset: *const u8, y: *mut c_void, final_states: *mut f32, hip_stream: *mut c_void) -> c_int;
     pub fn ssd_chunk_scan_is_onepass(dims: *const SsdDims, dtype: c_int, is_onepass: *mut c_int) -> c_int;
     pub fn ssd_chunk_scan_segments(dims: *const SsdDims, dtype: c_int, segments: *mut c_int) -> c_int;
     pub fn ssd_state_passing_fwd(dims: *const SsdDims, chunk_states: *const f32, dtcs: *const f32,
@@ -207,6 +213,23 @@ pub fn ssd_chunk_scan(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tenso
                                  y.data_ptr(), fin.data_ptr() as *mut f32, ws.data_ptr(), need, std::ptr::null_mut())
     })?;
     Ok((y, fin))
+}
+
+/// The same into caller-owned outputs and without any allocation (graph capture, serving loops): scratch comes
+/// from the library's static array, so shapes whose workspace exceeds `SSD_STATIC_SCRATCH_BYTES` are refused
+/// unless they run as one launch of the one-pass kernel.  Calls that overlap on one GPU race on that array.
+pub fn ssd_chunk_scan_noalloc(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tensor, d: Option<&Tensor>,
+                              chunk: i64, initial_states: Option<&Tensor>, reset: Option<&Tensor>, y: &mut Tensor,
+                              final_states: &mut Tensor) -> Result<()> {
+    let dims = scan_dims(x, b, chunk)?;
+    validate_scan(&dims, x, dt, a, b, c, d, initial_states, reset)?;
+    require("y", y, &x.size(), x.kind())?;
+    require("final_states", final_states, &[dims.batch, dims.nheads, dims.headdim, dims.dstate], Kind::Float)?;
+    check(unsafe {
+        ssd_chunk_scan_noalloc_fwd(&dims, dtype_code(x)?, x.data_ptr(), dt.data_ptr(), a.data_ptr() as *const f32,
+                                   b.data_ptr(), c.data_ptr(), opt_f32(d), opt_f32(initial_states), opt_u8(reset),
+                                   y.data_ptr(), final_states.data_ptr() as *mut f32, std::ptr::null_mut())
+    })
 }
 
 /// Advances `state` `[B,H,P,N]` f32 in place by one timestep; returns y `[B,H,P]`.

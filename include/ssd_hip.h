@@ -136,6 +136,21 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
                              const uint8_t *reset, void *y, float *final_states, void *workspace,
                              size_t workspace_bytes, void *hip_stream);
 
+/* ssd_chunk_scan_reset_fwd for callers that cannot allocate device memory at all -- code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc -- and so cannot bring a workspace: the scratch the staged and
+ * segmented paths need comes from an array of SSD_STATIC_SCRATCH_BYTES (64 MiB) that is part of the library's device
+ * code (each GPU the library runs on holds it until the process ends).  No counterpart in the reference.  Same
+ * arguments and results as ssd_chunk_scan_reset_fwd minus the workspace.  Shapes whose workspace (ssd_workspace_bytes)
+ * exceeds the array return SSD_ERR_WORKSPACE, except those that run as one launch of the one-pass kernel
+ * (ssd_chunk_scan_is_onepass), which need no scratch at any size.  Calls no hipMalloc/hipFree or any other allocating
+ * routine.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different streams or
+ * threads) race on it; calls on one stream are ordered and safe.  Nothing in the array has to start at zero (every
+ * kernel writes what it later reads), so it is not cleared between calls. */
+#define SSD_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int ssd_chunk_scan_noalloc_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
+                               const void *Bm, const void *Cm, const float *D, const float *initial_states,
+                               const uint8_t *reset, void *y, float *final_states, void *hip_stream);
+
 /* *is_onepass = 1 if ssd_chunk_scan_fwd runs these dims as one launch of the one-pass kernel (its workspace is
  * then not touched), 0 otherwise (staged kernels, the one-pass kernel on segments, or a batch whose partial
  * last round of workgroups runs as a batch of its own).  A plan query like ssd_workspace_bytes; no reference counterpart. */

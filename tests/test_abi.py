@@ -208,6 +208,22 @@ def test_stage1_lds_bound_on_nheads(lib):
     assert "stage 1" in ssd.last_error(lib)
 
 
+def test_noalloc_entry_rejects_shapes_beyond_its_scratch(lib):
+    """Validation happens before the device is touched: a staged shape whose workspace exceeds the static array
+    is refused with the sizes in the message."""
+    d = dims(batch=64, seqlen=4096, nheads=8, headdim=32, dstate=64, chunk=128)   # float32: staged, 150 MB
+    need = c_size_t(0)
+    assert lib.ssd_workspace_bytes(byref(d), byref(need)) == 0 and need.value > (64 << 20)
+    args = [FAKE] * 5 + [None, None, None, FAKE, None]   # x dt A B C D init reset y final
+    assert lib.ssd_chunk_scan_noalloc_fwd(byref(d), 0, *args, None) == 3
+    msg = ssd.last_error(lib)
+    assert str(need.value) in msg and str(64 << 20) in msg
+    assert lib.ssd_chunk_scan_noalloc_fwd(byref(d), 0, None, *args[1:], None) == 3   # (size is checked first)
+    ssd.last_error(lib)
+    assert lib.ssd_chunk_scan_noalloc_fwd(None, 1, *args, None) == 1
+    assert "dims" in ssd.last_error(lib)
+
+
 def test_error_slot_is_thread_local(lib):
     import threading
     out = c_size_t(0)

@@ -9,7 +9,15 @@
 #include <cstdlib>
 #include <cstring>
 
+#include <atomic>
+
 #include "ssd_launch.h"
+
+// Scratch of ssd_chunk_scan_noalloc_fwd: device memory that exists from the moment the library's code object is
+// loaded on a GPU until the process ends, so that entry point never allocates.  Every call on a GPU shares that GPU's
+// copy; host code reaches it only through the address hipGetSymbolAddress returns (static_scratch_address below).
+constexpr size_t kStaticScratchBytes = (size_t)64 << 20;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
 
 namespace {
 
@@ -121,6 +129,29 @@ bool takes_one_pass(const ssd::ScanShape &s, int dtype) {
 
 int hip_fail(hipError_t e, const char *what) {
     return fail(SSD_ERR_RUNTIME, "ssd: %s failed: %s", what, hipGetErrorString(e));
+}
+
+// Device address of g_static_scratch on the current device.  In host code the array's name is only a handle for the
+// runtime's symbol lookup, not a device address, and every GPU holds its own copy at its own address: the address
+// is looked up once per device, with that device current, and kept.  Lock-free: two threads that race on a
+// device's first call look up the same address and store the same value.
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_static_scratch_ptr[kMaxDevices];
+
+int static_scratch_address(void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(SSD_ERR_UNSUPPORTED, "ssd: device index %d is beyond %d", dev, kMaxDevices - 1);
+    void *p = g_static_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress of the static scratch array");
+        if (p == nullptr) return fail(SSD_ERR_RUNTIME, "ssd: the static scratch array has no device address");
+        g_static_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return SSD_OK;
 }
 
 // Stages 1-4 one after the other.  mode as for launch_chunk_cumsum (0 = the forward's decays and weights).
@@ -420,6 +451,26 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
     if (workspace_bytes < w.total)
         return fail(SSD_ERR_WORKSPACE, "ssd: workspace has %zu bytes, %zu needed", workspace_bytes, w.total);
     return scan_forward(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states, workspace,
+                        (hipStream_t)hip_stream);
+}
+
+int ssd_chunk_scan_noalloc_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
+                               const void *Bm, const void *Cm, const float *D, const float *initial_states,
+                               const uint8_t *reset, void *y, float *final_states, void *hip_stream) {
+    ssd::ScanShape s;
+    if (int rc = make_shape(dims, dtype, &s)) return rc;
+    // what the forward of this shape would carve out of a caller's workspace: nothing when it runs as one launch of
+    // the one-pass kernel
+    const size_t need = (takes_one_pass(s, dtype) && ssd::fused_scan_tail_rows(s, dtype) == 0) ? 0 : carve(s).total;
+    if (need > kStaticScratchBytes)
+        return fail(SSD_ERR_WORKSPACE,
+                    "ssd: this shape needs %zu bytes of scratch, the library's static scratch array holds %zu; call "
+                    "ssd_chunk_scan_fwd with a workspace of ssd_workspace_bytes() instead",
+                    need, kStaticScratchBytes);
+    SSD_SCAN_POINTER_CHECKS;
+    void *scratch = nullptr;
+    if (int rc = static_scratch_address(&scratch)) return rc;
+    return scan_forward(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states, scratch,
                         (hipStream_t)hip_stream);
 }
 

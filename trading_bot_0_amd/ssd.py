@@ -47,6 +47,7 @@ EXPORTED_SYMBOLS = (
     "ssd_block_proj_fwd",
     "ssd_chunk_scan_bwd_workspace_bytes",
     "ssd_chunk_scan_bwd",
+    "ssd_chunk_scan_noalloc_fwd",
     "ssd_block_pre_reset_fwd",
 )
 
@@ -101,6 +102,7 @@ def load_library() -> ctypes.CDLL:
         lib.ssd_chunk_state_passing_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P]
         lib.ssd_chunk_scan_onepass_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_chunk_scan_reset_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, P, c_size_t, P]
+        lib.ssd_chunk_scan_noalloc_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_chunk_scan_is_onepass.argtypes = [POINTER(SsdDims), c_int, POINTER(c_int)]
         lib.ssd_chunk_scan_segments.argtypes = [POINTER(SsdDims), c_int, POINTER(c_int)]
         lib.ssd_chunk_scan_stage_fwd.argtypes = [POINTER(SsdDims), c_int, P, P, P, P, P, P, P, P]
