@@ -285,3 +285,29 @@ def test_reset_is_a_fresh_sequence_from_that_timestep():
     y2, f2 = orc.ssd_sequential(x[2:], dt[2:], A, Bm[2:], Cm[2:], D, None)
     np.testing.assert_allclose(y[2:], y2, rtol=1e-12, atol=1e-13)
     np.testing.assert_allclose(f[2:], f2, rtol=1e-12, atol=1e-13)
+
+
+def test_torch_cpu_restatement_matches_the_oracle():
+    """oracle/ssd_torch_cpu.py (the ATen-CPU form bench.py times as the CPU baseline) against the float64
+    sequential recurrence: groups, a ragged length, an initial state; float64 to 1e-10, float32 to 1e-4."""
+    import torch
+    from oracle.ssd_torch_cpu import ssd_chunked_torch
+    rng = np.random.default_rng(5)
+    Bsz, L, H, P, N, G, Q = 2, 150, 4, 8, 16, 2, 64
+    x = rng.standard_normal((Bsz, L, H, P))
+    dt = np.log1p(np.exp(rng.standard_normal((Bsz, L, H)) - 2))
+    A = -np.exp(rng.uniform(0, np.log(16), H))
+    Bm = rng.standard_normal((Bsz, L, G, N)) / 4
+    Cm = rng.standard_normal((Bsz, L, G, N)) / 4
+    D = rng.standard_normal(H)
+    init = rng.standard_normal((Bsz, H, P, N)) * 0.1
+    yr, fr = orc.ssd_sequential(x, dt, A, Bm, Cm, D, init)
+    t = lambda a, d: torch.from_numpy(np.asarray(a)).to(d)
+    for dtype, tol in ((torch.float64, 1e-10), (torch.float32, 1e-4)):
+        y, f = ssd_chunked_torch(t(x, dtype), t(dt, dtype), t(A, dtype), t(Bm, dtype), t(Cm, dtype), t(D, dtype),
+                                 t(init, dtype), chunk=Q)
+        assert orc.rel_err(y.double().numpy(), yr) <= tol and orc.rel_err(f.double().numpy(), fr) <= tol
+    y, f = ssd_chunked_torch(t(x, torch.float64), t(dt, torch.float64), t(A, torch.float64), t(Bm, torch.float64),
+                             t(Cm, torch.float64), None, None, chunk=32)
+    y0, f0 = orc.ssd_sequential(x, dt, A, Bm, Cm)
+    assert orc.rel_err(y.numpy(), y0) <= 1e-10 and orc.rel_err(f.numpy(), f0) <= 1e-10
