@@ -479,7 +479,7 @@ def main():
                 rdo = torch.randn_like(ru)
 
                 def block_fwd_bwd():
-                    ctx = rblk.forward(ru, save_for_backward=True)
+                    _, ctx = rblk.forward(ru, save_for_backward=True)
                     rblk.backward(ctx, rdo)
 
                 spin(block_fwd_bwd, torch, 0.1)

@@ -114,6 +114,15 @@ extern "C" {
         u: *const c_void, w: *const c_void, out: *mut c_void, hip_stream: *mut c_void) -> c_int;
     pub fn ssd_block_post_fwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
         norm_w: *const f32, eps: f32, out: *mut c_void, hip_stream: *mut c_void) -> c_int;
+    pub fn ssd_block_bwd_workspace_bytes(dims: *const SsdBlockDims, dtype: c_int, out_bytes: *mut usize) -> c_int;
+    pub fn ssd_block_post_bwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
+        norm_w: *const f32, eps: f32, dout: *const c_void, dy: *mut c_void, dzxbcdt: *mut c_void, dnorm_w: *mut f32,
+        workspace: *mut c_void, workspace_bytes: usize, hip_stream: *mut c_void) -> c_int;
+    pub fn ssd_block_pre_bwd(dims: *const SsdBlockDims, dtype: c_int, zxbcdt: *const c_void, conv_w: *const f32,
+        conv_b: *const f32, dt_bias: *const f32, conv_state_in: *const c_void, reset: *const u8, dx: *const c_void,
+        db: *const c_void, dc: *const c_void, ddt: *const c_void, dconv_state_out: *const c_void,
+        dzxbcdt: *mut c_void, dconv_w: *mut f32, dconv_b: *mut f32, ddt_bias: *mut f32,
+        dconv_state_in: *mut c_void, workspace: *mut c_void, workspace_bytes: usize, hip_stream: *mut c_void) -> c_int;
 }
 
 /// Maps a return code to `anyhow`, with the library's message (malloc'd; freed here).

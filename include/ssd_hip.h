@@ -268,6 +268,32 @@ int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, 
 int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,
                        const float *norm_w, float eps, void *out, void *hip_stream);
 
+/* ---- Backward pass of the block's two stages -------------------------------------------------------------------
+ * With ssd_chunk_scan_bwd between them and two GEMMs per projection (the caller's BLAS), these make the block
+ * trainable: the reference's historical benchmark case for it is mamba2_fwd_bwd_train
+ * (benchmark_results/bench_20260112_070055.json:16-23), the update they would run in is
+ * trading_bots/src/torch/train/update.rs:206-330.  dzxbcdt [B,L,zxbcdt_ld] is the gradient of zxbcdt, laid out like it:
+ * ssd_block_post_bwd writes its z channels, ssd_block_pre_bwd its x | B | C | dt channels (padding columns are not
+ * touched).  Parameter gradients are float32 and are summed in a fixed order (same bits on every run); the partial
+ * sums live in a workspace of ssd_block_bwd_workspace_bytes, which the two calls of one backward pass may share. */
+int ssd_block_bwd_workspace_bytes(const ssd_block_dims *dims, int dtype, size_t *out_bytes);
+
+/* Gradients of ssd_block_post_fwd: dout [B,L,H*P] -> dy [B,L,H,P] (activation dtype), dz into dzxbcdt, dnorm_w [H*P].
+ * y is the scan's output as the forward took it (dtype 2: float32 y with bf16 activations). */
+int ssd_block_post_bwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                       float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *workspace,
+                       size_t workspace_bytes, void *hip_stream);
+
+/* Gradients of ssd_block_pre_reset_fwd: from dx [B,L,H,P], dB, dC [B,L,G,N], ddt [B,L,H] (what ssd_chunk_scan_bwd
+ * returns) and, optionally, dconv_state_out [B,d_conv-1,C] (a gradient on the conv state the forward returned) to
+ * the x | B | C | dt channels of dzxbcdt, dconv_w [C,d_conv], dconv_b [C], ddt_bias [H] and, when asked for,
+ * dconv_state_in [B,d_conv-1,C].  conv_state_in and reset are the forward's (NULL allowed). */
+int ssd_block_pre_bwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt, const float *conv_w, const float *conv_b,
+                      const float *dt_bias, const void *conv_state_in, const uint8_t *reset, const void *dx, const void *dB,
+                      const void *dC, const void *ddt, const void *dconv_state_out, void *dzxbcdt, float *dconv_w,
+                      float *dconv_b, float *ddt_bias, void *dconv_state_in, void *workspace, size_t workspace_bytes,
+                      void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -113,3 +113,76 @@ def test_block_is_its_stages_composed_and_streams():
         outs.append(o)
     np.testing.assert_allclose(np.concatenate(outs, 1), out, rtol=1e-10, atol=1e-12)
     np.testing.assert_allclose(ss, final, rtol=1e-10, atol=1e-12)
+
+
+def _central(f, a, eps=1e-6):
+    """Central differences of the scalar function f with respect to the array a (varied in place)."""
+    g = np.zeros_like(a)
+    it = np.nditer(a, flags=["multi_index"])
+    for _ in it:
+        i = it.multi_index
+        keep = a[i]
+        a[i] = keep + eps
+        up = f()
+        a[i] = keep - eps
+        dn = f()
+        a[i] = keep
+        g[i] = (up - dn) / (2 * eps)
+    return g
+
+
+def test_post_backward_matches_central_differences():
+    y = RNG.standard_normal((2, 3, H, P))
+    z = RNG.standard_normal((2, 3, E))
+    w = RNG.standard_normal(DI)
+    dout = RNG.standard_normal((2, 3, DI))
+    dy, dz, dw = blk.block_post_bwd(y, z, w, 1e-3, dout)
+    loss = lambda: (blk.block_post(y, z, w, 1e-3) * dout).sum()
+    np.testing.assert_allclose(dy, _central(loss, y), rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(dz, _central(loss, z)[:, :, :DI], rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(dw, _central(loss, w), rtol=1e-6, atol=1e-8)
+
+
+def test_pre_backward_matches_central_differences_with_state_and_restarts():
+    p = params()
+    L = 9
+    z = RNG.standard_normal((2, L, E))
+    st = RNG.standard_normal((2, K - 1, C))
+    reset = np.zeros((2, L), np.uint8)
+    reset[0, [3, 4]] = 1
+    reset[1, L - 2] = 1
+    gx, gB, gC = RNG.standard_normal((2, L, H, P)), RNG.standard_normal((2, L, G, N)), RNG.standard_normal((2, L, G, N))
+    gdt, gst = RNG.standard_normal((2, L, H)), RNG.standard_normal((2, K - 1, C))
+    for rs, gs in ((None, None), (reset, gst)):
+        def loss():
+            x, Bm, Cm, dt, so = blk.block_pre(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, st, rs)
+            return (x * gx).sum() + (Bm * gB).sum() + (Cm * gC).sum() + (dt * gdt).sum() + (0.0 if gs is None else (so * gs).sum())
+        dxbc, ddt_raw, dcw, dcb, ddb, dst = blk.block_pre_bwd(z, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, gx, gB, gC,
+                                                             gdt, st, rs, gs)
+        dz = _central(loss, z)
+        np.testing.assert_allclose(dxbc, dz[:, :, DI:DI + C], rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(ddt_raw, dz[:, :, DI + C:], rtol=1e-6, atol=1e-8)
+        assert np.abs(dz[:, :, :DI]).max() < 1e-8                      # pre does not read z
+        np.testing.assert_allclose(dcw, _central(loss, p["conv_w"]), rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(dcb, _central(loss, p["conv_b"]), rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(ddb, _central(loss, p["dt_bias"]), rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(dst, _central(loss, st), rtol=1e-6, atol=1e-8)
+
+
+def test_block_backward_matches_central_differences():
+    d_model = 6
+    p = params()
+    p.update(in_proj=RNG.standard_normal((E, d_model)) / 3, out_proj=RNG.standard_normal((d_model, DI)) / 5,
+             A=-np.exp(RNG.uniform(0, 1.5, H)), D=RNG.standard_normal(H), norm_w=RNG.standard_normal(DI),
+             H=H, P=P, N=N, G=G, eps=1e-3)
+    u = RNG.standard_normal((2, 6, d_model))
+    dout = RNG.standard_normal((2, 6, d_model))
+    reset = np.zeros((2, 6), np.uint8)
+    reset[1, 3] = 1
+    for rs in (None, reset):
+        g = blk.block_backward(u, p, dout, reset=rs)
+        loss = lambda: (blk.block_forward(u, p, reset=rs)[0] * dout).sum()
+        np.testing.assert_allclose(g["du"], _central(loss, u), rtol=2e-5, atol=1e-7)
+        for name, key in (("in_proj", "din_proj"), ("conv_w", "dconv_w"), ("conv_b", "dconv_b"), ("dt_bias", "ddt_bias"),
+                          ("A", "dA"), ("D", "dD"), ("norm_w", "dnorm_w"), ("out_proj", "dout_proj")):
+            np.testing.assert_allclose(g[key], _central(loss, p[name]), rtol=2e-5, atol=1e-7, err_msg=name)

@@ -10,7 +10,7 @@ and post-scan kernels bound here and the scan / step of `ssd.py`.
 from __future__ import annotations
 
 import math
-from ctypes import POINTER, Structure, byref, c_float, c_int, c_int64, c_void_p
+from ctypes import POINTER, Structure, byref, c_float, c_int, c_int64, c_size_t, c_void_p
 from dataclasses import dataclass
 from typing import Optional, Tuple
 
@@ -37,6 +37,11 @@ def _lib():
         lib.ssd_block_proj_fwd.argtypes = [c_int64, c_int64, c_int64, c_int64, c_int, P, P, P, P]
         lib.ssd_block_pre_reset_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_block_pre_reset_fwd.restype = c_int
+        lib.ssd_block_bwd_workspace_bytes.argtypes = [POINTER(SsdBlockDims), c_int, POINTER(c_size_t)]
+        lib.ssd_block_post_bwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, P, P, P, P, c_size_t, P]
+        lib.ssd_block_pre_bwd.argtypes = [POINTER(SsdBlockDims), c_int] + [P] * 17 + [c_size_t, P]
+        for name in ("ssd_block_bwd_workspace_bytes", "ssd_block_post_bwd", "ssd_block_pre_bwd"):
+            getattr(lib, name).restype = c_int
         lib.ssd_block_pre_fwd.restype = c_int
         lib.ssd_block_post_fwd.restype = c_int
         lib.ssd_block_proj_fwd.restype = c_int
@@ -134,6 +139,90 @@ def block_post(y, zxbcdt, norm_w, nheads, headdim, dstate, ngroups, eps=1e-5):
     return out
 
 
+def block_bwd_workspace(batch, seqlen, nheads, headdim, dstate, ngroups, d_conv=4, dtype=torch.bfloat16, device="cuda"):
+    """Scratch for the partial sums of block_post_bwd / block_pre_bwd (one buffer serves both calls of a pass)."""
+    lib = _lib()
+    need = c_size_t(0)
+    dims = SsdBlockDims(batch, seqlen, nheads, headdim, dstate, ngroups, d_conv, 0)
+    code = ssd.SSD_DTYPE_F32 if dtype == torch.float32 else ssd.SSD_DTYPE_BF16
+    ssd._check(lib, lib.ssd_block_bwd_workspace_bytes(byref(dims), code, byref(need)))
+    return torch.empty(need.value, dtype=torch.uint8, device=device)
+
+
+def block_post_bwd(y, zxbcdt, norm_w, dout, dzxbcdt, nheads, headdim, dstate, ngroups, eps=1e-5, workspace=None):
+    """Gradients of block_post: returns (dy [B,L,H,P], dnorm_w [H*P]) and writes dz into the z channels of dzxbcdt
+    (a tensor laid out like zxbcdt, same row stride)."""
+    lib = _lib()
+    Bsz, L, E = zxbcdt.shape
+    H, P, N, G = nheads, headdim, dstate, ngroups
+    dtype = zxbcdt.dtype
+    code = ssd._dtype_code(zxbcdt)
+    if y.dtype != dtype:
+        if not (dtype == torch.bfloat16 and y.dtype == torch.float32):
+            raise ValueError(f"block y must be {dtype} (or float32 with bf16 activations), got {y.dtype}")
+        code = ssd.SSD_DTYPE_BF16_Y32
+    ld = _row_stride(zxbcdt)
+    if tuple(dzxbcdt.shape) != (Bsz, L, E) or dzxbcdt.dtype != dtype or _row_stride(dzxbcdt) != ld:
+        raise ValueError("dzxbcdt must have zxbcdt's shape, dtype and row stride")
+    ssd._require(y, "y", (Bsz, L, H, P), y.dtype)
+    ssd._require(dout, "dout", (Bsz, L, H * P), dtype)
+    ssd._require(norm_w, "norm_w", (H * P,), torch.float32)
+    dy = torch.empty((Bsz, L, H, P), dtype=dtype, device=zxbcdt.device)
+    dnorm_w = torch.empty(H * P, dtype=torch.float32, device=zxbcdt.device)
+    if workspace is None:
+        workspace = block_bwd_workspace(Bsz, L, H, P, N, G, 4, dtype, zxbcdt.device)
+    dims = SsdBlockDims(Bsz, L, H, P, N, G, 4, ld)
+    ssd._check(lib, lib.ssd_block_post_bwd(byref(dims), code, y.data_ptr(), zxbcdt.data_ptr(), norm_w.data_ptr(), c_float(eps),
+                                           dout.data_ptr(), dy.data_ptr(), dzxbcdt.data_ptr(), dnorm_w.data_ptr(),
+                                           workspace.data_ptr(), workspace.numel(), ssd._stream_ptr(zxbcdt)))
+    return dy, dnorm_w
+
+
+def block_pre_bwd(zxbcdt, conv_w, conv_b, dt_bias, dx, dB, dC, ddt, dzxbcdt, nheads, headdim, dstate, ngroups,
+                  conv_state=None, reset=None, dconv_state_out=None, need_dconv_state=False, workspace=None):
+    """Gradients of block_pre: writes the x | B | C | dt channels of dzxbcdt and returns (dconv_w [C,d_conv],
+    dconv_b [C], ddt_bias [H], dconv_state [B,d_conv-1,C] or None)."""
+    lib = _lib()
+    Bsz, L, E = zxbcdt.shape
+    H, P, N, G = nheads, headdim, dstate, ngroups
+    C = H * P + 2 * G * N
+    dtype = zxbcdt.dtype
+    code = ssd._dtype_code(zxbcdt)
+    ld = _row_stride(zxbcdt)
+    d_conv = conv_w.shape[1]
+    if tuple(dzxbcdt.shape) != (Bsz, L, E) or dzxbcdt.dtype != dtype or _row_stride(dzxbcdt) != ld:
+        raise ValueError("dzxbcdt must have zxbcdt's shape, dtype and row stride")
+    ssd._require(conv_w, "conv_w", (C, d_conv), torch.float32)
+    ssd._require(conv_b, "conv_b", (C,), torch.float32)
+    ssd._require(dt_bias, "dt_bias", (H,), torch.float32)
+    ssd._require(dx, "dx", (Bsz, L, H, P), dtype)
+    ssd._require(dB, "dB", (Bsz, L, G, N), dtype)
+    ssd._require(dC, "dC", (Bsz, L, G, N), dtype)
+    ssd._require(ddt, "ddt", (Bsz, L, H), dtype)
+    for name, t in (("conv_state", conv_state), ("dconv_state_out", dconv_state_out)):
+        if t is not None:
+            ssd._require(t, name, (Bsz, d_conv - 1, C), dtype)
+    if reset is not None:
+        if reset.dtype == torch.bool:
+            reset = reset.view(torch.uint8)
+        ssd._require(reset, "reset", (Bsz, L), torch.uint8)
+    dev = zxbcdt.device
+    dconv_w = torch.empty((C, d_conv), dtype=torch.float32, device=dev)
+    dconv_b = torch.empty(C, dtype=torch.float32, device=dev)
+    ddt_bias = torch.empty(H, dtype=torch.float32, device=dev)
+    dstate = torch.empty((Bsz, d_conv - 1, C), dtype=dtype, device=dev) if need_dconv_state else None
+    if workspace is None:
+        workspace = block_bwd_workspace(Bsz, L, H, P, N, G, d_conv, dtype, dev)
+    dims = SsdBlockDims(Bsz, L, H, P, N, G, d_conv, ld)
+    ssd._check(lib, lib.ssd_block_pre_bwd(byref(dims), code, zxbcdt.data_ptr(), conv_w.data_ptr(), conv_b.data_ptr(),
+                                          dt_bias.data_ptr(), ssd._ptr(conv_state), ssd._ptr(reset), dx.data_ptr(),
+                                          dB.data_ptr(), dC.data_ptr(), ddt.data_ptr(), ssd._ptr(dconv_state_out),
+                                          dzxbcdt.data_ptr(), dconv_w.data_ptr(), dconv_b.data_ptr(), ddt_bias.data_ptr(),
+                                          ssd._ptr(dstate), workspace.data_ptr(), workspace.numel(),
+                                          ssd._stream_ptr(zxbcdt)))
+    return dconv_w, dconv_b, ddt_bias, dstate
+
+
 def block_proj_supported(u: torch.Tensor, weight: torch.Tensor) -> bool:
     """Whether `block_proj` takes this product (else the caller's BLAS does it)."""
     return (u.is_cuda and u.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and u.shape[-1] in (128, 256)
@@ -217,11 +306,12 @@ class Mamba2Block:
         return Mamba2StreamState(conv, SsdStreamState.build(batch, self.H, self.P, self.N, device=self.in_proj.device))
 
     def forward(self, u: torch.Tensor, state: Optional[Mamba2StreamState] = None,
-                reset: Optional[torch.Tensor] = None) -> torch.Tensor:
+                reset: Optional[torch.Tensor] = None, save_for_backward: bool = False):
         """u [B,L,d_model] -> [B,L,d_model].  With `state`, continues from it and leaves it at the end of the
         window (a prefix scan; then `step` per bar).  `reset` [B,L]: episode boundaries inside the window -- a
         non-zero entry restarts both the SSM state and the conv's history before that timestep, exactly what
-        `Mamba2StreamState.reset_rows` does between two steps of a stream."""
+        `Mamba2StreamState.reset_rows` does between two steps of a stream.  With `save_for_backward` (windows
+        without a carried state) returns (out, ctx) for `backward`."""
         if u.dim() != 3 or u.shape[2] != self.d_model:
             raise ValueError(f"block input must be [batch, seqlen, {self.d_model}], got {tuple(u.shape)}")
         if reset is not None and state is not None:
@@ -238,7 +328,41 @@ class Mamba2Block:
             state.conv = conv
             y = state.ssm.init_from_prefix(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk)
         yn = block_post(y, zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
-        return self._project(yn, self.out_proj)
+        out = self._project(yn, self.out_proj)
+        if save_for_backward:
+            if state is not None:
+                raise ValueError("backward through a window that continues a carried state is not supported")
+            return out, dict(u=u, zxbcdt=zxbcdt, x=x, Bm=Bm, Cm=Cm, dt=dt, y=y, yn=yn, reset=reset)
+        return out
+
+    def backward(self, ctx: dict, dout: torch.Tensor) -> dict:
+        """Gradients of sum(out * dout) with respect to the input and every parameter, from the tensors `forward`
+        kept: two GEMMs per projection (torch), the library's post, scan and pre backward kernels between them.
+        Returns du [B,L,d_model] and float32 din_proj, dconv_w, dconv_b, ddt_bias, dA, dA_log, dD, dnorm_w, dout_proj."""
+        u, zxbcdt, y, yn, reset = ctx["u"], ctx["zxbcdt"], ctx["y"], ctx["yn"], ctx["reset"]
+        x, Bm, Cm, dt = ctx["x"], ctx["Bm"], ctx["Cm"], ctx["dt"]
+        Bsz, L, _ = u.shape
+        act = u.dtype
+        E = in_proj_width(self.H, self.P, self.N, self.G)
+        w_out = self.out_proj.to(act)
+        dout2 = dout.reshape(Bsz * L, self.d_model)
+        dyn = torch.matmul(dout2, w_out).view(Bsz, L, self.d_inner)
+        dout_proj = torch.matmul(dout2.t(), yn.reshape(Bsz * L, self.d_inner)).float()
+        # the gradient of zxbcdt, with zxbcdt's own (padded) row stride
+        ld = _row_stride(zxbcdt)
+        dbuf = torch.empty((Bsz, L, ld), dtype=act, device=u.device)
+        dzx = dbuf[..., :E] if ld != E else dbuf
+        ws = block_bwd_workspace(Bsz, L, self.H, self.P, self.N, self.G, self.d_conv, act, u.device)
+        dy, dnorm_w = block_post_bwd(y, zxbcdt, self.norm_w, dyn, dzx, self.H, self.P, self.N, self.G, self.eps, workspace=ws)
+        g = ssd.ssd_chunk_scan_backward(x, dt, self.A, Bm, Cm, self.D, dy, chunk=self.chunk, reset=reset)
+        dconv_w, dconv_b, ddt_bias, _ = block_pre_bwd(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, g["dx"], g["dB"],
+                                                      g["dC"], g["ddt"], dzx, self.H, self.P, self.N, self.G, reset=reset,
+                                                      workspace=ws)
+        dz2 = dbuf.view(Bsz * L, ld)[:, :E]
+        du = torch.matmul(dz2, self.in_proj.to(act)).view(Bsz, L, self.d_model)
+        din_proj = torch.matmul(dz2.t(), u.reshape(Bsz * L, self.d_model)).float()
+        return dict(du=du, din_proj=din_proj, dconv_w=dconv_w, dconv_b=dconv_b, ddt_bias=ddt_bias, dA=g["dA"],
+                    dA_log=g["dA"] * self.A, dD=g["dD"], dnorm_w=dnorm_w, dout_proj=dout_proj)
 
     def _project(self, u: torch.Tensor, weight: torch.Tensor, pad_rows: bool = False) -> torch.Tensor:
         """u . weight^T in the activation dtype: the library's kernel where it takes the shape (bf16, in_features 128

@@ -845,6 +845,68 @@ int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, 
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block projection launch");
 }
 
+int ssd_block_bwd_workspace_bytes(const ssd_block_dims *dims, int dtype, size_t *out_bytes) {
+    if (out_bytes == nullptr) return fail(SSD_ERR_INVALID, "ssd: out_bytes must not be NULL");
+    ssd::BlockShape s;
+    if (int rc = make_block_shape(dims, dtype, &s)) return rc;
+    *out_bytes = align_up(ssd::block_bwd_workspace_bytes(s), 256);
+    return SSD_OK;
+}
+
+int ssd_block_post_bwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                       float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *workspace,
+                       size_t workspace_bytes, void *hip_stream) {
+    ssd::BlockShape s;
+    if (int rc = make_block_shape(dims, dtype, &s)) return rc;
+    REQUIRE_PTR(y);
+    REQUIRE_PTR(zxbcdt);
+    REQUIRE_PTR(norm_w);
+    REQUIRE_PTR(dout);
+    REQUIRE_PTR(dy);
+    REQUIRE_PTR(dzxbcdt);
+    REQUIRE_PTR(dnorm_w);
+    REQUIRE_PTR(workspace);
+    if (!(eps > 0.f)) return fail(SSD_ERR_INVALID, "ssd: eps must be positive");
+    const size_t need = ssd::block_bwd_workspace_bytes(s);
+    if (workspace_bytes < need)
+        return fail(SSD_ERR_WORKSPACE, "ssd: block backward workspace has %zu bytes, %zu needed", workspace_bytes, need);
+    hipError_t e = ssd::launch_block_post_bwd(s, dtype, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, workspace,
+                                              (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "block post-scan backward launch");
+}
+
+int ssd_block_pre_bwd(const ssd_block_dims *dims, int dtype, const void *zxbcdt, const float *conv_w, const float *conv_b,
+                      const float *dt_bias, const void *conv_state_in, const uint8_t *reset, const void *dx, const void *dB,
+                      const void *dC, const void *ddt, const void *dconv_state_out, void *dzxbcdt, float *dconv_w,
+                      float *dconv_b, float *ddt_bias, void *dconv_state_in, void *workspace, size_t workspace_bytes,
+                      void *hip_stream) {
+    ssd::BlockShape s;
+    if (int rc = make_block_shape(dims, dtype, &s)) return rc;
+    REQUIRE_PTR(zxbcdt);
+    REQUIRE_PTR(conv_w);
+    REQUIRE_PTR(conv_b);
+    REQUIRE_PTR(dt_bias);
+    REQUIRE_PTR(dx);
+    REQUIRE_PTR(dB);
+    REQUIRE_PTR(dC);
+    REQUIRE_PTR(ddt);
+    REQUIRE_PTR(dzxbcdt);
+    REQUIRE_PTR(dconv_w);
+    REQUIRE_PTR(dconv_b);
+    REQUIRE_PTR(ddt_bias);
+    REQUIRE_PTR(workspace);
+    OPTIONAL_PTR(conv_state_in);
+    OPTIONAL_PTR(dconv_state_out);
+    OPTIONAL_PTR(dconv_state_in);
+    const size_t need = ssd::block_bwd_workspace_bytes(s);
+    if (workspace_bytes < need)
+        return fail(SSD_ERR_WORKSPACE, "ssd: block backward workspace has %zu bytes, %zu needed", workspace_bytes, need);
+    hipError_t e = ssd::launch_block_pre_bwd(s, dtype == SSD_DTYPE_F32 ? 0 : 1, zxbcdt, conv_w, conv_b, dt_bias, conv_state_in,
+                                             reset, dx, dB, dC, ddt, dconv_state_out, dzxbcdt, dconv_w, dconv_b, ddt_bias,
+                                             dconv_state_in, workspace, (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "block pre-scan backward launch");
+}
+
 int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,
                        const float *norm_w, float eps, void *out, void *hip_stream) {
     ssd::BlockShape s;

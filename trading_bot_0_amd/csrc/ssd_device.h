@@ -270,6 +270,65 @@ template <> __device__ inline void store_column<float>(float *yrow, float (&o)[1
     }
 }
 
+// The same through a buffer descriptor: rows that must not be written get an offset beyond the descriptor's range
+// and the hardware drops their stores, so the stores themselves are unconditional -- no branch around them.
+// byte_off addresses element p = 0 of the column's row, relative to the descriptor's base; all offsets of a
+// descriptor stay below 2^31.
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+constexpr unsigned kBufferDropOffset = 0x80000000u;
+__device__ inline __amdgpu_buffer_rsrc_t make_buffer(const void *base, unsigned bytes) {
+    // raw buffer, stride 0, range-checked: dword 3 = the 32-bit data format of gfx9-family descriptors
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+// One column's 32 outputs packed for the store, and where they go.
+template <typename TO> struct PackedColumn {
+    static constexpr int NV = sizeof(TO) == 2 ? 2 : 4;
+    u32x4 v[NV];
+    unsigned off = kBufferDropOffset;  // (nothing packed yet: emitting it writes nothing)
+};
+template <typename TO>
+__device__ inline void pack_column(PackedColumn<TO> &pc, unsigned byte_off, float (&o)[16], int half, bool row_ok);
+template <>
+__device__ inline void pack_column<__bf16>(PackedColumn<__bf16> &pc, unsigned byte_off, float (&o)[16], int half, bool row_ok) {
+    unsigned X[4], Y[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        X[k] = pack_bf16x2(o[2 * k], o[2 * k + 1]);
+        Y[k] = pack_bf16x2(o[8 + 2 * k], o[8 + 2 * k + 1]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) swap_halves(X[k], Y[k]);
+    pc.off = row_ok ? byte_off + 32u * half : kBufferDropOffset;
+    pc.v[0] = u32x4{X[0], X[1], Y[0], Y[1]};
+    pc.v[1] = u32x4{X[2], X[3], Y[2], Y[3]};
+}
+template <>
+__device__ inline void pack_column<float>(PackedColumn<float> &pc, unsigned byte_off, float (&o)[16], int half, bool row_ok) {
+    unsigned X[8], Y[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        X[k] = __float_as_uint(o[k]);
+        Y[k] = __float_as_uint(o[8 + k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) swap_halves(X[k], Y[k]);
+    pc.off = row_ok ? byte_off + 64u * half : kBufferDropOffset;
+    pc.v[0] = u32x4{X[0], X[1], X[2], X[3]};
+    pc.v[1] = u32x4{Y[0], Y[1], Y[2], Y[3]};
+    pc.v[2] = u32x4{X[4], X[5], X[6], X[7]};
+    pc.v[3] = u32x4{Y[4], Y[5], Y[6], Y[7]};
+}
+template <typename TO> __device__ inline void emit_column(__amdgpu_buffer_rsrc_t rs, const PackedColumn<TO> &pc) {
+#pragma unroll
+    for (int i = 0; i < PackedColumn<TO>::NV; ++i) __builtin_amdgcn_raw_buffer_store_b128(pc.v[i], rs, pc.off + 16u * i, 0, 0);
+}
+template <typename TO>
+__device__ inline void store_column_buffer(__amdgpu_buffer_rsrc_t rs, unsigned byte_off, float (&o)[16], int half, bool row_ok) {
+    PackedColumn<TO> pc;
+    pack_column<TO>(pc, byte_off, o, half, row_ok);
+    emit_column<TO>(rs, pc);
+}
+
 // hi + lo bf16 pairs of two products a0*f0 and a1*f1 (f = 1 to split plain values): hi is the product
 // rounded to bf16, lo the rounded remainder m - hi, which is exact in float before its own rounding.
 // The remainder takes one v_dot2c_f32_bf16 per element, m + (-1)*half + 0*other half, which reads the half

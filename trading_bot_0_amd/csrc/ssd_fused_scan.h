@@ -241,7 +241,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     const int dt_rows = ADJ ? s.dt_len : s.L;
     const T *dtb = dt + (size_t)b * dt_rows * s.H + h;
     const unsigned char *rsb = reset ? reset + (size_t)b * dt_rows : nullptr;  // state restarts, see kResetLog2
-    TO *yb = y + (size_t)b * trows * HP + h * s.P + pb * 32;
+    // this batch row's y as a range-checked buffer (the launchers keep a row below 2^31 bytes): the epilogue's stores
+    // go through it, so rows outside the sequence are dropped by the hardware instead of branched around
+    const __amdgpu_buffer_rsrc_t ybuf = make_buffer(y + (size_t)b * trows * HP, (unsigned)((size_t)trows * HP * sizeof(TO)));
+    const unsigned ycol_bytes = (unsigned)((h * s.P + pb * 32) * sizeof(TO));
     const float dh = D ? D[h] : 0.f;
     const double a_h = (double)A[h];
 
@@ -781,7 +784,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     pd += __shfl_xor(pd, 32, 64);
                     const int yrow = s.L - 1 - (t0 + ll);
                     const bool live = ll < rows && yrow >= 0 && yrow < trows;
-                    store_column<TO>(yb + (size_t)yrow * HP, o, he, 32, live);
+                    store_column_buffer<TO>(ybuf, (unsigned)yrow * (unsigned)(HP * sizeof(TO)) + ycol_bytes, o, he, live);
                     if (he == 0 && live)
                         *reinterpret_cast<float2 *>(seg_decay + 2 * (((size_t)b * trows + yrow) * s.H + h)) = make_float2(pe, pd);
                 } else {
@@ -795,7 +798,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                         for (int i = 0; i < 4; ++i) o[vg * 4 + i] = acc[vg * 4 + i] + dh * (float)x4[i];
                     }
                     const int yrow = ADJ ? s.L - 1 - (t0 + ll) : t0 + ll;
-                    store_column<TO>(yb + (size_t)yrow * HP, o, he, 32, ll < rows && (!ADJ || (yrow >= 0 && yrow < trows)));
+                    store_column_buffer<TO>(ybuf, (unsigned)yrow * (unsigned)(HP * sizeof(TO)) + ycol_bytes, o, he,
+                                            ll < rows && (!ADJ || (yrow >= 0 && yrow < trows)));
                 }
             }
         }

@@ -17,6 +17,8 @@ int fused_scan_waves(const ScanShape &s, int dtype) {
     if (s.N == 128) waves = (units % 4 == 0) ? 4 : 0;
     if (waves == 0 && units % 2 == 0 && s.N == 32 && dtype == 2) waves = 2;  // float y only: the backward's scans
     if (waves == 0 || fused_scan_lds_bytes(s.N, kOnePassTile, waves) > kLdsLimitBytes) return 0;
+    // the kernel writes a batch row's y through a 32-bit-offset buffer descriptor
+    if ((long long)(s.L > s.dt_len ? s.L : s.dt_len) * s.H * s.P * 4 >= (1LL << 31)) return 0;
     return waves;
 }
 

@@ -117,6 +117,19 @@ hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, 
 hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                              float eps, void *out, hipStream_t stream);
 
+// Backward of the two stages (dtype as the forward's; dtype 2 = bf16 activations with the scan's float32 y in
+// post_bwd).  dzxbcdt [B,L,ld] is the gradient of zxbcdt: post_bwd writes its z channels, pre_bwd its x | B | C | dt
+// channels.  workspace: block_bwd_workspace_bytes (partial sums of the parameter gradients).
+size_t block_bwd_workspace_bytes(const BlockShape &s);
+hipError_t launch_block_post_bwd(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                                 float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *workspace,
+                                 hipStream_t stream);
+hipError_t launch_block_pre_bwd(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w, const float *conv_b,
+                                const float *dt_bias, const void *state_in, const unsigned char *reset, const void *dx,
+                                const void *dB, const void *dC, const void *ddt, const void *dstate_out, void *dzxbcdt,
+                                float *dconv_w, float *dconv_b, float *ddt_bias, void *dstate_in, void *workspace,
+                                hipStream_t stream);
+
 // The backward pass's two scans of the transposed state with the sum over a group's heads taken on chip (bf16,
 // headdim 32, eight heads per group; sT is the transposed shape: P = dstate, N = 32, G = H; sT.mode / dt_len as
 // for the one-pass kernel when adjoint).  x [B,L,x_groups,P] is the operand a group's heads share, Bm and Cm

@@ -49,6 +49,9 @@ EXPORTED_SYMBOLS = (
     "ssd_chunk_scan_bwd",
     "ssd_chunk_scan_noalloc_fwd",
     "ssd_block_pre_reset_fwd",
+    "ssd_block_bwd_workspace_bytes",
+    "ssd_block_post_bwd",
+    "ssd_block_pre_bwd",
 )
 
 
