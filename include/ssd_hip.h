@@ -210,8 +210,8 @@ int ssd_steps_fwd(const ssd_step_dims *dims, int64_t nsteps, int dtype, float *s
  * optionally dfinal_states [B,H,P,N] (NULL if the final state does not reach the loss).
  * Out: dx [B,L,H,P], ddt [B,L,H], dA [H], dB, dC [B,L,G,N], dD [H] (NULL allowed; must be NULL without D),
  * dinitial_states [B,H,P,N] (NULL allowed; defined also when the forward had no initial state).
- * dstate <= 64 and headdim 16, 32 or 64 (the pass runs the forward's kernels on the transposed state);
- * other shapes return SSD_ERR_UNSUPPORTED.  Workspace size from ssd_chunk_scan_bwd_workspace_bytes. */
+ * headdim 16, 32 or 64 (the pass runs the forward's kernels on the transposed state, a 128-wide state in two parts of
+ * 64 rows); other shapes return SSD_ERR_UNSUPPORTED.  Workspace size from ssd_chunk_scan_bwd_workspace_bytes. */
 int ssd_chunk_scan_bwd_workspace_bytes(const ssd_dims *dims, int dtype, size_t *out_bytes);
 int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A, const void *Bm,
                        const void *Cm, const float *D, const float *initial_states, const uint8_t *reset, const void *dy,

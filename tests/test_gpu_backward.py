@@ -64,6 +64,8 @@ SHAPES = [
     Workload("bwd_per_head_bc", 2, 256, 4, 64, 32, 4, 32, init_std=0.5),
     Workload("bwd_tiny_state", 2, 130, 2, 16, 64, 1, 64, init_std=0.5),
     Workload("bwd_three_heads_per_group", 2, 100, 6, 32, 32, 2, 64, init_std=0.5),   # group sums in their own kernel
+    Workload("bwd_long_lookback_heads", 2, 200, 16, 64, 128, 2, 64, init_std=0.3),    # a 128-wide state: scanned in two parts
+    Workload("bwd_wide_state_small_heads", 2, 150, 4, 32, 128, 1, 64, init_std=0.3),
 ]
 
 
@@ -126,11 +128,11 @@ def test_directional_derivative_of_the_gpu_forward():
 
 
 def test_unsupported_shapes_are_refused():
-    w = Workload("bwd_big_state", 1, 64, 2, 32, 128, 1, 64, dtype="bf16")
+    w = Workload("bwd_narrow_heads", 1, 64, 4, 8, 64, 1, 64, dtype="bf16")
     dev = to_dev(make_inputs(w, seed=0))
     with pytest.raises(SsdError) as e:
         ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], torch.zeros_like(dev["x"]), chunk=64)
-    assert "dstate <= 64" in str(e.value)
+    assert "headdim 16, 32 or 64" in str(e.value)
     w = Workload("bwd_ok", 1, 64, 2, 32, 64, 1, 64, dtype="bf16")
     dev = to_dev(make_inputs(w, seed=0))
     with pytest.raises(ValueError):

@@ -57,14 +57,16 @@ def test_random_shape(case):
         y_ref, f_ref = orc.ssd_sequential(np64(sub["x"]), np64(sub["dt"]), np64(sub["A"]), np64(sub["B"]), np64(sub["C"]),
                                           np64(sub["D"]), np64(sub["init"]), reset=mask[rows])
     assert rel_err(y[rows], y_ref) <= tol and rel_err(fin[rows], f_ref) <= tol, f"{w}"
-    if w.dstate > 64:
-        return   # the backward pass takes no dstate above 64
     g = torch.Generator().manual_seed(case + 1000)
     dy = torch.randn(cpu["x"].shape, generator=g).to(w.torch_dtype)
     dfin = torch.randn(w.batch, w.nheads, w.headdim, w.dstate, generator=g) if with_dfinal else None
-    got = ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], dy.cuda(), chunk=w.chunk,
-                                  initial_states=dev["init"], dfinal_states=None if dfin is None else dfin.cuda(),
-                                  need_dinitial_states=True, reset=reset)
+    try:
+        got = ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], dy.cuda(), chunk=w.chunk,
+                                      initial_states=dev["init"], dfinal_states=None if dfin is None else dfin.cuda(),
+                                      need_dinitial_states=True, reset=reset)
+    except SsdError as e:   # as for the forward: float32 tiles of the largest head sizes do not fit the LDS
+        assert e.code == 2 and w.dtype == "f32", str(e)
+        return
     torch.cuda.synchronize()
     ref = bwd.ssd_backward_sequential(np64(sub["x"]), np64(sub["dt"]), np64(sub["A"]), np64(sub["B"]), np64(sub["C"]),
                                       np64(sub["D"]), np64(sub["init"]), np64(dy[rows]),

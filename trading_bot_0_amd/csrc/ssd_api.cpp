@@ -182,7 +182,7 @@ int run_staged(const ssd::ScanShape &s, int dtype, const void *x, const void *dt
 // array), the gathered operands (reversed ones padded to whole chunks) and the scans' float outputs.
 struct BwdWorkspace {
     size_t scan_off, states2, dy_rev, x_rev, c_rev_g, b_rev_g, c_rev_h, b_fwd_h, r_rev, yb_rev, yc, gfin, gfin_t, ffin_t,
-        init_t, dfin_t, e1, dd, u, parts, anchor, da_part, total;
+        init_t, dfin_t, e1, dd, u, parts, anchor, da_part, dt_parts, a_parts, total;
 };
 
 // Which kernels a backward pass of a given shape runs on (a function of shape and dtype only: the workspace is laid
@@ -215,7 +215,7 @@ BwdPlan plan_bwd(const ssd::ScanShape &s, const ssd::ScanShape &sT, int dtype) {
     return p;
 }
 
-BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes, const BwdPlan &plan) {
+BwdWorkspace carve_bwd(const ssd::ScanShape &s, const ssd::ScanShape &sT, int elem_bytes, const BwdPlan &plan) {
     BwdWorkspace w;
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -227,7 +227,8 @@ BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes, const BwdPlan &p
     const size_t BL = (size_t)s.B * s.L, BLp = (size_t)s.B * s.nc * s.Q;  // true and padded rows
     const size_t HP = (size_t)s.H * s.P, HN = (size_t)s.H * s.N, GN = (size_t)s.G * s.N;
     const size_t st = (size_t)s.B * s.H * s.P * s.N * sizeof(float);
-    w.scan_off = take(carve(s).total);
+    // (the transposed scans of a 128-wide state run on twice the heads: more stage-1 rows, the same state elements)
+    w.scan_off = take(sT.H > s.H ? carve(sT).total : carve(s).total);
     w.states2 = take_if(!plan.sum_on_chip, (size_t)s.nc * st);
     w.dy_rev = take_if(!plan.fast_r || !plan.fast_t, BLp * HP * elem_bytes);
     w.x_rev = take_if(!plan.fast_t, BLp * HP * elem_bytes);
@@ -249,6 +250,9 @@ BwdWorkspace carve_bwd(const ssd::ScanShape &s, int elem_bytes, const BwdPlan &p
     w.parts = take(BL * s.H * (size_t)((s.N + 31) / 32) * sizeof(float));
     w.anchor = take((size_t)s.B * (s.nc + 1) * s.H * sizeof(double) * (size_t)((s.N + 31) / 32));  // or its pieces
     w.da_part = take((size_t)2 * s.B * s.nc * s.H * sizeof(double));  // and the parts of dD behind them
+    // dt and A once per part of a head, for the transposed scans of a state scanned in parts
+    w.dt_parts = take_if(sT.H > s.H, BL * sT.H * elem_bytes);
+    w.a_parts = take_if(sT.H > s.H, (size_t)sT.H * sizeof(float));
     w.total = off;
     return w;
 }
@@ -266,11 +270,14 @@ int make_bwd_shapes(const ssd_dims *dims, int dtype, ssd::ScanShape *s, ssd::Sca
     ssd_dims own = *dims;
     if (own.chunk > kBackwardChunk) own.chunk = kBackwardChunk;
     if (int rc = make_shape(&own, dtype, s)) return rc;
-    if (dims->dstate > 64 || dims->headdim < 16 || (dims->headdim & (dims->headdim - 1)) != 0)
-        return fail(SSD_ERR_UNSUPPORTED,
-                    "ssd: the backward pass needs dstate <= 64 and headdim 16, 32 or 64, got %lld and %lld",
-                    (long long)dims->dstate, (long long)dims->headdim);
-    const ssd_dims t = {dims->batch, dims->seqlen, dims->nheads, dims->dstate, dims->headdim, dims->nheads, own.chunk};
+    if (dims->headdim < 16 || (dims->headdim & (dims->headdim - 1)) != 0)
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: the backward pass needs headdim 16, 32 or 64, got %lld", (long long)dims->headdim);
+    // The transposed state is [dstate, headdim] per head, and the stage kernels take a head-dim of at most 64: a
+    // 128-wide state is scanned as two parts of 64 rows, i.e. as twice as many heads in groups of two that share
+    // their B and C operands -- the same memory, read as [.., 2 nheads, 64, ..].
+    const int64_t parts = dims->dstate > 64 ? 2 : 1;
+    const ssd_dims t = {dims->batch, dims->seqlen, dims->nheads * parts, dims->dstate / parts, dims->headdim, dims->nheads,
+                        own.chunk};
     return make_shape(&t, dtype, sT);
 }
 
@@ -478,7 +485,7 @@ int ssd_chunk_scan_bwd_workspace_bytes(const ssd_dims *dims, int dtype, size_t *
     if (out_bytes == nullptr) return fail(SSD_ERR_INVALID, "ssd: out_bytes must not be NULL");
     ssd::ScanShape s, sT;
     if (int rc = make_bwd_shapes(dims, dtype, &s, &sT)) return rc;
-    *out_bytes = carve_bwd(s, dtype == SSD_DTYPE_F32 ? 4 : 2, plan_bwd(s, sT, dtype)).total;
+    *out_bytes = carve_bwd(s, sT, dtype == SSD_DTYPE_F32 ? 4 : 2, plan_bwd(s, sT, dtype)).total;
     return SSD_OK;
 }
 
@@ -508,13 +515,13 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     if (dD != nullptr && D == nullptr) return fail(SSD_ERR_INVALID, "ssd: dD asked for without D");
     const int eb = dtype == SSD_DTYPE_F32 ? 4 : 2;
     const BwdPlan plan = plan_bwd(s, sT, dtype);
-    const BwdWorkspace w = carve_bwd(s, eb, plan);
+    const BwdWorkspace w = carve_bwd(s, sT, eb, plan);
     if (workspace_bytes < w.total)
         return fail(SSD_ERR_WORKSPACE, "ssd: backward workspace has %zu bytes, %zu needed", workspace_bytes, w.total);
     char *base = static_cast<char *>(workspace);
     auto at = [&](size_t off) { return static_cast<void *>(base + off); };
     auto atf = [&](size_t off) { return reinterpret_cast<float *>(base + off); };
-    const Workspace sw = carve(s);
+    const Workspace sw = sT.H > s.H ? carve(sT) : carve(s);
     float *dtcs = atf(w.scan_off + sw.dtcs_off), *states = atf(w.scan_off + sw.st_off);
     hipStream_t st = (hipStream_t)hip_stream;
     const int inner = dtype == SSD_DTYPE_F32 ? SSD_DTYPE_F32 : SSD_DTYPE_BF16_Y32;  // the scans write float y
@@ -563,17 +570,24 @@ int ssd_chunk_scan_bwd(const ssd_dims *dims, int dtype, const void *x, const voi
     }
     auto scan = [&](const ssd::ScanShape &shape, bool fast, const void *sx, const void *sb, const void *sc, const float *sinit,
                     int mode, void *sy, float *sfinal, float *sstates, bool keep_states, int x_groups) -> int {
+        // a state scanned in parts: dt and A once per part of a head
+        const void *sdt = shape.H > s.H ? at(w.dt_parts) : dt;
+        const float *sA = shape.H > s.H ? atf(w.a_parts) : A;
         if (fast) {
             ssd::ScanShape f = shape;
             f.mode = mode;
             f.dt_len = s.L;
             f.x_groups = x_groups;
-            hipError_t err = ssd::launch_fused_scan(f, inner, sx, dt, A, sb, sc, nullptr, sinit, reset, sy, sfinal, st,
+            hipError_t err = ssd::launch_fused_scan(f, inner, sx, sdt, sA, sb, sc, nullptr, sinit, reset, sy, sfinal, st,
                                                      keep_states ? sstates : nullptr);
             return err == hipSuccess ? SSD_OK : hip_fail(err, "one-pass scan launch (backward)");
         }
-        return run_staged(shape, inner, sx, dt, A, sb, sc, nullptr, sinit, reset, mode, sy, sfinal, dtcs, sstates, st, s.L);
+        return run_staged(shape, inner, sx, sdt, sA, sb, sc, nullptr, sinit, reset, mode, sy, sfinal, dtcs, sstates, st, s.L);
     };
+    if (sT.H > s.H) {
+        BWD_LAUNCH(ssd::launch_replicate_columns(el, dt, at(w.dt_parts), (long long)s.B * s.L, s.H, sT.H / s.H, st), "dt per part");
+        BWD_LAUNCH(ssd::launch_replicate_columns(0, A, at(w.a_parts), 1, s.H, sT.H / s.H, st), "A per part");
+    }
     // r = g B: the adjoint recurrence, reversed in time; its last state is g_0
     if (rows_in_scan) {
         ssd::ScanShape f = sR;

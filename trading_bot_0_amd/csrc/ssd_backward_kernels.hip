@@ -128,39 +128,43 @@ __global__ __launch_bounds__(256) void bwd_rows_kernel(const T *__restrict__ x, 
         }
         o.store(dx + row);
     }
-    Row8<float> sb, sy;  // this head's dt yB and yC pieces
+    // the state columns, 64 per pass of the row's eight lanes (dstate 128: two passes)
+    for (int n0 = 0; n0 < s.N; n0 += 64) {
+        const int np = n0 + piece;
+        Row8<float> sb, sy;  // this head's dt yB and yC pieces
 #pragma unroll
-    for (int i = 0; i < 8; ++i) sb.v[i] = sy.v[i] = 0.f;
-    if (piece < s.N) {
-        const Row8<T> cv = Row8<T>::load(Cm + ((size_t)bt * s.G + g) * s.N + piece);
-        sy = Row8<float>::load(yC + (size_t)gid * s.N + piece);
+        for (int i = 0; i < 8; ++i) sb.v[i] = sy.v[i] = 0.f;
+        if (np < s.N) {
+            const Row8<T> cv = Row8<T>::load(Cm + ((size_t)bt * s.G + g) * s.N + np);
+            sy = Row8<float>::load(yC + (size_t)gid * s.N + np);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) sc += cv.v[i] * sy.v[i];
+            for (int i = 0; i < 8; ++i) sc += cv.v[i] * sy.v[i];
+            if (SUMS) {
+                const size_t brow = LrevB ? (size_t)(b * LrevB + (LrevB - 1 - t)) : (size_t)bt;
+                sb = Row8<float>::load(yB_rev + (brow * s.H + h) * s.N + np);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sb.v[i] *= dtv;
+            }
+        }
         if (SUMS) {
-            const size_t brow = LrevB ? (size_t)(b * LrevB + (LrevB - 1 - t)) : (size_t)bt;
-            sb = Row8<float>::load(yB_rev + (brow * s.H + h) * s.N + piece);
+            const int hpg = s.H / s.G;
+            for (int m = 8; m < 8 * hpg; m <<= 1) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) sb.v[i] *= dtv;
-        }
-    }
-    if (SUMS) {
-        const int hpg = s.H / s.G;
-        for (int m = 8; m < 8 * hpg; m <<= 1) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                sb.v[i] += __shfl_xor(sb.v[i], m, 64);
-                sy.v[i] += __shfl_xor(sy.v[i], m, 64);
+                for (int i = 0; i < 8; ++i) {
+                    sb.v[i] += __shfl_xor(sb.v[i], m, 64);
+                    sy.v[i] += __shfl_xor(sy.v[i], m, 64);
+                }
             }
-        }
-        if (h % hpg == 0 && piece < s.N) {
-            Row8<T> ob, oc;
+            if (h % hpg == 0 && np < s.N) {
+                Row8<T> ob, oc;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                ob.v[i] = sb.v[i];
-                oc.v[i] = sy.v[i];
+                for (int i = 0; i < 8; ++i) {
+                    ob.v[i] = sb.v[i];
+                    oc.v[i] = sy.v[i];
+                }
+                ob.store(dB + ((size_t)bt * s.G + g) * s.N + np);
+                oc.store(dC + ((size_t)bt * s.G + g) * s.N + np);
             }
-            ob.store(dB + ((size_t)bt * s.G + g) * s.N + piece);
-            oc.store(dC + ((size_t)bt * s.G + g) * s.N + piece);
         }
     }
 #pragma unroll
@@ -519,6 +523,18 @@ hipError_t gather_t(const void *src, void *dst, int B, int Lsrc, int L, int grou
     return hipGetLastError();
 }
 
+// out[row, h * rep + k] = in[row, h] for k < rep: dt (and A, as one row) given once per part of a head whose state
+// dimension is scanned in `rep` parts
+template <typename T>
+__global__ __launch_bounds__(256) void replicate_columns_kernel(const T *__restrict__ in, T *__restrict__ out, int H, int rep,
+                                                                long long total) {
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const long long row = gid / (H * rep);
+    const int hk = (int)(gid % (H * rep));
+    out[gid] = in[row * H + hk / rep];
+}
+
 template <typename T>
 hipError_t rows_t(const ScanShape &s, int Lrev, const void *x, const void *dy, const void *dt, const void *Cm, const float *D,
                   const float *r_rev, const float *yC, void *dx, float *e1, float *dd, float *u, const float *yB_rev,
@@ -659,6 +675,17 @@ hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const
 hipError_t launch_bwd_dinit(const ScanShape &s, int dtype, const void *dt, const float *A, const float *gfin,
                             const unsigned char *reset, float *dinit, hipStream_t st) {
     return dtype ? dinit_t<__bf16>(s, dt, A, gfin, reset, dinit, st) : dinit_t<float>(s, dt, A, gfin, reset, dinit, st);
+}
+
+hipError_t launch_replicate_columns(int dtype, const void *in, void *out, long long rows, int H, int rep, hipStream_t st) {
+    const long long total = rows * H * rep;
+    if (dtype == 0)
+        replicate_columns_kernel<float><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(static_cast<const float *>(in),
+                                                                                     static_cast<float *>(out), H, rep, total);
+    else
+        replicate_columns_kernel<__bf16><<<dim3(blocks_for(total)), dim3(256), 0, st>>>(static_cast<const __bf16 *>(in),
+                                                                                      static_cast<__bf16 *>(out), H, rep, total);
+    return hipGetLastError();
 }
 
 }  // namespace ssd

@@ -167,6 +167,8 @@ hipError_t launch_adjoint_rows_scan(const ScanShape &sR, const void *dy, const v
 // else t'; rows with t >= Lsrc are zero.  W a multiple of 8.
 hipError_t launch_gather_rows(int dtype, const void *src, void *dst, int B, int Lsrc, int Ldst, int groups, int W,
                               int rep, bool reverse, hipStream_t stream);
+// out [rows, H*rep] = in [rows, H] with every column repeated rep times (dtype: 0 = float32, 1 = bf16)
+hipError_t launch_replicate_columns(int dtype, const void *in, void *out, long long rows, int H, int rep, hipStream_t stream);
 // [BH, P, N] -> [BH, N, P]
 hipError_t launch_transpose_state(const float *src, float *dst, long long BH, int P, int N, hipStream_t stream);
 // per (b,t,h): dx = D dy + dt r, e1 = x . r, dd = dy . x, u = C . yC - dt e1.  r_rev (and yB_rev below) hold
