@@ -40,19 +40,26 @@ namespace ssd {
 
 template <int COLS> struct ChunkTile {  // bf16 [rows][COLS], COLS = 32, 64 or 128
     static_assert(COLS == 32 || COLS == 64 || COLS == 128, "tile rows are 64, 128 or 256 bytes");
-    // XOR mask on the index of an 8-byte piece within its row.  32 consecutive rows map a fixed logical
-    // piece to 32 different bank pairs, and 4 consecutive rows (first one a multiple of 4) keep their
-    // 64-byte halves in different quarters of the banks.
+    // XOR mask on the index of an 8-byte piece within its row, chosen against what the LDS of this chip does
+    // (measured with a 16-wave probe): a plain 8-byte read is served 16 consecutive lanes at a time from 32 banks
+    // (128 bytes a cycle), the transposing read 32 lanes at a time from 64.  So for the 8-byte reads of one logical
+    // piece of 32 consecutive rows, any 16 consecutive rows must spread that piece over all 16 eight-byte positions
+    // of the 128-byte bank line, and for the transposing read (4 consecutive rows x 64 bytes per 32 lanes) the four
+    // rows must keep their 64-byte pieces in different quarters of 256 bytes.  Both reads then run at their full
+    // rate (4.2 and 2.3 cycles per wave-instruction; with the four-row rule alone the plain reads took 8).
     static __device__ inline int f(int row) {
         if constexpr (COLS == 32) {
-            return (row >> 2) & 7;
+            // 64-byte rows: two rows per bank line; rows of one parity need 8 different masks over 16 rows, and rows
+            // 0,1 against 2,3 of a group of four must differ in the 32-byte half
+            return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
         } else if constexpr (COLS == 128) {
-            // a row fills all banks: the row's low two bits pick the 64-byte quarter, the next three the piece
-            // within it (the staging writes of four rows then share bank pairs two by two)
-            return ((row & 3) << 3) | ((row >> 2) & 7);
+            // 256-byte rows: bits 3-4 of the piece index (the 64-byte quarter) from the row's low two bits, bits 0-3
+            // (the position in the bank line) a bijection of the row's low four bits
+            return (((row >> 1) & 1) << 4) | ((row & 1) << 3) | (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);
         } else {
-            const int v = (row >> 1) & 15;
-            return ((v & 1) << 3) | (v >> 1);
+            // 128-byte rows: one row per bank line; the 32-byte quarter from the row's low two bits, the piece within
+            // it from the next two
+            return ((row & 3) << 2) | ((row >> 2) & 3);
         }
     }
     static __device__ inline int off(int row, int col) {
