@@ -26,8 +26,11 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
   reference_suite  the reference's historical benchmark cases for this path (batch 4, seq_len 4096,
                BFloat16) in the reference's result schema: mamba2_* rows time this library's whole Mamba-2 block
                (sizes in each row's config), ssd_scan_* rows the scan op alone
-  forward_float32  the same workload with float32 inputs (the other parity mode): staged kernels on float MFMAs,
-               time per call and dense flops against the 157.3 TFLOP/s float MFMA peak, which binds it
+  forward_float32  the same workload with float32 inputs (the other parity mode): time per call, which path ran (the
+               float one-pass kernel on three bf16 terms per operand, or the staged kernels on float MFMAs), its
+               compulsory traffic against the HBM peak and the op's dense flops against the 157.3 TFLOP/s float MFMA
+               peak (the one-pass kernel multiplies on the bf16 matrix pipe, so that fraction may pass 1), and its
+               parity errors against the oracle on the first batch rows
   backward     the backward pass of the scan at the same shape: time per call, and its compulsory traffic
                (x, dt, B, C, dy read; dx, ddt, dB, dC written) against the HBM peak
   mamba2_block the block around the scan at the policy shape (d_model = nheads*headdim): whole block, and the
@@ -340,10 +343,34 @@ def main():
             spin(f32_call, torch)
             t32, _ = event_time_steps(f32_call, 20, torch)
             fl = sum(sf[k] for k in ("chunk_state", "chunk_scan"))   # dense MFMA flops of the op
-            out["forward_float32"] = {"ms": round(t32 * 1e3, 4), "path": "staged", "bound": "mfma (float32)",
+            f32_onepass = ssd.chunk_scan_is_onepass(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk,
+                                                    dtype=torch.float32)
+            io32 = 4 * (2 * w.batch * w.seqlen * w.nheads * w.headdim + w.batch * w.seqlen * w.nheads +
+                        2 * w.batch * w.seqlen * w.ngroups * w.dstate) + \
+                4 * w.batch * w.nheads * w.headdim * w.dstate * (2 if init is not None else 1)
+            y32o, f32o = f32_call()
+            torch.cuda.synchronize()
+            from oracle import c_oracle
+            from oracle import ssd_oracle as orc
+            nb_err = min(w.batch, 2)
+
+            def f64(t):
+                return None if t is None else t[:nb_err].cpu().numpy().astype(np.float64)
+
+            y_ref, f_ref = c_oracle.ssd_sequential_c(f64(x32), f64(dt32), A.cpu().numpy().astype(np.float64), f64(B32), f64(C32),
+                                                     None if D is None else D.cpu().numpy().astype(np.float64), f64(init),
+                                                     nthreads=min(16, os.cpu_count() or 1))
+            e32 = (orc.rel_err(y32o[:nb_err].cpu().numpy(), y_ref), orc.rel_err(f32o[:nb_err].cpu().numpy(), f_ref))
+            del y_ref, f_ref
+            out["forward_float32"] = {"ms": round(t32 * 1e3, 4),
+                                      "path": "one-pass (three bf16 terms per operand)" if f32_onepass else "staged",
+                                      "compulsory_io_bytes": io32,
+                                      "hbm_frac": round(io32 / t32 / 1e9 / HBM_PEAK_GBS, 4),
                                       "dense_TFLOPs": round(fl / t32 / 1e12, 1), "peak_TFLOPs": MFMA_F32_PEAK_TFLOPS,
                                       "mfma_frac": round(fl / t32 / 1e12 / MFMA_F32_PEAK_TFLOPS, 4),
-                                      "units_per_s": round(w.batch * w.seqlen / t32, 1)}
+                                      "units_per_s": round(w.batch * w.seqlen / t32, 1),
+                                      "err_y": e32[0], "err_final": e32[1], "tolerance": 1e-4}
+            del y32o, f32o
         del x32, dt32, B32, C32, f32_call
 
     # ---- the backward pass at the benchmark shape ------------------------------------------------------

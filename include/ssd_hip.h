@@ -112,14 +112,17 @@ int ssd_chunk_state_passing_fwd(const ssd_dims *dims, int dtype, const void *x, 
                                 const float *dtcs, const float *initial_states, float *prev_states,
                                 float *final_states, void *hip_stream);
 
-/* The whole forward in one kernel and one pass over the inputs (bf16 inputs only): a wave keeps the running
+/* The whole forward in one kernel and one pass over the inputs: a wave keeps the running
  * state of 32 head-dim columns of one (batch, head) in registers while it walks the chunks, so no workspace
  * is needed and nothing but x, dt, B, C is read and y, final_states written.  Same arguments (with the
  * optional reset mask of ssd_chunk_scan_reset_fwd) and results as ssd_chunk_scan_fwd.  Parallel over
- * (batch, head) sequences only; ssd_chunk_scan_fwd takes this path by itself when there are enough of them.  SSD_ERR_UNSUPPORTED unless dtype is bf16 (1 or 2), headdim is a
- * multiple of 32, dstate is 32, 64 or 128 and (nheads/ngroups)*(headdim/32) is a multiple of 4.  dims->chunk must
+ * (batch, head) sequences only; ssd_chunk_scan_fwd takes this path by itself when there are enough of them.  SSD_ERR_UNSUPPORTED unless headdim is a
+ * multiple of 32 and, for bf16 inputs (dtype 1 or 2), dstate is 32, 64 or 128 and (nheads/ngroups)*(headdim/32) a
+ * multiple of 4; for float32 inputs (every operand enters the matrix cores as three bf16 terms, six products per
+ * multiplication: float accuracy at three eighths of the float instruction's cost), dstate is 32 or 64 and
+ * (nheads/ngroups)*(headdim/32) a multiple of 8.  dims->chunk must
  * be a valid chunk length but does not enter: with no workspace layout to honour, the kernel tiles time by
- * its own block of 64 steps (results agree with every chunk length to rounding).  Replaces the same slot as ssd_chunk_scan_fwd (model/trading_model.rs:589-606). */
+ * its own block (64 steps, float32 inputs 32; results agree with every chunk length to rounding).  Replaces the same slot as ssd_chunk_scan_fwd (model/trading_model.rs:589-606). */
 int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
                                const void *Bm, const void *Cm, const float *D, const float *initial_states,
                                const uint8_t *reset, void *y, float *final_states, void *hip_stream);

@@ -114,7 +114,9 @@ def test_chunk_length_does_not_enter():
 
 def test_unsupported_shapes_are_refused():
     cases = [
-        WORKLOADS["plumbing_f32"],                                  # float32 inputs
+        WORKLOADS["plumbing_f32"],                                  # headdim 16 (float32 inputs)
+        Workload("f32_n128", 2, 128, 8, 32, 128, 1, 128, dtype="f32"),  # float32 inputs: state 32 or 64 only
+        Workload("f32_units4", 2, 128, 4, 32, 64, 1, 128, dtype="f32"), # float32 inputs: 8 units per group
         Workload("p16", 2, 128, 8, 16, 64, 1, 128),                 # headdim not a multiple of 32
         Workload("n16", 2, 256, 8, 32, 16, 1, 128),                 # state narrower than an MFMA tile
         Workload("units2", 2, 128, 2, 32, 64, 1, 128),              # 2 units per group
@@ -124,6 +126,55 @@ def test_unsupported_shapes_are_refused():
         with pytest.raises(SsdError) as ei:
             run(dev, w.chunk)
         assert ei.value.code == 2, w.name
+
+
+FLOAT_SHAPES = {
+    "policy": (2, 1024, 8, 32, 64, 1, 128),
+    "wide_head": (2, 300, 4, 64, 64, 1, 128),        # two 32-column units per head
+    "small_state": (3, 257, 16, 32, 32, 2, 64),      # N=32, two groups
+    "many_units": (1, 384, 16, 64, 64, 2, 128),      # 16 units per group: two workgroups per (batch, group)
+}
+
+
+@pytest.mark.parametrize("name", list(FLOAT_SHAPES))
+def test_float32_shapes_against_oracle(name):
+    """float32 inputs run on their own one-pass kernel (three bf16 terms per operand, tiles of 32 steps)."""
+    b, l, h, p, n, g, q = FLOAT_SHAPES[name]
+    check(Workload(name, b, l, h, p, n, g, q, dtype="f32"), seed=2)
+
+
+@pytest.mark.parametrize("seqlen", [1, 31, 32, 33, 100, 1000])
+def test_float32_ragged_lengths_initial_state_and_no_skip_term(seqlen):
+    check(Workload("ragged_f32", 2, seqlen, 8, 32, 64, 1, 128, dtype="f32", init_std=0.5), seed=seqlen)
+    check(Workload("ragged_f32_no_D", 2, seqlen, 8, 32, 64, 1, 128, dtype="f32", init_std=0.5), seed=seqlen + 1, drop_D=True)
+
+
+def test_float32_strong_decay_and_heavy_tails():
+    check(WORKLOADS["decay_extreme"].with_batch(2).with_dtype("f32"), seed=5, seqlen=1024)
+    check(Workload("all_large_dt_f32", 2, 256, 8, 32, 64, 1, 128, dtype="f32", a_log_range=(32.0, 64.0), dt_law="mixture",
+                   x_law="student-t3"), seed=6)
+
+
+def test_float32_restarts_inside_a_sequence():
+    w = Workload("reset_f32", 3, 500, 8, 32, 64, 1, 128, dtype="f32", init_std=0.5)
+    cpu = make_inputs(w, seed=13)
+    dev = to_dev(cpu)
+    m = (np.random.default_rng(5).random((w.batch, w.seqlen)) < 0.02).astype(np.uint8)
+    m[0, 0] = 1          # a restart before the first step: the initial state is not read
+    m[1, 31] = m[1, 32] = 1   # either side of a tile boundary
+    y, f = run(dev, w.chunk, reset=torch.from_numpy(m).cuda())
+    yr, fr = orc.ssd_sequential(np64(cpu["x"]), np64(cpu["dt"]), np64(cpu["A"]), np64(cpu["B"]), np64(cpu["C"]),
+                                np64(cpu["D"]), np64(cpu["init"]), reset=m)
+    assert_close(y, yr, torch.float32, "reset_f32 y")
+    assert_close(f, fr, torch.float32, "reset_f32 final")
+
+
+def test_float32_large_batches_take_the_one_pass_path():
+    w = WORKLOADS["policy_bf16"].with_batch(128).with_dtype("f32")
+    dev = to_dev(make_inputs(w, seed=2, seqlen=256))
+    y1, f1 = run(dev, w.chunk)
+    y2, f2 = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk)
+    assert torch.equal(y1, y2) and torch.equal(f1, f2)
 
 
 def test_one_pass_kernel_on_a_side_stream_and_inside_a_captured_graph():

@@ -34,8 +34,6 @@ def masks(Bsz, L, rng):
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("seqlen", [300, 77])
 def test_reset_mask_matches_the_oracle(fn, dtype, seqlen):
-    if fn == "onepass" and dtype == "f32":
-        pytest.skip("the one-pass kernel takes bf16 inputs")
     w = Workload("reset", 4, seqlen, 8, 32, 64, 1, 128, dtype=dtype, init_std=0.7)
     cpu = make_inputs(w, seed=13)
     dev = to_dev(cpu)

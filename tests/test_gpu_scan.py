@@ -239,6 +239,46 @@ def test_decay_extreme_full_size_properties():
     full_size_properties(WORKLOADS["decay_extreme"], [0, 17, 63])
 
 
+def full_size_properties_float32(w, rows, seed=0):
+    """float32 mode at a workload's full size: batch rows against the oracle at the float bar, exact homogeneity
+    under a power-of-two scaling of x, and state hand-over across a split."""
+    dev = make_inputs(w, seed=seed, device="cuda")
+    y, final = run(dev, w.chunk)
+    assert y.dtype == torch.float32 and torch.isfinite(y).all() and torch.isfinite(final).all()
+    sub = {k: (v[rows].cpu() if k in ("x", "dt", "B", "C", "init") and v is not None else (None if v is None else v.cpu()))
+           for k, v in dev.items()}
+    yr, fr = oracle_scan(sub)
+    ey = assert_close(y[rows], yr, torch.float32, f"{w.name} rows y")
+    ef = assert_close(final[rows], fr, torch.float32, f"{w.name} rows final")
+    print(f"{w.name} float32 full size B={w.batch} L={w.seqlen}: rows {rows} err_y={ey:.2e} err_final={ef:.2e}")
+    s = dict(dev)
+    s["x"] = dev["x"] * 4
+    if dev["init"] is not None:
+        s["init"] = dev["init"] * 4
+    y4, f4 = run(s, w.chunk)
+    assert (y4 - y * 4).abs().max() <= 1e-20 and (f4 - final * 4).abs().max() <= 1e-20
+    del y4, f4, s
+    h = w.seqlen // 2
+    a = {k: (v[:, :h].contiguous() if k in ("x", "dt", "B", "C") else v) for k, v in dev.items()}
+    b = {k: (v[:, h:].contiguous() if k in ("x", "dt", "B", "C") else v) for k, v in dev.items()}
+    y1, f1 = run(a, w.chunk)
+    b["init"] = f1
+    y2, f2 = run(b, w.chunk)
+    rms = float(y.double().pow(2).mean().sqrt())
+    assert float((y1 - y[:, :h]).abs().max()) <= 1e-4 * rms and float((y2 - y[:, h:]).abs().max()) <= 1e-4 * rms
+    assert rel_err(f2, np64(final)) <= 1e-4
+
+
+def test_policy_shape_float32_full_size_properties():
+    """B=256, L=2048, H=8, P=32, N=64 in float32 mode (the float one-pass kernel)."""
+    full_size_properties_float32(WORKLOADS["policy_bf16"].with_dtype("f32"), [0, 1, 254, 255])
+
+
+def test_decay_extreme_float32_full_size_properties():
+    """B=64, L=4096, A down to -64, 10 % near-total decays, Student-t x, in float32 mode."""
+    full_size_properties_float32(WORKLOADS["decay_extreme"].with_dtype("f32"), [0, 17, 63])
+
+
 def test_prepared_call_matches_the_plain_call():
     from trading_bot_0_amd import PreparedChunkScan
     w = WORKLOADS["policy_bf16"].with_batch(3)

@@ -83,15 +83,16 @@ def test_noalloc_forward_equals_the_workspace_forward_twice_in_a_row(name, first
 
 def test_noalloc_forward_takes_the_full_policy_shape_and_refuses_what_does_not_fit():
     """Batch 256 at the policy shape needs 302 MB of workspace on the staged path but runs as one launch of the
-    one-pass kernel, so the no-alloc entry point takes it; the same batch in float32 (staged) is refused."""
+    one-pass kernel, so the no-alloc entry point takes it; the same batch with heads of 16 (which only the staged
+    kernels take) is refused."""
     lib = ssd.load_library()
     prime(lib)
     w = WORKLOADS["policy_bf16"]
     run_pair(lib, w, w.seqlen, with_reset=False, with_init=True)
     inp = make_inputs(w, seed=0, device="cuda")
-    x32, dt32, b32, c32 = (inp[k].float() for k in ("x", "dt", "B", "C"))
-    dims = ssd.SsdDims(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk)
-    y = torch.empty_like(x32)
-    rc = lib.ssd_chunk_scan_noalloc_fwd(byref(dims), ssd.SSD_DTYPE_F32, x32.data_ptr(), dt32.data_ptr(), inp["A"].data_ptr(),
-                                        b32.data_ptr(), c32.data_ptr(), None, None, None, y.data_ptr(), None, None)
+    x16 = inp["x"][..., :16].contiguous()
+    dims = ssd.SsdDims(w.batch, w.seqlen, w.nheads, 16, w.dstate, w.ngroups, w.chunk)
+    y = torch.empty_like(x16)
+    rc = lib.ssd_chunk_scan_noalloc_fwd(byref(dims), ssd.SSD_DTYPE_BF16, x16.data_ptr(), inp["dt"].data_ptr(), inp["A"].data_ptr(),
+                                        inp["B"].data_ptr(), inp["C"].data_ptr(), None, None, None, y.data_ptr(), None, None)
     assert rc == 3 and "static scratch" in ssd.last_error(lib)

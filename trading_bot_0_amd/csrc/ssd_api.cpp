@@ -701,10 +701,10 @@ int ssd_chunk_scan_onepass_fwd(const ssd_dims *dims, int dtype, const void *x, c
     OPTIONAL_PTR(D);
     OPTIONAL_PTR(initial_states);
     OPTIONAL_PTR(final_states);
-    if (ssd::fused_scan_waves(s, dtype) == 0)
+    if (dtype == SSD_DTYPE_F32 ? ssd::fused_scan_f32_waves(s) == 0 : ssd::fused_scan_waves(s, dtype) == 0)
         return fail(SSD_ERR_UNSUPPORTED,
-                    "ssd: the one-pass scan needs bf16 inputs, headdim a multiple of 32, dstate 32, 64 or 128 and "
-                    "(nheads/ngroups)*(headdim/32) a multiple of 4");
+                    "ssd: the one-pass scan needs headdim a multiple of 32, dstate 32, 64 or 128 and "
+                    "(nheads/ngroups)*(headdim/32) a multiple of 4 (float32 inputs: dstate 32 or 64, a multiple of 8)");
     hipError_t e = ssd::launch_fused_scan(s, dtype, x, dt, A, Bm, Cm, D, initial_states, reset, y, final_states,
                                           (hipStream_t)hip_stream);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "one-pass scan launch");

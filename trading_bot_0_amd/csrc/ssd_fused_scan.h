@@ -656,7 +656,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
 #pragma unroll
                     for (int kk = 0; kk < NK; ++kk) {
                         accs[sl] = mma32(Hhi[sl * NK + kk], Cf[kk], accs[sl]);
+#ifndef SSD_ABLATE_STATE_LO
                         accs[sl] = mma32(Hlo[sl * NK + kk], Cf[kk], accs[sl]);
+#endif
                     }
                     accs[sl] = accs[sl] * blk_s[lb];
                 }
@@ -712,7 +714,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
 #pragma unroll
                         for (int j = 0; j < 2; ++j) {
                             accs[sl] = mma32(xf[sl][j], mh[j], accs[sl]);
+#ifndef SSD_ABLATE_M_LO
                             accs[sl] = mma32(xf[sl][j], ml[j], accs[sl]);
+#endif
                         }
                         if (diag && fast) accs[sl] = accs[sl] * El;  // everything summed so far shares the factor E[l]
                     }
@@ -894,7 +898,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) {
                     st[sl * NB + nb] = mma32(bf[nb], xhf, st[sl * NB + nb]);
+#ifndef SSD_ABLATE_WX_LO
                     st[sl * NB + nb] = mma32(bf[nb], xlf, st[sl * NB + nb]);
+#endif
                 }
             }
         }

@@ -26,6 +26,10 @@ hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const
                              const void *Bm, const void *Cm, const float *D, const float *init,
                              const unsigned char *reset, void *y, float *final_states, hipStream_t st,
                              float *tile_states) {
+    if (dtype == 0) {
+        if (tile_states != nullptr) return hipErrorInvalidValue;
+        return launch_fused_scan_f32(s, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
+    }
     const int waves = fused_scan_waves(s, dtype);
     if (waves == 0) return hipErrorInvalidValue;
     if (s.x_groups != 0 && (s.G != s.H || s.H % s.x_groups != 0 || (s.P / 32) % waves != 0)) return hipErrorInvalidValue;

@@ -41,6 +41,8 @@ __global__ __launch_bounds__(256) void segment_states_kernel(float *states, cons
     }
 }
 
+constexpr double kFloatTileUs = 7.5;
+
 int tiles_of(const ScanShape &s) { return (s.L + kOnePassTile - 1) / kOnePassTile; }
 
 }  // namespace
@@ -52,6 +54,15 @@ int tiles_of(const ScanShape &s) { return (s.L + kOnePassTile - 1) / kOnePassTil
 // every sequence side by side, about 510 per 2048 units x 32 tiles; a launch costs about 5.
 int fused_scan_plan(const ScanShape &s, int dtype, int *segments) {
     *segments = 1;
+    if (dtype == 0) {
+        // float inputs: the one-pass kernel on three bf16 terms per operand walks a tile of 32 steps in about
+        // kFloatTileUs; the staged float kernels take about 1345 per 2048 units x 32 tiles of 64
+        if (fused_scan_f32_waves(s) == 0) return 0;
+        const long long groups = (long long)s.B * s.G * ((s.H / s.G) * (s.P / 32) / 8);
+        const double staged = 20.0 + 1345.0 * ((double)groups * 8 * tiles_of(s)) / (2048.0 * 32.0);
+        const double whole = 5.0 + kFloatTileUs * ((s.L + 31) / 32) * (double)((groups + 255) / 256);
+        return whole < staged ? 1 : 0;
+    }
     const int waves = fused_scan_waves(s, dtype);
     const int full = s.N == 128 ? 4 : 8;  // waves of a workgroup that fills a CU
     if (waves != full) return 0;
@@ -80,7 +91,7 @@ int fused_scan_plan(const ScanShape &s, int dtype, int *segments) {
 // its own (by the plan's estimates) than as one more round: the rows of that remainder, else 0.
 int fused_scan_tail_rows(const ScanShape &s, int dtype) {
     int segments;
-    if (fused_scan_plan(s, dtype, &segments) != 1) return 0;
+    if (dtype == 0 || fused_scan_plan(s, dtype, &segments) != 1) return 0;
     const int full = s.N == 128 ? 4 : 8;
     const int per_row = s.G * ((s.H / s.G) * (s.P / 32) / full);  // workgroups per batch row
     const long long groups = (long long)s.B * per_row;

@@ -78,6 +78,12 @@ hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const
 // first every segment's own contribution to the state and its total decay (states only, no y, no C), then the
 // state entering every segment by a recurrence over the segments, then the forward proper per segment.
 // seg_states [B, segments, H, P, N] and seg_decay [B, segments, H] are scratch of the caller.
+// Float inputs on the one-pass kernel (three bf16 terms per operand): fused_scan_f32_waves is 0 when the shape
+// cannot run there, else the waves per workgroup (8).
+int fused_scan_f32_waves(const ScanShape &s);
+hipError_t launch_fused_scan_f32(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
+                                 const void *Cm, const float *D, const float *init, const unsigned char *reset, void *y,
+                                 float *final_states, hipStream_t st);
 // fused_scan_plan: which way a forward of this shape runs fastest by the library's cost estimates: 0 = the
 // staged kernels, 1 = the one-pass kernel, 2 = the one-pass kernel on *segments segments.
 int fused_scan_plan(const ScanShape &s, int dtype, int *segments);

@@ -397,7 +397,7 @@ def ssd_chunk_scan_onepass(
     y_dtype: Optional[torch.dtype] = None,
     reset: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    """The forward as one kernel and one pass over the inputs (bf16 only, no workspace); same results
+    """The forward as one kernel and one pass over the inputs (no workspace); same results
     as ssd_chunk_scan, which takes this path by itself when the batch is large enough.  Raises
     SsdError(unsupported) for shapes the one-pass kernel does not cover."""
     lib = load_library()
