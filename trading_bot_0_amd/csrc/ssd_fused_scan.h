@@ -117,9 +117,13 @@ constexpr float kFastDiagSpan = 120.f;  // log2-decay across a diagonal block up
 // Consecutive x tiles start 32 bytes (8 banks) apart modulo the bank width, so the staging writes, which hit
 // the same row and column of all tiles at once, do not collide.
 constexpr int fused_scan_xtile_elems(int Q) { return Q * 32 + 16; }
+// The eight-wave forward with a state of 64 or less keeps two sets of tiles and alternates between them: a tile's
+// staging writes then go to the set last read two tiles ago, which every wave left before the barrier of the tile in
+// between, so the barrier in front of the staging writes is not needed (one barrier per tile instead of two).
+constexpr bool fused_scan_two_tile_sets(int N, int waves) { return waves == 8 && N <= 64; }
 constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
-    return (size_t)2 * Q * N * 2 +
-           (size_t)waves * ((size_t)fused_scan_xtile_elems(Q) * 2 + (size_t)(5 + Q / 32) * Q * 4 + 64);
+    return ((size_t)2 * Q * N * 2 + (size_t)waves * fused_scan_xtile_elems(Q) * 2) * (fused_scan_two_tile_sets(N, waves) ? 2 : 1) +
+           (size_t)waves * ((size_t)(5 + Q / 32) * Q * 4 + 64);
 }
 
 // KIND 0: the forward.  KIND 1: the reversed-adjoint recurrence of the backward pass.  KIND 2: states only --
@@ -184,20 +188,22 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     constexpr int XS = SL == 2 ? wide_transposed_tile_elems(Q) : fused_scan_xtile_elems(Q);
     __shared__ __attribute__((aligned(16))) unsigned char smem[SL == 2 ? wide_transposed_scan_lds_bytes(Q)
                                                                         : TR ? transposed_scan_lds_bytes(Q)
-                                                                             : fused_scan_lds_bytes(N, Q, WAVES)];
+                                                                             : fused_scan_lds_bytes(N, Q, WAVES)];  // (kind 5 uses one set of the two)
     const int tid = threadIdx.x;
     const int lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // forward: B and C tiles [Q][N] of the workgroup, then one x tile [Q][32] per wave (+16 elements between tiles).
     // transposed: a B and a C tile [Q][32] per wave, then the shared x tile and the shared tile of the second
     // operand of the C . y products, each [Q][32].
+    // (forward with two tile sets: B, B', C, C', the x tiles, the x tiles')
+    constexpr bool kTwoSets = !TR && KIND != 5 && fused_scan_two_tile_sets(N, WAVES);  // (kind 5 would spill)
+    constexpr int SETS = kTwoSets ? 2 : 1;
     T *tiles = reinterpret_cast<T *>(smem);
-    T *Bs = TR ? tiles + wave * XS : tiles;
-    T *Cs = TR ? tiles + (WAVES + wave) * XS : tiles + Q * N;
-    T *xs_all = TR ? tiles + 2 * WAVES * XS : tiles + 2 * Q * N;
-    T *xs = TR ? xs_all : xs_all + wave * XS;
-    T *aux_s = xs_all + SL * XS;  // transposed only (one tile per slice, behind the x tiles)
-    float *wf0 = reinterpret_cast<float *>(TR ? xs_all + 2 * SL * XS : xs_all + WAVES * XS);
+    T *const Bs0 = TR ? tiles + wave * XS : tiles;
+    T *const Cs0 = TR ? tiles + (WAVES + wave) * XS : tiles + SETS * Q * N;
+    T *const xs_all0 = TR ? tiles + 2 * WAVES * XS : tiles + 2 * SETS * Q * N;
+    T *aux_s = xs_all0 + SL * XS;  // transposed only (one tile per slice, behind the x tiles)
+    float *wf0 = reinterpret_cast<float *>(TR ? xs_all0 + 2 * SL * XS : xs_all0 + SETS * WAVES * XS);
     float *wf = wf0 + wave * ((5 + QB) * Q + 16);
     // transposed only: every head's output tile, [WAVES][Q][33], or [WAVES][32][65] with two slices per wave
     float *red = wf0 + WAVES * ((5 + QB) * Q + 16);
@@ -478,12 +484,16 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
 
     float seg_total = 1.f;  // product of the tiles' decays (KIND 2)
     prefetch(c_first);
-    for (int c = c_first; c < c_end; ++c) {
+    // one tile; `set` (a compile-time 0 or 1) is the set of LDS tiles it uses; false when the scan ends inside it
+    auto tile = [&](const int c, auto set) -> bool {
+        constexpr int SET = decltype(set)::value;
+        T *const Bs = Bs0 + SET * Q * N, *const Cs = Cs0 + SET * Q * N, *const xs_all = xs_all0 + SET * WAVES * XS;
+        T *const xs = TR ? xs_all : xs_all + wave * XS;
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
         // the state entering every tile, for a caller that needs it (the backward pass): [B, nc, H, P, N]
         if (tile_states) store_state(tile_states + (((size_t)b * s.nc + c) * s.H + h) * s.P * N);
-        block_sync_lds();  // every wave is done reading the previous chunk's tiles
+        if (!kTwoSets) block_sync_lds();  // every wave is done reading the previous chunk's tiles
         // ---- registers -> LDS tiles ----
         // where the pieces go: the swizzle repeats every 32 rows, so all passes of a thread share the
         // offsets of its first (B, C) or first two (x: passes are 16 rows apart) rows
@@ -843,7 +853,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         // ---- phase 2: the state leaving this chunk ----
         // (the forward's last tile of a segment other than the last, or of a call that asks for no final state: nobody
         // reads the state it leaves)
-        if (KIND == 0 && c + 1 == c_end && !(final_states != nullptr && seg == S - 1)) break;
+        if (KIND == 0 && c + 1 == c_end && !(final_states != nullptr && seg == S - 1)) return false;
         if (!kEarlyPrefetch && c + 1 < c_end) prefetch(c + 1);
         // the other scan's state where this tile ends: the first slice in flight during phase 2, the second (two
         // slices per wave leave no registers to hold both) requested after it
@@ -913,6 +923,16 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 }
             }
         }
+        return true;
+    };
+    if constexpr (kTwoSets) {
+        for (int c = c_first; c < c_end; c += 2) {
+            if (!tile(c, std::integral_constant<int, 0>{})) break;
+            if (c + 1 < c_end && !tile(c + 1, std::integral_constant<int, 1>{})) break;
+        }
+    } else {
+        for (int c = c_first; c < c_end; ++c)
+            if (!tile(c, std::integral_constant<int, 0>{})) break;
     }
 
     if (STATES_ONLY) {
