@@ -1,9 +1,9 @@
 // One-pass forward for batches too small to fill the chip with one workgroup per 8 units: the sequence is cut
 // into segments that different workgroups walk side by side.
 //   1. states only (no y, no C): what every segment adds to the state, from a zero state, and its total decay;
-//   2. the state entering every segment: a recurrence over the few segments, one lane per 4 state elements;
-//   3. the forward proper per segment, each from its entering state.
-// Step 1 costs about 0.4 of step 3 (staging, scan and the state update, without the output phase); the two
+//   2. the forward proper per segment; each workgroup first runs the recurrence over the states of the segments
+//      before its own (a few fused multiply-adds per state element), which gives the state entering its segment.
+// Step 1 costs about 0.4 of step 2 (staging, scan and the state update, without the output phase); the two
 // together run S times as many workgroups as the uncut kernel.
 #include "ssd_fused_scan.h"
 
@@ -13,33 +13,6 @@ namespace {
 
 constexpr int kSegmentMinTiles = 4;        // shorter segments are mostly prologue
 constexpr int kSegmentTargetGroups = 192;  // workgroups to aim for (256 CUs; the last quarter gains little)
-
-// enter[b,0] = init (or zero); enter[b,s+1] = decay[b,s] * enter[b,s] + local[b,s], written over local in place
-// (local and decay of the last segment are not read: the states-only pass does not compute them)
-__global__ __launch_bounds__(256) void segment_states_kernel(float *states, const float *__restrict__ decay,
-                                                             const float *__restrict__ init,
-                                                             const unsigned char *__restrict__ reset, int L, int S, int H,
-                                                             int pn4, long long total) {
-    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= total) return;
-    const int idx = (int)(gid % pn4);
-    const long long bh = gid / pn4;
-    const int h = (int)(bh % H);
-    const long long b = bh / H;
-    const bool fresh = reset != nullptr && reset[b * L] != 0;  // restarts before its first step: init is not read
-    float4 cur = init && !fresh ? reinterpret_cast<const float4 *>(init)[bh * pn4 + idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s = 0; s < S; ++s) {
-        float4 *slot = reinterpret_cast<float4 *>(states) + ((b * S + s) * H + h) * (long long)pn4 + idx;
-        if (s + 1 == S) {
-            *slot = cur;
-            break;
-        }
-        const float4 loc = *slot;
-        const float a = decay[(b * S + s) * H + h];
-        *slot = cur;
-        cur = make_float4(a * cur.x + loc.x, a * cur.y + loc.y, a * cur.z + loc.z, a * cur.w + loc.w);
-    }
-}
 
 constexpr double kFloatTileUs = 7.5;
 
@@ -127,15 +100,12 @@ hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segmen
     hipError_t e = t.N == 32 ? fused_launch_states<2, kOnePassTile / 32, 8>(t, x, dt, A, Bm, nullptr, reset, seg_states, seg_decay, st)
                              : fused_launch_states<4, kOnePassTile / 32, 8>(t, x, dt, A, Bm, nullptr, reset, seg_states, seg_decay, st);
     if (e != hipSuccess) return e;
-    const int pn4 = s.P * s.N / 4;
-    const long long total = (long long)s.B * s.H * pn4;
-    segment_states_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(seg_states, seg_decay, init, reset, s.L, segments,
-                                                                                     s.H, pn4, total);
-    e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    // the forward per segment; its prologue runs the recurrence over the segment states
     ScanShape f = s;
     f.seg_tiles = t.seg_tiles;
-    return launch_fused_scan(f, dtype, x, dt, A, Bm, Cm, D, seg_states, reset, y, final_states, st);
+    f.seg_local = seg_states;
+    f.seg_local_decay = seg_decay;
+    return launch_fused_scan(f, dtype, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
 }
 
 }  // namespace ssd

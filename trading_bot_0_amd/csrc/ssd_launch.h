@@ -20,6 +20,10 @@ struct ScanShape {
     // The one-pass kernel only: the sequence cut into segments of seg_tiles tiles of 64 steps (0 = not cut) that
     // different workgroups walk; initial states are then given per segment, [B, segments, H, P, N].
     int seg_tiles = 0;
+    // The forward on segments: what the states-only pass left, per segment but the last, [B, segments, H, P, N] (the
+    // state a segment adds from zero) and [B, segments, H] (its total decay).  A workgroup's prologue runs the
+    // recurrence over the segments before its own, from the true initial state [B, H, P, N].
+    const float *seg_local = nullptr, *seg_local_decay = nullptr;
     // The staged kernels that read the initial state only: the restart mask [B, L] (or NULL).  A sequence that
     // restarts before its first step does not read its initial state at all, whatever that holds.
     const unsigned char *fresh = nullptr;
