@@ -40,26 +40,30 @@ namespace ssd {
 
 template <int COLS> struct ChunkTile {  // bf16 [rows][COLS], COLS = 32, 64 or 128
     static_assert(COLS == 32 || COLS == 64 || COLS == 128, "tile rows are 64, 128 or 256 bytes");
-    // XOR mask on the index of an 8-byte piece within its row, chosen against what the LDS of this chip does
-    // (measured with a 16-wave probe): a plain 8-byte read is served 16 consecutive lanes at a time from 32 banks
-    // (128 bytes a cycle), the transposing read 32 lanes at a time from 64.  So for the 8-byte reads of one logical
-    // piece of 32 consecutive rows, any 16 consecutive rows must spread that piece over all 16 eight-byte positions
-    // of the 128-byte bank line, and for the transposing read (4 consecutive rows x 64 bytes per 32 lanes) the four
-    // rows must keep their 64-byte pieces in different quarters of 256 bytes.  Both reads then run at their full
-    // rate (4.2 and 2.3 cycles per wave-instruction; with the four-row rule alone the plain reads took 8).
+    // XOR mask on the index of an 8-byte piece within its row (period: 32 rows).  Two descriptions of this chip's LDS
+    // had to be satisfied at once.  Timed with a 16-wave probe, a plain 8-byte access is served 16 consecutive lanes
+    // at a time from 128 bytes of banks (4.2 cycles per wave-instruction at best, 8 when two of the 16 lanes share an
+    // 8-byte slot) and the transposing read 32 lanes at a time from 256 bytes.  The hardware's bank-conflict counter,
+    // though, charges a plain 8-byte access by 32 lanes over 256 bytes: a mask that is a bijection of the low four
+    // row bits only (free of conflicts by the timing) doubled the counter against one that spreads 32 rows over 256
+    // bytes (free of conflicts by the counter, 8 cycles by the timing), with no difference in the kernels' run time
+    // either way.  The masks below satisfy both: for the 8-byte reads of one logical piece of 32 consecutive rows,
+    // any aligned 16 rows fill the 16 slots of 128 bytes and all 32 rows fill the 32 slots of 256 bytes; and the
+    // transposing read's four consecutive rows keep their 64-byte pieces in different quarters of 256 bytes.
     static __device__ inline int f(int row) {
+        const int r0 = row & 1, r1 = (row >> 1) & 1, r2 = (row >> 2) & 1, r3 = (row >> 3) & 1, r4 = (row >> 4) & 1;
         if constexpr (COLS == 32) {
-            // 64-byte rows: two rows per bank line; rows of one parity need 8 different masks over 16 rows, and rows
-            // 0,1 against 2,3 of a group of four must differ in the 32-byte half
-            return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+            // 64-byte rows, 8 pieces: per row parity a bijection of rows 1-3 (16 rows, 128 bytes), per row mod 4 a
+            // bijection of rows 2-4 (32 rows, 256 bytes)
+            return (r3 << 2) | (r2 << 1) | (r1 ^ r4);
         } else if constexpr (COLS == 128) {
-            // 256-byte rows: bits 3-4 of the piece index (the 64-byte quarter) from the row's low two bits, bits 0-3
-            // (the position in the bank line) a bijection of the row's low four bits
-            return (((row >> 1) & 1) << 4) | ((row & 1) << 3) | (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);
+            // 256-byte rows, 32 pieces: the 64-byte quarter from the row's low two bits, the low four mask bits a
+            // bijection of the row's low four bits, all five of all five
+            return ((r1 ^ r4) << 4) | (r0 << 3) | (r1 << 2) | (r2 << 1) | r3;
         } else {
-            // 128-byte rows: one row per bank line; the 32-byte quarter from the row's low two bits, the piece within
-            // it from the next two
-            return ((row & 3) << 2) | ((row >> 2) & 3);
+            // 128-byte rows, 16 pieces: a bijection of the low four row bits, and per row parity of rows 1-4; the
+            // 64-byte half from row bit 1
+            return (r1 << 3) | (r3 << 2) | (r2 << 1) | (r0 ^ r4);
         }
     }
     static __device__ inline int off(int row, int col) {
@@ -114,9 +118,12 @@ constexpr int kOnePassTile = 64;
 constexpr float kFastDiagSpan = 120.f;  // log2-decay across a diagonal block up to which E*F is safe
 
 // LDS of one workgroup: B and C tiles, one x tile per wave, (5 + Q/32) float rows and 16 block scalars per wave.
-// Consecutive x tiles start 32 bytes (8 banks) apart modulo the bank width, so the staging writes, which hit
-// the same row and column of all tiles at once, do not collide.
 constexpr int fused_scan_xtile_elems(int Q) { return Q * 32 + 16; }
+// Where unit u's x tile starts inside the x region of the forward's layout (waves * fused_scan_xtile_elems(Q)
+// elements): tiles of exactly Q * 32 elements, odd units 8 bytes further, every pair of units 64 bytes further.
+// A staging write hits one row and four 8-byte pieces of the same parity in each of the workgroup's tiles at once;
+// with these offsets the 16 (or 32) lanes served together fill 128 (256) bytes of banks exactly.
+__device__ inline int fused_scan_xtile_base(int Q, int u) { return u * (Q * 32) + (u & 1) * 4 + (u >> 1) * 32; }
 // The eight-wave forward with a state of 64 or less keeps two sets of tiles and alternates between them: a tile's
 // staging writes then go to the set last read two tiles ago, which every wave left before the barrier of the tile in
 // between, so the barrier in front of the staging writes is not needed (one barrier per tile instead of two; the tile
@@ -511,7 +518,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     auto tile = [&](const int c, auto set) -> bool {
         constexpr int SET = decltype(set)::value;
         T *const Bs = Bs0 + SET * Q * N, *const Cs = Cs0 + SET * Q * N, *const xs_all = xs_all0 + SET * WAVES * XS;
-        T *const xs = TR ? xs_all : xs_all + wave * XS;
+        T *const xs = TR ? xs_all : xs_all + fused_scan_xtile_base(Q, wave);
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
         // the state entering every tile, for a caller that needs it (the backward pass): [B, nc, H, P, N]
@@ -527,7 +534,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             bw[hf] = BT::off(tw / BPR, (tw % BPR) * 8 + 4 * hf);
 #pragma unroll
             for (int par = 0; par < 2; ++par)
-                xw[par][hf] = ((tw % XPR) / 4) * XS + XT::off(tw / XPR + 16 * par, ((tw % XPR) % 4) * 8 + 4 * hf);
+                xw[par][hf] = (TR ? ((tw % XPR) / 4) * XS : fused_scan_xtile_base(Q, (tw % XPR) / 4)) +
+                              XT::off(tw / XPR + 16 * par, ((tw % XPR) % 4) * 8 + 4 * hf);
         }
         if constexpr (TR) {
 #pragma unroll

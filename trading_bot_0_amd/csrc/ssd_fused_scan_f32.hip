@@ -28,8 +28,8 @@ constexpr int kFloatTile = 32;
 // large as the span, rounded to float, so their product is off by about 2^-24 span ln 2
 constexpr float kFloatFastSpan = 4.f;
 
-constexpr int f32_xterm_elems() { return kFloatTile * 32 + 16; }  // bf16 elements of one x term tile
-constexpr int f32_xfloat_elems() { return kFloatTile * 32 + 8; }  // floats of one float x tile
+constexpr int f32_xterm_elems() { return kFloatTile * 32 + 32; }  // bf16 elements per unit of an x term region
+constexpr int f32_xfloat_elems() { return kFloatTile * 32 + 16; }  // floats per unit of the float x region
 constexpr int f32_table_floats() { return 6 * kFloatTile + 16; }
 // bf16 elements from one term tile of B (or C) to the next: 16 bytes more than the tile, so that no two-address
 // LDS read (whose two offsets are multiples of 512 bytes) reaches from one term into another -- the compiler
@@ -39,6 +39,13 @@ constexpr size_t fused_scan_f32_lds_bytes(int N, int waves) {
     return (size_t)2 * 3 * f32_bcterm_elems(N) * 2 + (size_t)waves * 3 * f32_xterm_elems() * 2 +
            (size_t)waves * f32_xfloat_elems() * 4 + (size_t)waves * f32_table_floats() * 4;
 }
+
+// Where unit u's tiles start inside their regions (waves * f32_xterm_elems() bf16 elements per term, waves *
+// f32_xfloat_elems() floats): a staging write hits one row and all eight 8-byte pieces (term tiles), or every other
+// one (float tile), of several units' tiles at once; these offsets spread the 16 (or 32) lanes served together over
+// 128 (256) bytes of banks (the offsets grow with u, so the tiles do not overlap).
+__device__ inline int f32_xterm_base(int u) { return u * (kFloatTile * 32) + (u & 3) * 32 + (u >> 2) * 128; }
+__device__ inline int f32_xfloat_base(int u) { return u * (kFloatTile * 32) + (u & 1) * 2 + ((u >> 1) & 1) * 32 + (u >> 2) * 64; }
 
 // float x tile [32][32]: the 8-byte pieces of a row XOR-swizzled with the row's low four bits, so that 8-byte reads
 // of one column pair of 16 consecutive rows, 4-byte reads along a row and the staging writes all spread over the
@@ -111,8 +118,8 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
     T *xt_all = Cs + 3 * TB;               // [3][WAVES][XS]
     float *xf_all = reinterpret_cast<float *>(xt_all + 3 * WAVES * XS);  // [WAVES][XF]
     float *wf = xf_all + WAVES * XF + wave * WF;
-    T *xt = xt_all + wave * XS;            // term t of this wave's unit: xt + t * WAVES * XS
-    float *xf = xf_all + wave * XF;
+    T *xt = xt_all + f32_xterm_base(wave);  // term t of this wave's unit: xt + t * WAVES * XS
+    float *xf = xf_all + f32_xfloat_base(wave);
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
 
     // ---- which units this workgroup owns (as the bf16 kernel) ----
@@ -194,10 +201,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
             unsigned t3[3][2];
             split3_pair(xq[u].x, xq[u].y, t3[0][0], t3[1][0], t3[2][0]);
             split3_pair(xq[u].z, xq[u].w, t3[0][1], t3[1][1], t3[2][1]);
-            const int o = x_unit * XS + XT::off(row, x_col);
+            const int o = f32_xterm_base(x_unit) + XT::off(row, x_col);
 #pragma unroll
             for (int t = 0; t < 3; ++t) *reinterpret_cast<uint2 *>(xt_all + t * WAVES * XS + o) = make_uint2(t3[t][0], t3[t][1]);
-            float *xr = xf_all + x_unit * XF;
+            float *xr = xf_all + f32_xfloat_base(x_unit);
             *reinterpret_cast<float2 *>(xr + xfloat_off(row, x_col)) = make_float2(xq[u].x, xq[u].y);
             *reinterpret_cast<float2 *>(xr + xfloat_off(row, x_col + 2)) = make_float2(xq[u].z, xq[u].w);
         }
