@@ -57,10 +57,15 @@ import sys
 import time
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
-# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE
-# on this very command (profiles/chunk_scan_forward_policy_bf16.md: 200 800 + 278 500 KiB, copy-kernel
-# calibration factor 1.00); counters cannot be read from inside this script, so the figure is carried here
-MEASURED_TRAFFIC_BYTES = {("policy_bf16", 256, "onepass_scan"): 490.8e6}
+# HBM bytes per forward of the dominant kernel(s), measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on
+# this very command at the library revision the profiles name (profiles/chunk_scan_forward_*.md give the KiB per
+# dispatch of each counter and the copy-kernel calibration, factor 1.00); counters cannot be read from inside this
+# script, so the figures are carried here, keyed by (workload, batch): a run at any other size reports null.
+# Reads come out below the compulsory bytes because inputs that stay in the 256 MB last-level cache from one call
+# of the loop to the next are not fetched from HBM again.
+MEASURED_TRAFFIC_BYTES = {("policy_bf16", 256): 491.9e6,          # 201 100 + 279 300 KiB, one launch
+                          ("long_lookback_bf16", 32): 2012.4e6,   # 900 200 + 1 065 000 KiB, one launch
+                          ("decay_extreme", 64): 325.0e6}         # states only 63 060 + 12 290, forward 106 700 + 135 400 KiB
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 
@@ -304,7 +309,7 @@ def main():
                         "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)}
         roofline = {"kernel": "onepass_scan" if onepass else f"onepass_scan on {segments} segments", "bound": "hbm", "achieved": onepass_info["GBps"],
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": onepass_info["hbm_frac"],
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, w.batch, "onepass_scan"))}
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, w.batch))}
     else:
         dom = max(stages, key=lambda k: stages[k]["ms"])
         roofline = {"kernel": dom, "bound": "hbm", "achieved": stages[dom]["GBps"], "peak": HBM_PEAK_GBS,
@@ -561,7 +566,19 @@ def main():
                                "post_ms": round(t_post, 4), "post_GBps": round(post_bytes / t_post / 1e6, 1),
                                "out_proj_ms": round(t_out, 4), "out_proj_GBps": round(out_bytes / t_out / 1e6, 1),
                                "out_proj_blas_ms": round(t_out_blas, 4)}
-        del u, zx, xs_, bs_, cs_, ds_, ys_, yn, blk
+        if hasattr(blk, "backward") and not args.no_backward:
+            # forward with what the backward needs kept, then the block's backward (stage kernels of this library,
+            # the scan's backward, four GEMMs)
+            del xs_, bs_, cs_, ds_, ys_, yn
+            dout = torch.randn_like(u)
+
+            def fwd_bwd():
+                _, ctx = blk.forward(u, save_for_backward=True)
+                blk.backward(ctx, dout)
+
+            out["mamba2_block"]["fwd_bwd_ms"] = round(timed(fwd_bwd, n=5), 4)
+            del dout
+        del u, zx, blk
 
     # ---- CPU baseline: the same arithmetic on this box's host cores, on bounded batch slices -----------------
     # (1) the plain-C sequential recurrence (float32, OpenMP) -- the headline cpu_baseline;
