@@ -14,9 +14,31 @@ namespace ssd {
 
 namespace {
 
-constexpr int kBwdSteps = 16;    // timesteps per thread of the conv backward (its forward's run length)
-constexpr int kPiecesPerBlock = 16;  // channel pieces (of 8) per workgroup of the conv backward
-constexpr int kRunsPerBlock = 16;
+constexpr int kBwdSteps = 32;    // timesteps per thread of the conv backward
+constexpr int kBwdCh = 4;            // channels per thread of the conv backward (eight would take 290 registers)
+constexpr int kPiecesPerBlock = 32;  // channel pieces (of kBwdCh) per workgroup of the conv backward
+constexpr int kRunsPerBlock = 8;
+
+template <typename T> struct PackCh;  // kBwdCh = four consecutive channels
+template <> struct PackCh<__bf16> {
+    uint2 u;
+    __device__ inline float get(int i) const {
+        const unsigned w = (&u.x)[i >> 1];
+        return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+    }
+    static __device__ inline PackCh load(const __bf16 *p) { return PackCh{*reinterpret_cast<const uint2 *>(p)}; }
+    static __device__ inline void store(__bf16 *p, const float (&v)[4]) {
+        *reinterpret_cast<uint2 *>(p) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    }
+};
+template <> struct PackCh<float> {
+    float4 a;
+    __device__ inline float get(int i) const { return (&a.x)[i]; }
+    static __device__ inline PackCh load(const float *p) { return PackCh{*reinterpret_cast<const float4 *>(p)}; }
+    static __device__ inline void store(float *p, const float (&v)[4]) {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+};
 constexpr int kPostBlocks = 1024;    // workgroups of post_bwd (each walks rows with a grid stride)
 
 // ---- post ----------------------------------------------------------------------------------------------------
@@ -116,42 +138,69 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
     }
 }
 
-// out[c] = sum over parts of part[p][c], in order (columns = channels)
+// out[c] = sum over parts of part[p][c] (columns = channels), in a fixed order: a workgroup is 64 columns x 4 slices
+// of its share of the parts (blockIdx.y of gridDim.y shares); a slice adds every fourth part of the share in order,
+// the four slices are added in order, and the shares' sums [gridDim.y][cols] go through the same kernel once more.
+constexpr int kSumShares = 32;
 __global__ __launch_bounds__(256) void column_sums_kernel(const float *__restrict__ part, int nparts, int cols,
                                                           float *__restrict__ out) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= cols) return;
+    __shared__ float sm[4][64];
+    const int cl = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + cl;
+    const int per = (nparts + gridDim.y - 1) / gridDim.y;
+    const int p0 = blockIdx.y * per, p1 = min(nparts, p0 + per);
     float acc = 0.f;
-    for (int p = 0; p < nparts; ++p) acc += part[(size_t)p * cols + c];
-    out[c] = acc;
+    if (c < cols) {
+#pragma unroll 4
+        for (int p = p0 + q; p < p1; p += 4) acc += part[(size_t)p * cols + c];
+    }
+    sm[q][cl] = acc;
+    __syncthreads();
+    if (q == 0 && c < cols) out[(size_t)blockIdx.y * cols + c] = ((sm[0][cl] + sm[1][cl]) + sm[2][cl]) + sm[3][cl];
+}
+
+// sums of nparts rows of `cols` floats into out[cols]; tmp holds kSumShares * cols floats
+static hipError_t launch_column_sums(const float *part, int nparts, int cols, float *tmp, float *out, hipStream_t st) {
+    const dim3 blocks((cols + 63) / 64, nparts >= 4 * kSumShares ? kSumShares : 1);
+    if (blocks.y == 1) {
+        column_sums_kernel<<<blocks, dim3(256), 0, st>>>(part, nparts, cols, out);
+        return hipGetLastError();
+    }
+    column_sums_kernel<<<blocks, dim3(256), 0, st>>>(part, nparts, cols, tmp);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    column_sums_kernel<<<dim3(blocks.x, 1), dim3(256), 0, st>>>(tmp, kSumShares, cols, out);
+    return hipGetLastError();
 }
 
 // ---- pre -----------------------------------------------------------------------------------------------------
-// One thread per (run of kBwdSteps timesteps, 8 channels of x | B | C).  pre[t] = b + sum_k w[k] in[t-(K-1)+k]
-// (taps before the latest restart at or before t cut), out = silu(pre); with dpre[t] = dout[t] silu'(pre[t]):
-//   din[s]  = sum_{j=0..K-1} w[K-1-j] dpre[s+j]      over the j whose output s+j exists and lies before any restart
+// One thread per (run of kBwdSteps timesteps, kBwdCh channels of x | B | C).  pre[t] = b + sum_k w[k] in[t-(K-1)+k]
+// (taps before the latest restart at or before t cut: the window's older rows are zeroed at a restart, as in the
+// forward), out = silu(pre); with dpre[t] = dout[t] silu'(pre[t]):
+//   din[s]  = sum_{q=0..K-1} w[K-1-q] dpre[s+q]      over the q whose output s+q exists and lies before any restart
 //                                                     after s
-//   dw[k]  += dpre[t] in[t-(K-1)+k] (live taps),  db += dpre[t]
-// The thread recomputes pre over its run and K-1 timesteps beyond it.  The run that starts at t = 0 also leaves the
-// gradient of the conv state (the inputs before t = 0); a gradient on the returned conv state joins din of the last
-// K-1 timesteps.
+//   dw[k]  += dpre[t] in[t-(K-1)+k],  db += dpre[t]
+// The thread walks its run and K-1 timesteps beyond it once, with the last K input rows and the last K dpre rows in
+// two rings of registers (the loop is unrolled by K, so ring positions are compile-time): dpre[t] is formed at step t
+// and din[t-(K-1)] leaves at the same step.  A gradient on the returned conv state joins din of the last K-1
+// timesteps; the gradient of the incoming conv state is block_pre_bwd_state_kernel's.
 template <typename T, int K>
 __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict__ zxbcdt, const float *__restrict__ conv_w,
                                                             const float *__restrict__ conv_b, const T *__restrict__ state_in,
                                                             const unsigned char *__restrict__ reset, const T *__restrict__ dx,
                                                             const T *__restrict__ dB, const T *__restrict__ dC,
                                                             const T *__restrict__ dstate_out, T *__restrict__ dzxbcdt,
-                                                            T *__restrict__ dstate_in, float *__restrict__ part, BlockShape s) {
+                                                            float *__restrict__ part, BlockShape s) {
     const int DI = s.H * s.P, GN = s.G * s.N, C = DI + 2 * GN;
-    const int CP = C / 8;
+    const int CP = C / kBwdCh;
     const int runs = (s.L + kBwdSteps - 1) / kBwdSteps;
     const int pl = threadIdx.x % kPiecesPerBlock, rl = threadIdx.x / kPiecesPerBlock;
     const int piece = blockIdx.x * kPiecesPerBlock + pl;
     const long long br = (long long)blockIdx.y * kRunsPerBlock + rl;
     const bool active = piece < CP && br < (long long)s.B * runs;
-    float dwacc[8][K], dbacc[8];
+    float dwacc[kBwdCh][K], dbacc[kBwdCh];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kBwdCh; ++i) {
         dbacc[i] = 0.f;
 #pragma unroll
         for (int k = 0; k < K; ++k) dwacc[i][k] = 0.f;
@@ -159,12 +208,12 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
     if (active) {
         const int t0 = (int)(br % runs) * kBwdSteps, b = (int)(br / runs);
         const int t1 = min(t0 + kBwdSteps, s.L);
-        const int c0 = piece * 8;
+        const int c0 = piece * kBwdCh;
         const T *row0 = zxbcdt + ((size_t)b * s.L) * s.ld + DI + c0;
         const unsigned char *rs = reset ? reset + (size_t)b * s.L : nullptr;
-        float w[8][K], bias[8];
+        float w[kBwdCh][K], bias[kBwdCh];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < kBwdCh; ++i) {
             bias[i] = conv_b[c0 + i];
 #pragma unroll
             for (int k = 0; k < K; ++k) w[i][k] = conv_w[(size_t)(c0 + i) * K + k];
@@ -183,135 +232,117 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
             gstride = GN;
         }
         // input row of timestep ts (history before 0 from the conv state, zero without one)
-        auto in_row = [&](int ts, float (&v)[8]) {
+        auto in_row = [&](int ts, float (&v)[kBwdCh]) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = 0.f;
+            for (int i = 0; i < kBwdCh; ++i) v[i] = 0.f;
             if (ts >= 0) {
-                const Pack8<T> p = Pack8<T>::load(row0 + (size_t)ts * s.ld);
+                const PackCh<T> p = PackCh<T>::load(row0 + (size_t)ts * s.ld);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[i] = p.get(i);
+                for (int i = 0; i < kBwdCh; ++i) v[i] = p.get(i);
             } else if (state_in != nullptr) {
-                const Pack8<T> p = Pack8<T>::load(state_in + ((size_t)b * (K - 1) + (K - 1 + ts)) * C + c0);
+                const PackCh<T> p = PackCh<T>::load(state_in + ((size_t)b * (K - 1) + (K - 1 + ts)) * C + c0);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[i] = p.get(i);
+                for (int i = 0; i < kBwdCh; ++i) v[i] = p.get(i);
             }
         };
-        // dpre of the timesteps t0 .. t0 + kBwdSteps + K - 2 (zero past the sequence), from a window of inputs that slides
-        constexpr int NT = kBwdSteps + K - 1;
-        float dpre[NT][8];
-        float win[K][8];
-        // `depth` = how many of the window's older rows are still live: a restart at t makes it zero for t itself
-        int depth = K - 1;
+        // rings: step j (timestep t0 + j) uses position j % K; position of step j - m is (j - m) mod K
+        float win[K][kBwdCh], dq[K][kBwdCh];
+        bool fl[K];
 #pragma unroll
-        for (int k = 0; k < K - 1; ++k) in_row(t0 - (K - 1) + k, win[k]);
+        for (int k = 0; k < K; ++k) {
+            fl[k] = false;
+#pragma unroll
+            for (int i = 0; i < kBwdCh; ++i) dq[k][i] = 0.f;
+        }
+#pragma unroll
+        for (int m = 1; m <= K - 1; ++m) in_row(t0 - m, win[K - m]);
         if (rs != nullptr) {
-            // restarts at the K-2 timesteps before the run cut the rows before them
-            depth = K - 1;
+            // a restart at one of the K-2 timesteps before the run cuts the rows before it
+#pragma unroll
             for (int back = 1; back <= K - 2; ++back) {
                 const int ts = t0 - back;
                 if (ts >= 0 && rs[ts] != 0) {
-                    depth = back;
-                    break;
+#pragma unroll
+                    for (int m = back + 1; m <= K - 1; ++m) {
+#pragma unroll
+                        for (int i = 0; i < kBwdCh; ++i) win[K - m][i] = 0.f;
+                    }
                 }
             }
         }
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-            const int t = t0 + j;
-            const bool exists = t < s.L;
-            if (exists) in_row(t, win[K - 1]);
-            if (exists && rs != nullptr && rs[t] != 0) depth = 0;
-            float gin[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) gin[i] = 0.f;
-            if (exists) {
-                const Pack8<T> p = Pack8<T>::load(gsrc + (size_t)t * gstride);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) gin[i] = p.get(i);
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                float a = bias[i];
-#pragma unroll
-                for (int k = 0; k < K; ++k) a += (K - 1 - k <= depth) ? w[i][k] * win[k][i] : 0.f;
-                dpre[j][i] = exists ? gin[i] * dsilu(a) : 0.f;
-            }
-            if (exists && t < t1) {  // this thread's own timesteps: the parameter gradients
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    dbacc[i] += dpre[j][i];
-#pragma unroll
-                    for (int k = 0; k < K; ++k) dwacc[i][k] += (K - 1 - k <= depth) ? dpre[j][i] * win[k][i] : 0.f;
-                }
-            }
-#pragma unroll
-            for (int k = 0; k < K - 1; ++k) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) win[k][i] = win[k + 1][i];
-            }
-            if (depth < K - 1) ++depth;
-        }
-        // din[s] for the run's timesteps: outputs s .. s+K-1 while no restart lies after s
         T *drow = dzxbcdt + ((size_t)b * s.L) * s.ld + DI + c0;
+        constexpr int NT = kBwdSteps + K - 1;
+#pragma unroll 1
+        for (int jb = 0; jb < NT; jb += K) {
 #pragma unroll
-        for (int j = 0; j < kBwdSteps; ++j) {
-            const int sidx = t0 + j;
-            if (sidx >= t1) break;
-            float o[8];
+            for (int u = 0; u < K; ++u) {  // ring position of this step: u
+                const int t = t0 + jb + u;
+                const bool exists = t < s.L && jb + u < NT;
+                const bool r = exists && rs != nullptr && rs[t] != 0;
+                if (r) {  // the rows before a restart do not reach it
 #pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = 0.f;
-            bool open = true;
+                    for (int m = 1; m <= K - 1; ++m) {
 #pragma unroll
-            for (int q = 0; q < K; ++q) {
-                const int t = sidx + q;
-                if (q > 0 && open && t < s.L && rs != nullptr && rs[t] != 0) open = false;
-                if (open && t < s.L) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) o[i] += w[i][K - 1 - q] * dpre[j + q][i];
-                }
-            }
-            // a gradient on the conv state the forward returned: that state is the last K-1 input rows, those before
-            // the window's last restart zeroed
-            if (dstate_out != nullptr && sidx >= s.L - (K - 1)) {
-                bool kept = true;
-                for (int t = sidx + 1; t < s.L; ++t) kept = kept && !(rs != nullptr && rs[t] != 0);
-                if (kept) {
-                    const Pack8<T> p = Pack8<T>::load(dstate_out + ((size_t)b * (K - 1) + (sidx - (s.L - (K - 1)))) * C + c0);
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) o[i] += p.get(i);
-                }
-            }
-            Pack8<T>::store(drow + (size_t)sidx * s.ld, o);
-        }
-        // the gradient of the conv state: inputs at s = -(K-1) .. -1 reach outputs 0 .. s+K-1, up to the first restart
-        if (t0 == 0 && dstate_in != nullptr) {
-#pragma unroll
-            for (int jrow = 0; jrow < K - 1; ++jrow) {
-                const int sidx = jrow - (K - 1);
-                float o[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) o[i] = 0.f;
-                bool open = true;
-#pragma unroll
-                for (int t = 0; t < K - 1; ++t) {
-                    if (open && t < s.L && rs != nullptr && rs[t] != 0) open = false;
-                    const int k = sidx - t + (K - 1);
-                    if (open && t < s.L && k >= 0) {
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) o[i] += w[i][k] * dpre[t][i];
+                        for (int i = 0; i < kBwdCh; ++i) win[(u + K - m) % K][i] = 0.f;
                     }
                 }
-                // rows of the old state that are still part of the new one (fewer than K-1 new timesteps)
-                if (dstate_out != nullptr && sidx >= s.L - (K - 1)) {
-                    bool kept = true;
-                    for (int t = 0; t < s.L; ++t) kept = kept && !(rs != nullptr && rs[t] != 0);
-                    if (kept) {
-                        const Pack8<T> p = Pack8<T>::load(dstate_out + ((size_t)b * (K - 1) + (sidx - (s.L - (K - 1)))) * C + c0);
+                float gin[kBwdCh];
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) o[i] += p.get(i);
+                for (int i = 0; i < kBwdCh; ++i) {
+                    gin[i] = 0.f;
+                    win[u][i] = 0.f;
+                }
+                if (exists) {
+                    const PackCh<T> p = PackCh<T>::load(row0 + (size_t)t * s.ld);
+                    const PackCh<T> g = PackCh<T>::load(gsrc + (size_t)t * gstride);
+#pragma unroll
+                    for (int i = 0; i < kBwdCh; ++i) {
+                        win[u][i] = p.get(i);
+                        gin[i] = g.get(i);
                     }
                 }
-                Pack8<T>::store(dstate_in + ((size_t)b * (K - 1) + jrow) * C + c0, o);
+                const bool own = exists && t < t1;  // this thread's own timesteps: the parameter gradients
+#pragma unroll
+                for (int i = 0; i < kBwdCh; ++i) {
+                    float a = bias[i];
+#pragma unroll
+                    for (int k = 0; k < K; ++k) a += w[i][k] * win[(u + k + 1) % K][i];
+                    const float d = gin[i] * dsilu(a);  // (gin is zero past the sequence)
+                    dq[u][i] = d;
+                    const float dm = own ? d : 0.f;
+                    dbacc[i] += dm;
+#pragma unroll
+                    for (int k = 0; k < K; ++k) dwacc[i][k] += dm * win[(u + k + 1) % K][i];
+                }
+                fl[u] = r;
+                // din of timestep sidx = t - (K-1): outputs sidx .. t while no restart lies after sidx
+                const int sidx = t - (K - 1);
+                if (jb + u >= K - 1 && sidx < t1) {
+                    float o[kBwdCh];
+#pragma unroll
+                    for (int i = 0; i < kBwdCh; ++i) o[i] = w[i][K - 1] * dq[(u + 1) % K][i];
+                    bool open = true;
+#pragma unroll
+                    for (int q = 1; q < K; ++q) {
+                        open = open && !fl[(u + 1 + q) % K];
+                        if (open) {
+#pragma unroll
+                            for (int i = 0; i < kBwdCh; ++i) o[i] += w[i][K - 1 - q] * dq[(u + 1 + q) % K][i];
+                        }
+                    }
+                    // a gradient on the conv state the forward returned: that state is the last K-1 input rows,
+                    // those before the window's last restart zeroed
+                    if (dstate_out != nullptr && sidx >= s.L - (K - 1)) {
+                        bool kept = true;
+                        for (int tt = sidx + 1; tt < s.L; ++tt) kept = kept && !(rs != nullptr && rs[tt] != 0);
+                        if (kept) {
+                            const PackCh<T> p = PackCh<T>::load(dstate_out + ((size_t)b * (K - 1) + (sidx - (s.L - (K - 1)))) * C + c0);
+#pragma unroll
+                            for (int i = 0; i < kBwdCh; ++i) o[i] += p.get(i);
+                        }
+                    }
+                    PackCh<T>::store(drow + (size_t)sidx * s.ld, o);
+                }
             }
         }
     }
@@ -319,14 +350,14 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
     __shared__ float red[256 * (K + 1)];
     const int cols = C * (K + 1);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kBwdCh; ++i) {
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < K; ++k) red[threadIdx.x * (K + 1) + k] = dwacc[i][k];
         red[threadIdx.x * (K + 1) + K] = dbacc[i];
         __syncthreads();
         if (rl == 0 && piece < CP) {
-            const int c = piece * 8 + i;
+            const int c = piece * kBwdCh + i;
 #pragma unroll
             for (int k = 0; k <= K; ++k) {
                 float acc = 0.f;
@@ -334,6 +365,89 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
                 part[(size_t)blockIdx.y * cols + (size_t)c * (K + 1) + k] = acc;
             }
         }
+    }
+}
+
+// The gradient of the incoming conv state: one thread per (batch row, 8 channels).  The inputs at s = -(K-1) .. -1
+// reach outputs 0 .. s+K-1, up to the first restart; the thread recomputes dpre of those K-1 outputs.
+template <typename T, int K>
+__global__ __launch_bounds__(256) void block_pre_bwd_state_kernel(const T *__restrict__ zxbcdt, const float *__restrict__ conv_w,
+                                                                  const float *__restrict__ conv_b, const T *__restrict__ state_in,
+                                                                  const unsigned char *__restrict__ reset, const T *__restrict__ dx,
+                                                                  const T *__restrict__ dB, const T *__restrict__ dC,
+                                                                  const T *__restrict__ dstate_out, T *__restrict__ dstate_in,
+                                                                  BlockShape s) {
+    const int DI = s.H * s.P, GN = s.G * s.N, C = DI + 2 * GN, CP = C / 8;
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (long long)s.B * CP) return;
+    const int piece = (int)(gid % CP), b = (int)(gid / CP), c0 = piece * 8;
+    const T *row0 = zxbcdt + ((size_t)b * s.L) * s.ld + DI + c0;
+    const unsigned char *rs = reset ? reset + (size_t)b * s.L : nullptr;
+    float w[8][K], bias[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        bias[i] = conv_b[c0 + i];
+#pragma unroll
+        for (int k = 0; k < K; ++k) w[i][k] = conv_w[(size_t)(c0 + i) * K + k];
+    }
+    const T *gsrc = c0 < DI ? dx + ((size_t)b * s.L) * DI + c0
+                            : c0 < DI + GN ? dB + ((size_t)b * s.L) * GN + (c0 - DI) : dC + ((size_t)b * s.L) * GN + (c0 - DI - GN);
+    const int gstride = c0 < DI ? DI : GN;
+    // dpre of outputs 0 .. K-2; `open` = no restart at 0 .. t (a restart at t cuts the state off output t as well)
+    float acc[K - 1][8];
+#pragma unroll
+    for (int jr = 0; jr < K - 1; ++jr) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[jr][i] = 0.f;
+    }
+    bool open = true;
+#pragma unroll
+    for (int t = 0; t < K - 1; ++t) {
+        if (t < s.L) {
+            if (rs != nullptr && rs[t] != 0) open = false;
+            if (open) {  // no restart so far: the window is the state's rows and inputs 0 .. t, none zeroed
+                float a[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) a[i] = bias[i];
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    const int ts = t - (K - 1) + k;
+                    if (ts >= 0) {
+                        const Pack8<T> p = Pack8<T>::load(row0 + (size_t)ts * s.ld);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) a[i] += w[i][k] * p.get(i);
+                    } else if (state_in != nullptr) {
+                        const Pack8<T> p = Pack8<T>::load(state_in + ((size_t)b * (K - 1) + (K - 1 + ts)) * C + c0);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) a[i] += w[i][k] * p.get(i);
+                    }
+                }
+                const Pack8<T> g = Pack8<T>::load(gsrc + (size_t)t * gstride);
+#pragma unroll
+                for (int jr = 0; jr < K - 1; ++jr) {
+                    const int k = jr - t;  // tap of input s = jr - (K-1) in output t
+                    if (k >= 0) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) acc[jr][i] += w[i][k] * (g.get(i) * dsilu(a[i]));
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int jr = 0; jr < K - 1; ++jr) {
+        const int sidx = jr - (K - 1);
+        // rows of the old state that are still part of the new one (fewer than K-1 new timesteps)
+        if (dstate_out != nullptr && sidx >= s.L - (K - 1)) {
+            bool kept = true;
+            for (int t = 0; t < s.L; ++t) kept = kept && !(rs != nullptr && rs[t] != 0);
+            if (kept) {
+                const Pack8<T> p = Pack8<T>::load(dstate_out + ((size_t)b * (K - 1) + (sidx - (s.L - (K - 1)))) * C + c0);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[jr][i] += p.get(i);
+            }
+        }
+        Pack8<T>::store(dstate_in + ((size_t)b * (K - 1) + jr) * C + c0, acc[jr]);
     }
 }
 
@@ -389,8 +503,8 @@ size_t block_bwd_workspace_bytes(const BlockShape &s) {
     const size_t DI = (size_t)s.H * s.P, C = DI + 2 * (size_t)s.G * s.N;
     const size_t runs = (s.L + kBwdSteps - 1) / kBwdSteps;
     const size_t run_blocks = ((size_t)s.B * runs + kRunsPerBlock - 1) / kRunsPerBlock;
-    const size_t post = (size_t)kPostBlocks * DI;
-    const size_t pre = (run_blocks + 1) * C * (s.d_conv + 1) + (size_t)kDtBlocks * s.H;
+    const size_t post = (size_t)(kPostBlocks + kSumShares) * DI;
+    const size_t pre = (run_blocks + 1 + kSumShares) * C * (s.d_conv + 1) + (size_t)(kDtBlocks + kSumShares) * s.H;
     return sizeof(float) * (post > pre ? post : pre);  // the two stages run one after the other and share it
 }
 
@@ -415,8 +529,7 @@ static hipError_t post_bwd_dispatch(const BlockShape &s, const void *y, const vo
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    column_sums_kernel<<<dim3((DI + 255) / 256), dim3(256), 0, st>>>(part, blocks, DI, dnorm_w);
-    return hipGetLastError();
+    return launch_column_sums(part, blocks, DI, part + (size_t)kPostBlocks * DI, dnorm_w, st);
 }
 
 hipError_t launch_block_post_bwd(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
@@ -436,7 +549,7 @@ static hipError_t pre_bwd_dispatch(const BlockShape &s, const void *zxbcdt, cons
                                    const void *dB, const void *dC, const void *ddt, const void *dstate_out, void *dzxbcdt,
                                    float *dconv_w, float *dconv_b, float *ddt_bias, void *dstate_in, float *part,
                                    hipStream_t st) {
-    const int DI = s.H * s.P, C = DI + 2 * s.G * s.N, CP = C / 8, K = s.d_conv;
+    const int DI = s.H * s.P, C = DI + 2 * s.G * s.N, CP = C / kBwdCh, K = s.d_conv;
     const long long runs = (s.L + kBwdSteps - 1) / kBwdSteps;
     const long long run_blocks = ((long long)s.B * runs + kRunsPerBlock - 1) / kRunsPerBlock;
     if (run_blocks > 65535LL * 32768LL) return hipErrorInvalidValue;
@@ -445,26 +558,35 @@ static hipError_t pre_bwd_dispatch(const BlockShape &s, const void *zxbcdt, cons
     const T *gx = static_cast<const T *>(dx), *gb = static_cast<const T *>(dB), *gc = static_cast<const T *>(dC);
     const T *gso = static_cast<const T *>(dstate_out);
     T *out = static_cast<T *>(dzxbcdt), *gsi = static_cast<T *>(dstate_in);
+    const dim3 sgrid((unsigned)(((long long)s.B * (C / 8) + 255) / 256));
     switch (K) {
-        case 2: block_pre_bwd_kernel<T, 2><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, gsi, part, s); break;
-        case 3: block_pre_bwd_kernel<T, 3><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, gsi, part, s); break;
-        case 4: block_pre_bwd_kernel<T, 4><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, gsi, part, s); break;
+        case 2:
+            block_pre_bwd_kernel<T, 2><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            if (gsi) block_pre_bwd_state_kernel<T, 2><<<sgrid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, gsi, s);
+            break;
+        case 3:
+            block_pre_bwd_kernel<T, 3><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            if (gsi) block_pre_bwd_state_kernel<T, 3><<<sgrid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, gsi, s);
+            break;
+        case 4:
+            block_pre_bwd_kernel<T, 4><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            if (gsi) block_pre_bwd_state_kernel<T, 4><<<sgrid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, gsi, s);
+            break;
         default: return hipErrorInvalidValue;
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     // the partials hold, per run block, [C][K+1] = (dw[0..K-1], db): sum the columns, then split them
     const int cols = C * (K + 1);
-    float *sums = part + (size_t)run_blocks * cols;  // (behind the partials: cols floats)
-    column_sums_kernel<<<dim3((cols + 255) / 256), dim3(256), 0, st>>>(part, (int)run_blocks, cols, sums);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    float *dt_part = sums + cols;
+    float *sums = part + (size_t)run_blocks * cols;  // (behind the partials: cols floats, then the shares' sums)
+    float *tmp = sums + cols;
+    if ((e = launch_column_sums(part, (int)run_blocks, cols, tmp, sums, st)) != hipSuccess) return e;
+    float *dt_part = tmp + (size_t)kSumShares * cols;
     const long long rows = (long long)s.B * s.L;
     const int dt_blocks = (int)std::min<long long>(kDtBlocks, rows);
     block_dt_bwd_kernel<T><<<dim3(dt_blocks), dim3(256), 0, st>>>(in, dt_bias, static_cast<const T *>(ddt), out, dt_part, s);
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    column_sums_kernel<<<dim3((s.H + 255) / 256), dim3(256), 0, st>>>(dt_part, dt_blocks, s.H, ddt_bias);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
+    if ((e = launch_column_sums(dt_part, dt_blocks, s.H, dt_part + (size_t)kDtBlocks * s.H, ddt_bias, st)) != hipSuccess) return e;
     split_conv_sums_kernel<<<dim3((C + 255) / 256), dim3(256), 0, st>>>(sums, C, K, dconv_w, dconv_b);
     return hipGetLastError();
 }
