@@ -49,6 +49,24 @@ def _lib():
     return lib
 
 
+def _weight_gradient(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """a^T b in float32 for tall a [rows, E] (its rows may be a view into wider ones) and b [rows, D]: a sum over all
+    rows of the batch and the sequence.  As one GEMM the BLAS behind torch sees a contraction hundreds of thousands
+    long against outputs a few hundred wide and runs it at a fifth of its rate, so the rows are cut into equal slabs,
+    multiplied as one batched GEMM with float32 outputs, and the slabs' products added in order (measured on MI355X,
+    524 288 rows: 648 x 256 outputs 1 333 -> 232 us, 256 x 256 outputs 1 059 -> 129 us; the float32 partial products also
+    make the result more accurate than the single GEMM's bf16 output)."""
+    rows = a.shape[0]
+    slabs = 1
+    while slabs < 128 and rows % (2 * slabs) == 0 and rows // (2 * slabs) >= 4096:
+        slabs *= 2
+    if slabs == 1 or a.dtype == torch.float32:
+        return torch.matmul(a.t(), b).float()
+    a3 = a.unflatten(0, (slabs, rows // slabs))
+    b3 = b.unflatten(0, (slabs, rows // slabs))
+    return torch.bmm(a3.transpose(1, 2), b3, out_dtype=torch.float32).sum(0)
+
+
 def in_proj_width(nheads, headdim, dstate, ngroups) -> int:
     return 2 * nheads * headdim + 2 * ngroups * dstate + nheads
 
@@ -347,7 +365,7 @@ class Mamba2Block:
         w_out = self.out_proj.to(act)
         dout2 = dout.reshape(Bsz * L, self.d_model)
         dyn = torch.matmul(dout2, w_out).view(Bsz, L, self.d_inner)
-        dout_proj = torch.matmul(dout2.t(), yn.reshape(Bsz * L, self.d_inner)).float()
+        dout_proj = _weight_gradient(dout2, yn.reshape(Bsz * L, self.d_inner))
         # the gradient of zxbcdt, with zxbcdt's own (padded) row stride
         ld = _row_stride(zxbcdt)
         dbuf = torch.empty((Bsz, L, ld), dtype=act, device=u.device)
@@ -360,7 +378,7 @@ class Mamba2Block:
                                                       workspace=ws)
         dz2 = dbuf.view(Bsz * L, ld)[:, :E]
         du = torch.matmul(dz2, self.in_proj.to(act)).view(Bsz, L, self.d_model)
-        din_proj = torch.matmul(dz2.t(), u.reshape(Bsz * L, self.d_model)).float()
+        din_proj = _weight_gradient(dz2, u.reshape(Bsz * L, self.d_model))
         return dict(du=du, din_proj=din_proj, dconv_w=dconv_w, dconv_b=dconv_b, ddt_bias=ddt_bias, dA=g["dA"],
                     dA_log=g["dA"] * self.A, dD=g["dD"], dnorm_w=dnorm_w, dout_proj=dout_proj)
 
