@@ -350,6 +350,8 @@ def main():
             fl = sum(sf[k] for k in ("chunk_state", "chunk_scan"))   # dense MFMA flops of the op
             f32_onepass = ssd.chunk_scan_is_onepass(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk,
                                                     dtype=torch.float32)
+            f32_segments = ssd.chunk_scan_segments(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk,
+                                                   dtype=torch.float32)
             io32 = 4 * (2 * w.batch * w.seqlen * w.nheads * w.headdim + w.batch * w.seqlen * w.nheads +
                         2 * w.batch * w.seqlen * w.ngroups * w.dstate) + \
                 4 * w.batch * w.nheads * w.headdim * w.dstate * (2 if init is not None else 1)
@@ -368,7 +370,8 @@ def main():
             e32 = (orc.rel_err(y32o[:nb_err].cpu().numpy(), y_ref), orc.rel_err(f32o[:nb_err].cpu().numpy(), f_ref))
             del y_ref, f_ref
             out["forward_float32"] = {"ms": round(t32 * 1e3, 4),
-                                      "path": "one-pass (three bf16 terms per operand)" if f32_onepass else "staged",
+                                      "path": "one-pass (three bf16 terms per operand)" if f32_onepass
+                                      else (f"one-pass on {f32_segments} segments (three bf16 terms per operand)" if f32_segments > 1 else "staged"),
                                       "compulsory_io_bytes": io32,
                                       "hbm_frac": round(io32 / t32 / 1e9 / HBM_PEAK_GBS, 4),
                                       "dense_TFLOPs": round(fl / t32 / 1e12, 1), "peak_TFLOPs": MFMA_F32_PEAK_TFLOPS,

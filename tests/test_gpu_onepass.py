@@ -241,6 +241,35 @@ def test_mid_size_batches_run_cut_into_segments(seqlen, with_reset):
     assert rel_err(y32, np64(y1)) <= 1e-4 and rel_err(final, np64(f1)) <= 1e-4
 
 
+@pytest.mark.parametrize("with_reset", [False, True])
+def test_float32_mid_size_batches_run_cut_into_segments(with_reset):
+    """48 float32 sequences of 2048 steps: too few workgroups to fill the chip uncut, so the float one-pass kernel runs
+    on segments of the sequence (states-only pass, then the forward with the recurrence over the segment states in
+    its prologue).  Rows against the oracle at the float bar, and the whole against the uncut kernel."""
+    from trading_bot_0_amd.ssd import chunk_scan_segments
+    w = Workload("segments_f32", 48, 2048, 8, 32, 64, 1, 128, dtype="f32", init_std=0.5)
+    assert chunk_scan_segments(w.batch, w.seqlen, 8, 32, 64, 1, 128, dtype=torch.float32) >= 2
+    dev = make_inputs(w, seed=6, device="cuda")
+    reset = None
+    m = None
+    if with_reset:
+        m = (np.random.default_rng(3).random((w.batch, w.seqlen)) < 0.002).astype(np.uint8)
+        for t in (0, 511, 512, 513, 1024, 1535, 1536):
+            m[1, t] = 1
+        reset = torch.from_numpy(m).cuda()
+    y, final = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                              initial_states=dev["init"], reset=reset)
+    rows = [0, 1, 47]
+    yr, fr = orc.ssd_sequential(*(np64(dev[k][rows]) for k in ("x", "dt")), np64(dev["A"]), np64(dev["B"][rows]),
+                                np64(dev["C"][rows]), np64(dev["D"]), np64(dev["init"][rows]),
+                                reset=None if m is None else m[rows])
+    assert_close(y[rows], yr, torch.float32, "float segmented y")
+    assert_close(final[rows], fr, torch.float32, "float segmented final")
+    y1, f1 = ssd_chunk_scan_onepass(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                                    initial_states=dev["init"], reset=reset)
+    assert rel_err(y, np64(y1)) <= 1e-5 and rel_err(final, np64(f1)) <= 1e-5
+
+
 @pytest.mark.parametrize("batch,seqlen", [(288, 512), (272, 2048)])
 def test_partial_last_round_runs_as_a_batch_of_its_own(batch, seqlen):
     """256 workgroups fill the chip; the 32 or 16 sequences beyond run staged (short) or cut into segments (long)

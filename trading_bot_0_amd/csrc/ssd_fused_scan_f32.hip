@@ -94,11 +94,16 @@ __device__ inline f32x16 mma6(const Frag3 &a, const Frag3 &b, f32x16 c) {
     return c;
 }
 
-template <int NK, int WAVES>  // dstate N = 16 NK
+// STATES_ONLY: no outputs, no C: the state a segment of the sequence leaves behind from a zero state, into
+// final_states [B, segments, H, P, N], and the segment's total decay into seg_decay [B, segments, H] -- for sequences
+// cut into segments of s.seg_tiles tiles (of 32 steps here) that different workgroups walk side by side.  The
+// forward on segments (s.seg_local set) starts every segment from the recurrence over those states, run in its
+// workgroups' prologue, as in the bf16 kernel.
+template <int NK, int WAVES, bool STATES_ONLY>  // dstate N = 16 NK
 __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
     const float *__restrict__ x, const float *__restrict__ dt, const float *__restrict__ A, const float *__restrict__ Bm,
     const float *__restrict__ Cm, const float *__restrict__ D, const float *init, const unsigned char *__restrict__ reset,
-    float *__restrict__ y, float *final_states, ScanShape s) {
+    float *__restrict__ y, float *final_states, float *seg_decay, ScanShape s) {
     using T = __bf16;
     constexpr int N = 16 * NK, NB = NK / 2, Q = kFloatTile, nthr = 64 * WAVES;
     constexpr int XS = f32_xterm_elems(), XF = f32_xfloat_elems(), TB = f32_bcterm_elems(N), WF = f32_table_floats();
@@ -125,7 +130,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
     // ---- which units this workgroup owns (as the bf16 kernel) ----
     const int PBn = s.P / 32, HG = s.H / s.G;
     const int UW = (HG * PBn) / WAVES;
-    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int nc = (s.L + Q - 1) / Q;
+    const int S = s.seg_tiles > 0 ? (nc + s.seg_tiles - 1) / s.seg_tiles : 1;
+    const int slot = xcd_remap(blockIdx.x, gridDim.x);
+    const int seg = slot % S, logical = slot / S;
+    // states only: nothing comes after the last segment, its workgroups leave at once
+    if (STATES_ONLY && S > 1 && seg == S - 1) return;
+    const int c_first = seg * (s.seg_tiles > 0 ? s.seg_tiles : nc);
+    const int c_end = s.seg_tiles > 0 ? min(nc, c_first + s.seg_tiles) : nc;
     const int b = logical / (s.G * UW), g = (logical / UW) % s.G, unit0 = (logical % UW) * WAVES;
     const int unit = unit0 + wave, h = g * HG + unit / PBn, pb = unit % PBn;
     const int HP = s.H * s.P;
@@ -137,7 +149,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
     const unsigned ycol_bytes = (unsigned)((h * s.P + pb * 32) * sizeof(float));
     const float dh = D ? D[h] : 0.f;
     const double a_h = (double)A[h];
-    const int nc = (s.L + Q - 1) / Q;
 
     // ---- registers holding the next tile's inputs ----
     float4 xq[UX], bq, cq;
@@ -154,7 +165,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
         if (bc_thread && bc_row < rows) {
             const size_t o = (size_t)(t0 + bc_row) * s.G * N + bc_pc * 4;
             bq = *reinterpret_cast<const float4 *>(Bb + o);
-            cq = *reinterpret_cast<const float4 *>(Cb + o);
+            if (!STATES_ONLY) cq = *reinterpret_cast<const float4 *>(Cb + o);
         }
 #pragma unroll
         for (int u = 0; u < UX; ++u) {
@@ -172,8 +183,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
     // ---- running state: st[nb][v] = H[p = r, n = 32 nb + 8 (v/4) + 4 half + v%4] ----
     f32x16 st[NB];
     {
+        const bool folded = !STATES_ONLY && s.seg_local != nullptr;
         const bool fresh = rsb != nullptr && rsb[0] != 0;  // a restart before the first step: init is not read
-        const float *ib = init && !fresh ? init + ((((size_t)b * s.H + h) * s.P + pb * 32 + r) * N + 4 * half) : nullptr;
+        const size_t lane_off = (size_t)(pb * 32 + r) * N + 4 * half;
+        const float *ib = !STATES_ONLY && init && !fresh ? init + ((size_t)b * s.H + h) * s.P * N + lane_off : nullptr;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
@@ -185,12 +198,30 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
                 st[nb][4 * gq + 3] = v.w;
             }
         }
+        if (folded) {  // enter[j+1] = decay[j] * enter[j] + local[j] over the segments before this one
+            for (int j = 0; j < seg; ++j) {
+                const float a = s.seg_local_decay[((size_t)b * S + j) * s.H + h];
+                const float *lb = s.seg_local + (((size_t)b * S + j) * s.H + h) * s.P * N + lane_off;
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq) {
+                        const float4 v = *reinterpret_cast<const float4 *>(lb + 32 * nb + 8 * gq);
+                        st[nb][4 * gq + 0] = a * st[nb][4 * gq + 0] + v.x;
+                        st[nb][4 * gq + 1] = a * st[nb][4 * gq + 1] + v.y;
+                        st[nb][4 * gq + 2] = a * st[nb][4 * gq + 2] + v.z;
+                        st[nb][4 * gq + 3] = a * st[nb][4 * gq + 3] + v.w;
+                    }
+                }
+            }
+        }
     }
+    float seg_total = 1.f;  // product of the tiles' decays (states only)
 
     // where this thread's staged pieces go: 4 floats = one 8-byte piece of each term tile
     const int x_unit = x_pc / 8, x_col = (x_pc % 8) * 4;
-    prefetch(0);
-    for (int c = 0; c < nc; ++c) {
+    prefetch(c_first);
+    for (int c = c_first; c < c_end; ++c) {
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
         block_sync_lds();  // every wave is done reading the previous tile
@@ -198,12 +229,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
 #pragma unroll
         for (int u = 0; u < UX; ++u) {
             const int row = x_row0 + u * XROWS;
-            unsigned t3[3][2];
-            split3_pair(xq[u].x, xq[u].y, t3[0][0], t3[1][0], t3[2][0]);
-            split3_pair(xq[u].z, xq[u].w, t3[0][1], t3[1][1], t3[2][1]);
-            const int o = f32_xterm_base(x_unit) + XT::off(row, x_col);
+            if (!STATES_ONLY) {  // the term tiles of x serve phase 1 only
+                unsigned t3[3][2];
+                split3_pair(xq[u].x, xq[u].y, t3[0][0], t3[1][0], t3[2][0]);
+                split3_pair(xq[u].z, xq[u].w, t3[0][1], t3[1][1], t3[2][1]);
+                const int o = f32_xterm_base(x_unit) + XT::off(row, x_col);
 #pragma unroll
-            for (int t = 0; t < 3; ++t) *reinterpret_cast<uint2 *>(xt_all + t * WAVES * XS + o) = make_uint2(t3[t][0], t3[t][1]);
+                for (int t = 0; t < 3; ++t) *reinterpret_cast<uint2 *>(xt_all + t * WAVES * XS + o) = make_uint2(t3[t][0], t3[t][1]);
+            }
             float *xr = xf_all + f32_xfloat_base(x_unit);
             *reinterpret_cast<float2 *>(xr + xfloat_off(row, x_col)) = make_float2(xq[u].x, xq[u].y);
             *reinterpret_cast<float2 *>(xr + xfloat_off(row, x_col + 2)) = make_float2(xq[u].z, xq[u].w);
@@ -212,13 +245,15 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
             unsigned t3[3][2], u3[3][2];
             split3_pair(bq.x, bq.y, t3[0][0], t3[1][0], t3[2][0]);
             split3_pair(bq.z, bq.w, t3[0][1], t3[1][1], t3[2][1]);
-            split3_pair(cq.x, cq.y, u3[0][0], u3[1][0], u3[2][0]);
-            split3_pair(cq.z, cq.w, u3[0][1], u3[1][1], u3[2][1]);
+            if (!STATES_ONLY) {
+                split3_pair(cq.x, cq.y, u3[0][0], u3[1][0], u3[2][0]);
+                split3_pair(cq.z, cq.w, u3[0][1], u3[1][1], u3[2][1]);
+            }
             const int o = BT::off(bc_row, bc_pc * 4);
 #pragma unroll
             for (int t = 0; t < 3; ++t) {
                 *reinterpret_cast<uint2 *>(Bs + t * TB + o) = make_uint2(t3[t][0], t3[t][1]);
-                *reinterpret_cast<uint2 *>(Cs + t * TB + o) = make_uint2(u3[t][0], u3[t][1]);
+                if (!STATES_ONLY) *reinterpret_cast<uint2 *>(Cs + t * TB + o) = make_uint2(u3[t][0], u3[t][1]);
             }
         }
         // ---- scan of dt*A over the tile (float64 across the wave) and this unit's decay tables ----
@@ -243,11 +278,11 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
                 F_s[lane] = exp2_hw(fminf(-(hi + lo), 126.f)) * dtv;
             }
         }
-        if (c + 1 < nc) prefetch(c + 1);
+        if (c + 1 < c_end) prefetch(c + 1);
         block_sync_lds();  // tiles and tables are visible
 
         // ---- phase 1: y of this tile from the state entering it ----
-        {
+        if constexpr (!STATES_ONLY) {
             const bool fast = __builtin_amdgcn_readfirstlane(__float_as_int(span)) <= __float_as_int(kFloatFastSpan);
             Frag3 Cf[NK];  // C[l = r, n in the accumulator's row order]
 #pragma unroll
@@ -334,7 +369,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
         }
 
         // ---- phase 2: the state leaving this tile (nobody reads the one the last tile leaves unless asked) ----
-        if (c + 1 == nc && final_states == nullptr) break;
+        // (the forward's last tile of a segment other than the last, or of a call that asks for no final state)
+        if (!STATES_ONLY && c + 1 == c_end && !(final_states != nullptr && seg == S - 1)) break;
+        seg_total *= a_end;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) st[nb] = st[nb] * a_end;
 #pragma unroll
@@ -364,8 +401,8 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
         }
     }
 
-    if (final_states != nullptr) {
-        float *fb = final_states + (((size_t)b * s.H + h) * s.P + pb * 32 + r) * N + 4 * half;
+    if (STATES_ONLY || (final_states != nullptr && seg == S - 1)) {
+        float *fb = final_states + ((((size_t)b * (STATES_ONLY ? S : 1) + (STATES_ONLY ? seg : 0)) * s.H + h) * s.P + pb * 32 + r) * N + 4 * half;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
@@ -373,6 +410,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
                 *reinterpret_cast<float4 *>(fb + 32 * nb + 8 * gq) =
                     make_float4(st[nb][4 * gq], st[nb][4 * gq + 1], st[nb][4 * gq + 2], st[nb][4 * gq + 3]);
         }
+        if (STATES_ONLY && pb == 0 && lane == 0) seg_decay[((size_t)b * S + seg) * s.H + h] = seg_total;
     }
 }
 
@@ -381,25 +419,57 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
 // 8 when float inputs of this shape can run on the one-pass kernel (the waves per workgroup), else 0
 int fused_scan_f32_waves(const ScanShape &s) {
     if (s.P % 32 != 0 || (s.N != 32 && s.N != 64)) return 0;
-    if (s.mode != 0 || s.x_groups != 0 || s.seg_tiles != 0) return 0;
+    if (s.mode != 0 || s.x_groups != 0) return 0;
     const int units = (s.H / s.G) * (s.P / 32);
     if (units % 8 != 0) return 0;
     if ((long long)s.L * s.H * s.P * 4 >= (1LL << 31)) return 0;  // y rows go through a 32-bit-offset buffer descriptor
     return 8;
 }
 
+// s.seg_tiles (tiles of kFloatTile steps per segment, 0 = not cut) and s.seg_local / s.seg_local_decay as for the
+// bf16 kernel
 hipError_t launch_fused_scan_f32(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
                                  const void *Cm, const float *D, const float *init, const unsigned char *reset, void *y,
                                  float *final_states, hipStream_t st) {
     if (fused_scan_f32_waves(s) != 8) return hipErrorInvalidValue;
-    const int grid = s.B * s.G * ((s.H / s.G) * (s.P / 32) / 8);
+    const int nc = (s.L + kFloatTile - 1) / kFloatTile;
+    const int segments = s.seg_tiles > 0 ? (nc + s.seg_tiles - 1) / s.seg_tiles : 1;
+    if ((segments > 1) != (s.seg_local != nullptr)) return hipErrorInvalidValue;
+    const int grid = s.B * s.G * ((s.H / s.G) * (s.P / 32) / 8) * segments;
     const float *xx = static_cast<const float *>(x), *dd = static_cast<const float *>(dt);
     const float *bb = static_cast<const float *>(Bm), *cc = static_cast<const float *>(Cm);
     if (s.N == 64)
-        fused_scan_f32_kernel<4, 8><<<dim3(grid), dim3(512), 0, st>>>(xx, dd, A, bb, cc, D, init, reset, static_cast<float *>(y), final_states, s);
+        fused_scan_f32_kernel<4, 8, false><<<dim3(grid), dim3(512), 0, st>>>(xx, dd, A, bb, cc, D, init, reset, static_cast<float *>(y), final_states, nullptr, s);
     else
-        fused_scan_f32_kernel<2, 8><<<dim3(grid), dim3(512), 0, st>>>(xx, dd, A, bb, cc, D, init, reset, static_cast<float *>(y), final_states, s);
+        fused_scan_f32_kernel<2, 8, false><<<dim3(grid), dim3(512), 0, st>>>(xx, dd, A, bb, cc, D, init, reset, static_cast<float *>(y), final_states, nullptr, s);
     return hipGetLastError();
+}
+
+int fused_scan_f32_tile() { return kFloatTile; }
+
+// The float forward on `segments` segments of the sequence: the states-only pass, then the forward per segment
+// (seg_states [B, segments, H, P, N] and seg_decay [B, segments, H] floats of scratch).
+hipError_t launch_fused_scan_f32_segmented(const ScanShape &s, int segments, const void *x, const void *dt, const float *A,
+                                           const void *Bm, const void *Cm, const float *D, const float *init,
+                                           const unsigned char *reset, void *y, float *final_states, float *seg_states,
+                                           float *seg_decay, hipStream_t st) {
+    if (segments < 2 || fused_scan_f32_waves(s) != 8) return hipErrorInvalidValue;
+    const int nc = (s.L + kFloatTile - 1) / kFloatTile;
+    ScanShape t = s;
+    t.seg_tiles = (nc + segments - 1) / segments;
+    if ((nc + t.seg_tiles - 1) / t.seg_tiles != segments) return hipErrorInvalidValue;
+    const int grid = s.B * s.G * ((s.H / s.G) * (s.P / 32) / 8) * segments;
+    const float *xx = static_cast<const float *>(x), *dd = static_cast<const float *>(dt);
+    const float *bb = static_cast<const float *>(Bm);
+    if (s.N == 64)
+        fused_scan_f32_kernel<4, 8, true><<<dim3(grid), dim3(512), 0, st>>>(xx, dd, A, bb, bb, nullptr, nullptr, reset, nullptr, seg_states, seg_decay, t);
+    else
+        fused_scan_f32_kernel<2, 8, true><<<dim3(grid), dim3(512), 0, st>>>(xx, dd, A, bb, bb, nullptr, nullptr, reset, nullptr, seg_states, seg_decay, t);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    t.seg_local = seg_states;
+    t.seg_local_decay = seg_decay;
+    return launch_fused_scan_f32(t, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
 }
 
 }  // namespace ssd

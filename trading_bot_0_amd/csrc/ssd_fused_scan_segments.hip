@@ -29,11 +29,25 @@ int fused_scan_plan(const ScanShape &s, int dtype, int *segments) {
     *segments = 1;
     if (dtype == 0) {
         // float inputs: the one-pass kernel on three bf16 terms per operand walks a tile of 32 steps in about
-        // kFloatTileUs; the staged float kernels take about 1345 per 2048 units x 32 tiles of 64
+        // kFloatTileUs (states only: 0.45 of that); the staged float kernels take about 1345 per 2048 units x 32
+        // tiles of 64
         if (fused_scan_f32_waves(s) == 0) return 0;
         const long long groups = (long long)s.B * s.G * ((s.H / s.G) * (s.P / 32) / 8);
+        const int nc = (s.L + fused_scan_f32_tile() - 1) / fused_scan_f32_tile();
         const double staged = 20.0 + 1345.0 * ((double)groups * 8 * tiles_of(s)) / (2048.0 * 32.0);
-        const double whole = 5.0 + kFloatTileUs * ((s.L + 31) / 32) * (double)((groups + 255) / 256);
+        const double whole = 5.0 + kFloatTileUs * nc * (double)((groups + 255) / 256);
+        double cut = 1e30;
+        int S = 1;
+        while (groups * S < kSegmentTargetGroups && nc / (2 * S) >= 2 * kSegmentMinTiles) S *= 2;
+        if (S >= 2) {
+            const int seg_tiles = (nc + S - 1) / S;
+            S = (nc + seg_tiles - 1) / seg_tiles;
+            cut = 10.0 + 1.45 * kFloatTileUs * seg_tiles * (double)((groups * S + 255) / 256);
+        }
+        if (cut < whole && cut < staged) {
+            *segments = S;
+            return 2;
+        }
         return whole < staged ? 1 : 0;
     }
     const int waves = fused_scan_waves(s, dtype);
@@ -91,6 +105,9 @@ hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segmen
                                        const float *A, const void *Bm, const void *Cm, const float *D, const float *init,
                                        const unsigned char *reset, void *y, float *final_states, float *seg_states,
                                        float *seg_decay, hipStream_t st) {
+    if (dtype == 0)
+        return launch_fused_scan_f32_segmented(s, segments, x, dt, A, Bm, Cm, D, init, reset, y, final_states, seg_states,
+                                               seg_decay, st);
     if (segments < 2 || fused_scan_waves(s, dtype) != 8 || s.N == 128) return hipErrorInvalidValue;
     ScanShape t = s;
     t.Q = kOnePassTile;

@@ -88,6 +88,11 @@ int fused_scan_f32_waves(const ScanShape &s);
 hipError_t launch_fused_scan_f32(const ScanShape &s, const void *x, const void *dt, const float *A, const void *Bm,
                                  const void *Cm, const float *D, const float *init, const unsigned char *reset, void *y,
                                  float *final_states, hipStream_t st);
+int fused_scan_f32_tile();  // time steps per tile of the float one-pass kernel
+hipError_t launch_fused_scan_f32_segmented(const ScanShape &s, int segments, const void *x, const void *dt, const float *A,
+                                           const void *Bm, const void *Cm, const float *D, const float *init,
+                                           const unsigned char *reset, void *y, float *final_states, float *seg_states,
+                                           float *seg_decay, hipStream_t st);
 // fused_scan_plan: which way a forward of this shape runs fastest by the library's cost estimates: 0 = the
 // staged kernels, 1 = the one-pass kernel, 2 = the one-pass kernel on *segments segments.
 int fused_scan_plan(const ScanShape &s, int dtype, int *segments);
