@@ -85,7 +85,7 @@ def test_post_backward(shape, dtype):
 @pytest.mark.parametrize("shape", [(2, 50, 8, 32, 64, 1, 4), (3, 19, 8, 16, 16, 2, 3), (2, 33, 8, 32, 32, 1, 2),
                                    (3, 2, 8, 32, 64, 1, 4), (4, 1, 8, 32, 64, 1, 4), (2, 300, 16, 64, 128, 2, 4)])
 def test_pre_backward(shape, dtype):
-    """With and without a carried conv state, restarts (both sides of the kernel's runs of 16 steps, back to back, first
+    """With and without a carried conv state, restarts (both sides of the kernel's runs of 32 steps, back to back, first
     and last step) and a gradient on the returned conv state."""
     Bsz, L, H, P, N, G, K = shape
     p = params(H, P, N, G, K)
@@ -100,7 +100,7 @@ def test_pre_backward(shape, dtype):
     ddt = torch.randn(Bsz, L, H, generator=g).to(dtype).cuda()
     dso = torch.randn(Bsz, K - 1, C, generator=g).to(dtype).cuda()
     reset = torch.zeros(Bsz, L, dtype=torch.uint8)
-    for t in (0, 5, 6, 15, 16, 17, 31, 33, L - 1):
+    for t in (0, 5, 6, 15, 16, 17, 30, 31, 32, 33, 34, 63, 64, 65, 66, L - 1):
         if 0 <= t < L:
             reset[t % Bsz, t] = 1
     for state, rs, gso in ((None, None, None), (st, None, dso), (st, reset, dso), (None, reset, None)):
