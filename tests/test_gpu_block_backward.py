@@ -30,7 +30,9 @@ def check_act(out, ref, dtype, what):
     o = out.detach().float().cpu().numpy().astype(np.float64).reshape(ref.shape)
     rms = float(np.sqrt(np.mean(ref * ref)))
     assert np.isfinite(o).all(), what
-    if dtype == torch.float32:
+    if rms == 0.0:  # an all-zero reference (a gradient cut off by a restart): exactly zero
+        assert not o.any(), f"{what}: the reference is zero, the output is not"
+    elif dtype == torch.float32:
         e = np.abs(o - ref).max() / rms
         assert e <= 1e-4, f"{what}: {e:.3e}"
     else:
