@@ -143,9 +143,11 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
  * tight serving loops, harnesses that forbid hipMalloc -- and so cannot bring a workspace: the scratch the staged and
  * segmented paths need comes from an array of SSD_STATIC_SCRATCH_BYTES (64 MiB) that is part of the library's device
  * code (each GPU the library runs on holds it until the process ends).  No counterpart in the reference.  Same
- * arguments and results as ssd_chunk_scan_reset_fwd minus the workspace.  Shapes whose workspace (ssd_workspace_bytes)
- * exceeds the array return SSD_ERR_WORKSPACE, except those that run as one launch of the one-pass kernel
- * (ssd_chunk_scan_is_onepass), which need no scratch at any size.  Calls no hipMalloc/hipFree or any other allocating
+ * arguments and results as ssd_chunk_scan_reset_fwd minus the workspace.  SSD_ERR_WORKSPACE when the scratch that the
+ * shape's own path uses exceeds the array: all of ssd_workspace_bytes on the staged kernels, the segment states and
+ * decays (batch * segments * nheads * (headdim * dstate + 1) floats) when the sequences run cut into segments
+ * (ssd_chunk_scan_segments > 1), nothing when the shape runs as one launch of the one-pass kernel
+ * (ssd_chunk_scan_is_onepass), at any size.  Calls no hipMalloc/hipFree or any other allocating
  * routine.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different streams or
  * threads) race on it; calls on one stream are ordered and safe.  Nothing in the array has to start at zero (every
  * kernel writes what it later reads), so it is not cleared between calls. */

@@ -71,6 +71,19 @@ CASES = [
 ]
 
 
+def test_noalloc_forward_takes_a_mid_size_batch_whose_staged_workspace_would_not_fit():
+    """64 sequences of 4096 steps: ssd_workspace_bytes (laid out for the staged kernels) is 168 MB, but the shape runs
+    on segments of the sequence and needs the segment states only (13 MB), which the static array holds."""
+    lib = ssd.load_library()
+    torch.cuda.set_device(0)
+    prime(lib)
+    w = WORKLOADS["decay_extreme"]
+    assert ssd.chunk_scan_segments(w.batch, w.seqlen, w.nheads, w.headdim, w.dstate, w.ngroups, w.chunk) > 1
+    need = run_pair(lib, w, w.seqlen, with_reset=True, with_init=True)
+    assert need > (64 << 20)
+    run_pair(lib, w.with_batch(40), 2048, with_reset=False, with_init=False)
+
+
 @pytest.mark.parametrize("name,first,second", CASES)
 def test_noalloc_forward_equals_the_workspace_forward_twice_in_a_row(name, first, second):
     lib = ssd.load_library()

@@ -380,6 +380,23 @@ int ssd_chunk_scan_fwd(const ssd_dims *dims, int dtype, const void *x, const voi
                                     workspace, workspace_bytes, hip_stream);
 }
 
+// Scratch of the forward on segments: the segments' decays [B, S, H], then their states [B, S, H, P, N] (fewer than the
+// chunk states the workspace is sized for)
+size_t segment_decay_bytes(const ssd::ScanShape &s, int segments) {
+    return align_up((size_t)s.B * segments * s.H * sizeof(float), 256);
+}
+
+// What the forward of this shape uses of its workspace: nothing as one launch of the one-pass kernel, the segment
+// states and decays on segments, everything carve() lays out on the staged kernels (or with a partial last round).
+size_t scan_scratch_bytes(const ssd::ScanShape &s, int dtype) {
+    int segments = 1;
+    const int plan = ssd::fused_scan_plan(s, dtype, &segments);
+    if (plan == 1 && ssd::fused_scan_tail_rows(s, dtype) == 0) return 0;
+    if (plan == 2)
+        return segment_decay_bytes(s, segments) + (size_t)s.B * segments * s.H * s.P * s.N * sizeof(float);
+    return carve(s).total;
+}
+
 // The forward proper, arguments checked: the way the plan says for this shape, with `workspace` (carve(s).total bytes,
 // or anything at all when scan_scratch_bytes says the shape needs none) as scratch.
 static int scan_forward(const ssd::ScanShape &s, int dtype, const void *x, const void *dt, const float *A, const void *Bm,
@@ -404,8 +421,10 @@ static int scan_forward(const ssd::ScanShape &s, int dtype, const void *x, const
             // too few sequences for one workgroup per 8 units to fill the chip, but long ones: the one-pass kernel
             // on segments of the sequence; the segment states (fewer than the chunk states) and decays use the
             // workspace
+            float *seg_decay = reinterpret_cast<float *>(base);
+            float *seg_states = reinterpret_cast<float *>(base + segment_decay_bytes(part, segments));
             e = ssd::launch_fused_scan_segmented(part, dtype, segments, px, pdt, A, pb, pc, D, pinit, preset, py, pfinal,
-                                                 states, dtcs, st);
+                                                 seg_states, seg_decay, st);
             return e == hipSuccess ? SSD_OK : hip_fail(e, "segmented one-pass scan launch");
         }
         return run_staged(part, dtype, px, pdt, A, pb, pc, D, pinit, preset, 0, py, pfinal, dtcs, states, st);
@@ -466,9 +485,7 @@ int ssd_chunk_scan_noalloc_fwd(const ssd_dims *dims, int dtype, const void *x, c
                                const uint8_t *reset, void *y, float *final_states, void *hip_stream) {
     ssd::ScanShape s;
     if (int rc = make_shape(dims, dtype, &s)) return rc;
-    // what the forward of this shape would carve out of a caller's workspace: nothing when it runs as one launch of
-    // the one-pass kernel
-    const size_t need = (takes_one_pass(s, dtype) && ssd::fused_scan_tail_rows(s, dtype) == 0) ? 0 : carve(s).total;
+    const size_t need = scan_scratch_bytes(s, dtype);
     if (need > kStaticScratchBytes)
         return fail(SSD_ERR_WORKSPACE,
                     "ssd: this shape needs %zu bytes of scratch, the library's static scratch array holds %zu; call "
