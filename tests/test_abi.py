@@ -211,7 +211,7 @@ def test_stage1_lds_bound_on_nheads(lib):
 def test_noalloc_entry_rejects_shapes_beyond_its_scratch(lib):
     """Validation happens before the device is touched: a staged shape whose workspace exceeds the static array
     is refused with the sizes in the message."""
-    d = dims(batch=64, seqlen=4096, nheads=8, headdim=32, dstate=64, chunk=128)   # float32: staged, 150 MB
+    d = dims(batch=256, seqlen=2048, nheads=8, headdim=16, dstate=64, chunk=128)   # heads of 16: staged, 200 MB
     need = c_size_t(0)
     assert lib.ssd_workspace_bytes(byref(d), byref(need)) == 0 and need.value > (64 << 20)
     args = [FAKE] * 5 + [None, None, None, FAKE, None]   # x dt A B C D init reset y final
