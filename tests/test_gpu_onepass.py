@@ -270,22 +270,26 @@ def test_float32_mid_size_batches_run_cut_into_segments(with_reset):
     assert rel_err(y, np64(y1)) <= 1e-5 and rel_err(final, np64(f1)) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
 @pytest.mark.parametrize("batch,seqlen", [(288, 512), (272, 2048)])
-def test_partial_last_round_runs_as_a_batch_of_its_own(batch, seqlen):
+def test_partial_last_round_runs_as_a_batch_of_its_own(batch, seqlen, dtype):
     """256 workgroups fill the chip; the 32 or 16 sequences beyond run staged (short) or cut into segments (long)
     after the whole round.  Rows of both parts against the oracle, and the whole against the uncut kernel."""
-    w = Workload("tail", batch, seqlen, 8, 32, 64, 1, 128, init_std=0.5)
+    w = Workload("tail", batch, seqlen, 8, 32, 64, 1, 128, dtype=dtype, init_std=0.5)
+    td = w.torch_dtype
     dev = make_inputs(w, seed=9, device="cuda")
     m = (np.random.default_rng(5).random((batch, seqlen)) < 0.002).astype(np.uint8)
     reset = torch.from_numpy(m).cuda()
+    yd = torch.float32 if dtype == "bf16" else None
     y32, final = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
-                                initial_states=dev["init"], y_dtype=torch.float32, reset=reset)
+                                initial_states=dev["init"], y_dtype=yd, reset=reset)
     rows = [0, 255, 256, batch - 1]
     yr, fr = orc.ssd_sequential(*(np64(dev[k][rows]) for k in ("x", "dt")), np64(dev["A"]), np64(dev["B"][rows]),
                                 np64(dev["C"][rows]), np64(dev["D"]), np64(dev["init"][rows]), reset=m[rows])
-    assert_close(y32[rows], yr, torch.bfloat16, "tail y (float32 y)")
-    assert_close(final[rows], fr, torch.bfloat16, "tail final")
+    assert_close(y32[rows], yr, td, "tail y (float32 y)")
+    assert_close(final[rows], fr, td, "tail final")
     y1, f1 = ssd_chunk_scan_onepass(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
-                                    initial_states=dev["init"], y_dtype=torch.float32, reset=reset)
+                                    initial_states=dev["init"], y_dtype=yd, reset=reset)
     assert torch.equal(y32[:256], y1[:256]) and torch.equal(final[:256], f1[:256])     # the whole round is that kernel
-    assert rel_err(y32[256:], np64(y1[256:])) <= 1e-4 and rel_err(final[256:], np64(f1[256:])) <= 1e-4
+    tol = 1e-4 if dtype == "bf16" else 1e-5
+    assert rel_err(y32[256:], np64(y1[256:])) <= tol and rel_err(final[256:], np64(f1[256:])) <= tol

@@ -78,8 +78,8 @@ int fused_scan_plan(const ScanShape &s, int dtype, int *segments) {
 // its own (by the plan's estimates) than as one more round: the rows of that remainder, else 0.
 int fused_scan_tail_rows(const ScanShape &s, int dtype) {
     int segments;
-    if (dtype == 0 || fused_scan_plan(s, dtype, &segments) != 1) return 0;
-    const int full = s.N == 128 ? 4 : 8;
+    if (fused_scan_plan(s, dtype, &segments) != 1) return 0;
+    const int full = (dtype != 0 && s.N == 128) ? 4 : 8;
     const int per_row = s.G * ((s.H / s.G) * (s.P / 32) / full);  // workgroups per batch row
     const long long groups = (long long)s.B * per_row;
     if (groups <= 256 || 256 % per_row != 0) return 0;
@@ -87,18 +87,29 @@ int fused_scan_tail_rows(const ScanShape &s, int dtype) {
     if (rest == 0) return 0;
     ScanShape tail = s;
     tail.B = rest / per_row;
-    const int nc = tiles_of(s);
     const int tail_plan = fused_scan_plan(tail, dtype, &segments);
-    double cost;  // of the remainder as its own batch, as fused_scan_plan estimates it
-    if (tail_plan == 2) {
-        const int seg_tiles = (nc + segments - 1) / segments;
-        cost = 15.0 + 1.4 * 6.5 * seg_tiles * (double)(((long long)rest * segments + 255) / 256);
-    } else if (tail_plan == 0) {
-        cost = 20.0 + 510.0 * ((double)rest * full * nc) / (2048.0 * 32.0) * (s.N == 128 ? 2.0 : 1.0);
+    if (tail_plan == 1) return 0;  // it would run as a round of the one-pass kernel anyway
+    double cost, round;  // of the remainder as its own batch, as fused_scan_plan estimates it; of one more round
+    if (dtype == 0) {
+        const int nc = (s.L + fused_scan_f32_tile() - 1) / fused_scan_f32_tile();
+        round = kFloatTileUs * nc;
+        if (tail_plan == 2) {
+            const int seg_tiles = (nc + segments - 1) / segments;
+            cost = 10.0 + 1.45 * kFloatTileUs * seg_tiles * (double)(((long long)rest * segments + 255) / 256);
+        } else {
+            cost = 20.0 + 1345.0 * ((double)rest * 8 * tiles_of(s)) / (2048.0 * 32.0);
+        }
     } else {
-        return 0;  // it would run as a round of the one-pass kernel anyway
+        const int nc = tiles_of(s);
+        round = 6.5 * nc;
+        if (tail_plan == 2) {
+            const int seg_tiles = (nc + segments - 1) / segments;
+            cost = 15.0 + 1.4 * 6.5 * seg_tiles * (double)(((long long)rest * segments + 255) / 256);
+        } else {
+            cost = 20.0 + 510.0 * ((double)rest * full * nc) / (2048.0 * 32.0) * (s.N == 128 ? 2.0 : 1.0);
+        }
     }
-    return cost < 6.5 * nc ? tail.B : 0;
+    return cost < round ? tail.B : 0;
 }
 
 hipError_t launch_fused_scan_segmented(const ScanShape &s, int dtype, int segments, const void *x, const void *dt,
