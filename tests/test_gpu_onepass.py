@@ -177,11 +177,12 @@ def test_float32_large_batches_take_the_one_pass_path():
     assert torch.equal(y1, y2) and torch.equal(f1, f2)
 
 
-def test_one_pass_kernel_on_a_side_stream_and_inside_a_captured_graph():
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_one_pass_kernel_on_a_side_stream_and_inside_a_captured_graph(dtype):
     """Same contract as the staged kernels: nothing allocated, nothing synchronised, so the launch can be
     captured (the reference captures its update, trading_bots/src/torch/train/update.rs:206-330).  Replays
     are interleaved with eager work and each is checked."""
-    w = Workload("graph", 4, 320, 8, 32, 64, 1, 128, init_std=0.2)
+    w = Workload("graph", 4, 320, 8, 32, 64, 1, 128, dtype=dtype, init_std=0.2)
     dev = to_dev(make_inputs(w, seed=8))
     y_ref, f_ref = run(dev, 128)
     out, fin = torch.empty_like(dev["x"]), torch.empty(4, 8, 32, 64, device="cuda")
