@@ -341,3 +341,26 @@ def test_block_stages_inside_a_captured_graph():
         eager = chain()
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(captured, eager)), f"replay {i}"
+
+
+def test_graphed_step_equals_the_eager_step_on_every_replay():
+    """The block's step captured in a graph (no memset nodes: every kernel writes what it later reads) and replayed
+    with the program's own eager work between the replays; outputs and both states equal the eager step's bit for bit."""
+    blk = Mamba2Block(d_model=256, nheads=8, headdim=32, dstate=64, seed=3)
+    g = torch.Generator().manual_seed(5)
+    prefix = torch.randn(4, 40, 256, generator=g).to(torch.bfloat16).cuda()
+    bars = torch.randn(6, 4, 256, generator=g).to(torch.bfloat16).cuda()
+    st_e, st_g = blk.new_state(4), blk.new_state(4)
+    blk.forward(prefix, state=st_e)
+    blk.forward(prefix, state=st_g)
+    conv0, ssm0 = st_g.conv.clone(), st_g.ssm.state.clone()
+    step = blk.graphed_step(st_g)
+    assert torch.equal(st_g.conv, conv0) and torch.equal(st_g.ssm.state, ssm0), "building the graph moved the state"
+    for i in range(bars.shape[0]):
+        out_e = blk.step(bars[i], st_e)
+        torch.cuda.synchronize()
+        out_g = step(bars[i]).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e), f"replay {i}: output"
+        assert torch.equal(st_g.conv, st_e.conv) and torch.equal(st_g.ssm.state, st_e.ssm.state), f"replay {i}: state"
+        _ = (prefix.float() * 2).sum().item()      # eager work and a synchronisation between the replays

@@ -17,5 +17,5 @@ from .ssd import (  # noqa: F401
     workspace_bytes,
 )
 from .stream_state import SsdStreamState  # noqa: F401
-from .block import (Mamba2Block, Mamba2StreamState, block_post, block_post_bwd, block_pre, block_pre_bwd,  # noqa: F401
+from .block import (GraphedBlockStep, Mamba2Block, Mamba2StreamState, block_post, block_post_bwd, block_pre, block_pre_bwd,  # noqa: F401
                     block_proj)

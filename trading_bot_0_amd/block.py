@@ -391,14 +391,61 @@ class Mamba2Block:
             return block_proj(u, w.contiguous(), pad_rows=pad_rows)
         return torch.matmul(u, w.t()).contiguous()
 
+    def _weights(self, dtype: torch.dtype):
+        """The two projection matrices in the activation dtype, converted once per dtype (and again when a master
+        copy has been modified in place)."""
+        key = (dtype, self.in_proj._version, self.out_proj._version, self.in_proj.data_ptr(), self.out_proj.data_ptr())
+        cached = getattr(self, "_weights_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, self.in_proj.to(dtype).contiguous(), self.out_proj.to(dtype).contiguous())
+            self._weights_cache = cached
+        return cached[1], cached[2]
+
     def step(self, u_t: torch.Tensor, state: Mamba2StreamState) -> torch.Tensor:
         """One timestep for every stream: u_t [B,d_model] -> [B,d_model]; advances `state` in place."""
         if u_t.dim() != 2 or u_t.shape[1] != self.d_model:
             raise ValueError(f"block step input must be [batch, {self.d_model}], got {tuple(u_t.shape)}")
-        dt_ = u_t.dtype
-        zxbcdt = torch.matmul(u_t, self.in_proj.to(dt_).t()).unsqueeze(1).contiguous()
+        w_in, w_out = self._weights(u_t.dtype)
+        zxbcdt = torch.matmul(u_t, w_in.t()).unsqueeze(1).contiguous()
         x, Bm, Cm, dt, _ = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N,
                                      self.G, conv_state=state.conv, conv_state_out=state.conv)  # in place
         y = state.ssm.step(x[:, 0], dt[:, 0], self.A, Bm[:, 0], Cm[:, 0], self.D)
         yn = block_post(y.unsqueeze(1), zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
-        return torch.matmul(yn[:, 0], self.out_proj.to(dt_).t())
+        return torch.matmul(yn[:, 0], w_out.t())
+
+    def graphed_step(self, state: Mamba2StreamState, dtype: torch.dtype = torch.bfloat16) -> "GraphedBlockStep":
+        """`step` for `state`'s streams captured once in a HIP graph and replayed per bar: at a few streams a step
+        is five launches of a few microseconds each and the host's time to issue them is what a step costs (the
+        reference captures its launch-bound loops the same way, trading_bots/src/torch/cuda/graph.rs)."""
+        return GraphedBlockStep(self, state, dtype)
+
+
+
+class GraphedBlockStep:
+    """A captured `Mamba2Block.step` over fixed buffers.  Calling it copies the bar's input into the captured input
+    buffer, replays the graph and returns the captured output buffer (overwritten by the next call).  The state it
+    was built for advances in place, as with `step`; the block's parameters are read at replay time, except the
+    projection matrices, whose activation-dtype copies are made at capture."""
+
+    def __init__(self, block: Mamba2Block, state: Mamba2StreamState, dtype: torch.dtype):
+        batch = state.conv.shape[0]
+        dev = state.conv.device
+        self.u = torch.zeros((batch, block.d_model), dtype=dtype, device=dev)
+        # what the warm-up steps below do to the state is undone afterwards
+        conv_keep, ssm_keep = state.conv.clone(), state.ssm.state.clone()
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            for _ in range(2):  # library handles, kernel modules and the weights' copies exist before the capture
+                block.step(self.u, state)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.out = block.step(self.u, state)
+        state.conv.copy_(conv_keep)
+        state.ssm.state.copy_(ssm_keep)
+
+    def __call__(self, u_t: torch.Tensor) -> torch.Tensor:
+        self.u.copy_(u_t)
+        self.graph.replay()
+        return self.out
