@@ -334,7 +334,7 @@ class Mamba2Block:
             raise ValueError(f"block input must be [batch, seqlen, {self.d_model}], got {tuple(u.shape)}")
         if reset is not None and state is not None:
             raise ValueError("restarts inside the window and a carried conv state cannot be combined")
-        zxbcdt = self._project(u, self.in_proj, pad_rows=True)  # internal to the block: rows of whole lines
+        zxbcdt = self._project(u, self._weights(u.dtype)[0], pad_rows=True)  # internal to the block: rows of whole lines
         if state is None:
             x, Bm, Cm, dt = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G,
                                       reset=reset)
@@ -346,7 +346,7 @@ class Mamba2Block:
             state.conv = conv
             y = state.ssm.init_from_prefix(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk)
         yn = block_post(y, zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
-        out = self._project(yn, self.out_proj)
+        out = self._project(yn, self._weights(u.dtype)[1])
         if save_for_backward:
             if state is not None:
                 raise ValueError("backward through a window that continues a carried state is not supported")
@@ -362,7 +362,7 @@ class Mamba2Block:
         Bsz, L, _ = u.shape
         act = u.dtype
         E = in_proj_width(self.H, self.P, self.N, self.G)
-        w_out = self.out_proj.to(act)
+        w_in, w_out = self._weights(act)
         dout2 = dout.reshape(Bsz * L, self.d_model)
         dyn = torch.matmul(dout2, w_out).view(Bsz, L, self.d_inner)
         dout_proj = _weight_gradient(dout2, yn.reshape(Bsz * L, self.d_inner))
@@ -377,7 +377,7 @@ class Mamba2Block:
                                                       g["dC"], g["ddt"], dzx, self.H, self.P, self.N, self.G, reset=reset,
                                                       workspace=ws)
         dz2 = dbuf.view(Bsz * L, ld)[:, :E]
-        du = torch.matmul(dz2, self.in_proj.to(act)).view(Bsz, L, self.d_model)
+        du = torch.matmul(dz2, w_in).view(Bsz, L, self.d_model)
         din_proj = _weight_gradient(dz2, u.reshape(Bsz * L, self.d_model))
         return dict(du=du, din_proj=din_proj, dconv_w=dconv_w, dconv_b=dconv_b, ddt_bias=ddt_bias, dA=g["dA"],
                     dA_log=g["dA"] * self.A, dD=g["dD"], dnorm_w=dnorm_w, dout_proj=dout_proj)
