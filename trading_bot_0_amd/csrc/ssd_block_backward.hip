@@ -477,7 +477,7 @@ __global__ __launch_bounds__(256) void block_dt_bwd_kernel(const T *__restrict__
         __syncthreads();
         red[threadIdx.x] = acc;
         __syncthreads();
-        if (threadIdx.x < hpt) {
+        if ((int)threadIdx.x < hpt) {
             float sum = 0.f;
             for (int q = 0; q < slots; ++q) sum += red[q * hpt + threadIdx.x];
             part[(size_t)blockIdx.x * s.H + h0 + threadIdx.x] = sum;
