@@ -158,11 +158,14 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
 // wave: the head's masked, decayed score tile -- the part of a tile's work that does not shrink with the state's
 // width -- and its B and C tiles are then formed and staged once instead of once per slice.  Their LDS holds two x
 // tiles and two tiles of the second operand of C . y, all tiles 8 elements apart instead of 16 to make room, and a
-// float tile per wave of 32 rows only: the workgroup writes its sums out after every block of 32 rows.
+// float tile per wave of 32 rows only: the workgroup writes its sums out after every block of 32 rows.  That tile's
+// rows are 64 floats with their 16-byte pieces XOR-swizzled by the row's low four bits, so that a lane's four
+// consecutive columns go out and come back as one 16-byte access and 16 consecutive rows of one logical piece
+// cover 256 bytes of banks.
 constexpr int wide_transposed_tile_elems(int Q) { return Q * 32 + 8; }
 constexpr size_t wide_transposed_scan_lds_bytes(int Q) {
     return (size_t)(2 * 8 + 4) * wide_transposed_tile_elems(Q) * 2 + (size_t)8 * ((5 + Q / 32) * Q * 4 + 64) +
-           (size_t)8 * 32 * 65 * 4;
+           (size_t)8 * 32 * 64 * 4;
 }
 constexpr size_t transposed_scan_lds_bytes(int Q) {
     return (size_t)(2 * 8 + 2) * fused_scan_xtile_elems(Q) * 2 + (size_t)8 * ((5 + Q / 32) * Q * 4 + 64) +
@@ -217,9 +220,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     T *aux_s = xs_all0 + SL * XS;  // transposed only (one tile per slice, behind the x tiles)
     float *wf0 = reinterpret_cast<float *>(TR ? xs_all0 + 2 * SL * XS : xs_all0 + SETS * WAVES * XS);
     float *wf = wf0 + wave * ((5 + QB) * Q + 16);
-    // transposed only: every head's output tile, [WAVES][Q][33], or [WAVES][32][65] with two slices per wave
+    // transposed only: every head's output tile, [WAVES][Q][33], or [WAVES][32][64] (swizzled) with two slices per wave
     float *red = wf0 + WAVES * ((5 + QB) * Q + 16);
-    constexpr int RS = SL == 2 ? 65 : 33;
+    constexpr int RS = SL == 2 ? 64 : 33;
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
     float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [8..8+QB): log2-decay across block lb
 
@@ -781,7 +784,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     for (int sl = 0; sl < SL; ++sl) {
                         float part = 0.f;  // forward: this slice's part of C_t . y_t
                         // where this lane's 16 elements of the head's tile go (two slices: tiles of 32 rows, side by side)
-                        float *rw = SL == 2 ? red + (wave * 32 + (le & 31)) * RS + sl * 32 : red + (wave * Q + ll) * RS;
+                        float *rw = SL == 2 ? red + (wave * 32 + (le & 31)) * RS : red + (wave * Q + ll) * RS;
 #pragma unroll
                         for (int vg = 0; vg < 4; ++vg) {
                             if (TR_FWD && aux != nullptr) {
@@ -789,8 +792,14 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
 #pragma unroll
                                 for (int i = 0; i < 4; ++i) part += accs[sl][vg * 4 + i] * (float)c4[i];
                             }
+                            if constexpr (SL == 2) {  // logical piece 8 sl + 2 vg + he of the row
+                                *reinterpret_cast<float4 *>(rw + 4 * ((8 * sl + 2 * vg + he) ^ (le & 15))) =
+                                    make_float4(wt * accs[sl][vg * 4], wt * accs[sl][vg * 4 + 1], wt * accs[sl][vg * 4 + 2],
+                                                wt * accs[sl][vg * 4 + 3]);
+                            } else {
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) rw[8 * vg + 4 * he + i] = wt * accs[sl][vg * 4 + i];
+                                for (int i = 0; i < 4; ++i) rw[8 * vg + 4 * he + i] = wt * accs[sl][vg * 4 + i];
+                            }
                         }
                         if (TR_FWD && seg_decay != nullptr) {  // (seg_decay: the per-head parts [B, L, H, P/32])
                             part += __shfl_xor(part, 32, 64);
@@ -806,11 +815,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                         float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
 #pragma unroll
                         for (int wv = 0; wv < WAVES; ++wv) {  // heads in order
-                            const float *rr = red + (wv * 32 + row) * RS + c4;
-                            v0 += rr[0];
-                            v1 += rr[1];
-                            v2 += rr[2];
-                            v3 += rr[3];
+                            const float4 rr = *reinterpret_cast<const float4 *>(red + (wv * 32 + row) * RS + 4 * ((tq & 15) ^ (row & 15)));
+                            v0 += rr.x;
+                            v1 += rr.y;
+                            v2 += rr.z;
+                            v3 += rr.w;
                         }
                         const int lr = lb * 32 + row;
                         const int orow = ADJ ? s.L - 1 - (t0 + lr) : t0 + lr;
