@@ -90,11 +90,8 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
                 }
             }
         }
-#pragma unroll
-        for (int m = LPR / 2; m >= 1; m >>= 1) {
-            ss += __shfl_xor(ss, m, 64);
-            gv += __shfl_xor(gv, m, 64);
-        }
+        ss = group_sum<LPR>(ss);
+        gv = group_sum<LPR>(gv);
         const float r = rsqrtf(ss * inv_di + eps);
         const float k3 = r * r * r * gv * inv_di;
 #pragma unroll

@@ -188,8 +188,7 @@ __global__ __launch_bounds__(256) void block_post_kernel(const TY *__restrict__ 
             }
         }
     }
-#pragma unroll
-    for (int m = LPR / 2; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
+    ss = group_sum<LPR>(ss);
     const float scale = rsqrtf(ss / (float)DI + eps);
 #pragma unroll
     for (int u = 0; u < MAXP; ++u) {

@@ -216,6 +216,23 @@ __device__ inline double wave_inclusive_scan(double v) {
     return v;
 }
 
+// Sum of v over aligned groups of NL consecutive lanes (NL = 4, 8, 16, 32 or 64), left in every lane of the group.
+// Inside a row of 16 lanes the data moves by DPP (quads, then the mirrored half row, then the mirrored row: no trip
+// through the LDS crossbar); wider groups take one lane exchange per doubling on top.
+template <int CTRL> __device__ inline float dpp_move_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int NL> __device__ inline float group_sum(float v) {
+    static_assert(NL == 4 || NL == 8 || NL == 16 || NL == 32 || NL == 64, "groups of 4, 8, 16, 32 or 64 lanes");
+    v += dpp_move_f<0xB1>(v);                           // quad_perm [1,0,3,2]
+    v += dpp_move_f<0x4E>(v);                           // quad_perm [2,3,0,1]
+    if constexpr (NL >= 8) v += dpp_move_f<0x141>(v);   // row_half_mirror: lane i <-> 7 - i of its half row
+    if constexpr (NL >= 16) v += dpp_move_f<0x140>(v);  // row_mirror: lane i <-> 15 - i of its row
+    if constexpr (NL >= 32) v += __shfl_xor(v, 16, 64);
+    if constexpr (NL >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
 // ------------------------------------------------------------------------------------------
 // Output columns of a transposed 32x32 accumulator tile, stored 16 bytes at a time
 // ------------------------------------------------------------------------------------------

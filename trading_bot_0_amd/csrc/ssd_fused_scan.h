@@ -209,7 +209,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // transposed: a B and a C tile [Q][32] per wave, then the shared x tile and the shared tile of the second
     // operand of the C . y products, each [Q][32].
     // (forward with two tile sets: B, B', C, C', the x tiles, the x tiles')
-        // (kind 5 spills ten registers with two sets and its early request of the next tile; with two sets and the late
+    // (kind 5 spills ten registers with two sets and its early request of the next tile; with two sets and the late
     // request the backward pass measured 1145 against 1123 us, so it keeps one set)
     constexpr bool kTwoSets = !TR && KIND != 5 && fused_scan_two_tile_sets(N, WAVES);
     constexpr int SETS = kTwoSets ? 2 : 1;
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // faster with bf16 y, 8 % with float y (217 against 222 us and 245 against 268 us at batch 256, 2048 steps, 8 heads
     // of 32, state 64).  The four-wave forward with a 128-wide state is 5 % slower with it and keeps the late request.
     // Of the backward pass's kinds, 5 and 6 take it without spilling (the pass 1.10 against 1.12 ms); 7 would spill.
-        constexpr bool kEarlyPrefetch = WAVES == 2 || (WAVES == 8 && (KIND == 0 || KIND == 5 || KIND == 6));
+    constexpr bool kEarlyPrefetch = WAVES == 2 || (WAVES == 8 && (KIND == 0 || KIND == 5 || KIND == 6));
     // (transposed: UX passes of the eight heads' B and C rows, one piece of the shared x tile and of the second
     // operand's tile)
     uint4 bq[TR ? UX : UBC], cq[TR ? UX : UBC], xq[TR ? 1 : UX], auxq = make_uint4(0, 0, 0, 0);
