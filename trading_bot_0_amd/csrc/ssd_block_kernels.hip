@@ -41,9 +41,11 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
         const T *src = zxbcdt + (size_t)bt * s.ld + 2 * DI + 2 * GN;
         if (s.H % 8 == 0) {  // eight heads are one aligned 16-byte (bf16) piece on both sides
             const Pack8<T> v = Pack8<T>::load(src + h0);
+            const float4 b0 = *reinterpret_cast<const float4 *>(dt_bias + h0), b1 = *reinterpret_cast<const float4 *>(dt_bias + h0 + 4);
+            const float bias[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
             float o[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = softplus(v.get(i) + dt_bias[h0 + i]);
+            for (int i = 0; i < 8; ++i) o[i] = softplus(v.get(i) + bias[i]);
             Pack8<T>::store(dt + (size_t)bt * s.H + h0, o);
             return;
         }
@@ -56,6 +58,35 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
     const int t1 = min(t0 + kPreSteps, s.L);
     const T *row0 = zxbcdt + ((size_t)b * s.L) * s.ld;  // this batch row's first timestep
     const int c0 = piece * 8;  // channel within [x | B | C]
+    // Every load of the thread is issued before the first is used and none is under a condition (a conditional load
+    // is a branch, and the compiler waits for all earlier loads -- and stores -- at every one): rows outside the
+    // sequence read a row inside it and are replaced by zeros or never stored.
+    // the run's input rows
+    Pack8<T> in[kPreSteps];
+#pragma unroll
+    for (int j = 0; j < kPreSteps; ++j) in[j] = Pack8<T>::load(row0 + (size_t)min(t0 + j, s.L - 1) * s.ld + DI + c0);
+    // the d_conv-1 rows before the run: rows of this call, of state_in, or zeros
+    Pack8<T> hist[DCONV - 1];
+#pragma unroll
+    for (int k = 0; k < DCONV - 1; ++k) {
+        const int ts = t0 - (DCONV - 1) + k;
+        const T *own = row0 + (size_t)max(ts, 0) * s.ld + DI + c0;
+        const T *old = state_in != nullptr ? state_in + ((size_t)b * (DCONV - 1) + max(DCONV - 1 + ts, 0)) * C + c0 : own;
+        hist[k] = Pack8<T>::load(ts >= 0 ? own : old);
+    }
+    // restart flags of the d_conv-2 steps before the run and of its own steps (bit j: step t0 - (DCONV-2) + j)
+    const unsigned char *rs = reset ? reset + (size_t)b * s.L : nullptr;
+    unsigned flags = 0;
+    if (rs != nullptr) {
+        unsigned char rv[kPreSteps + DCONV - 2];
+#pragma unroll
+        for (int j = 0; j < kPreSteps + DCONV - 2; ++j) rv[j] = rs[min(max(t0 - (DCONV - 2) + j, 0), s.L - 1)];
+#pragma unroll
+        for (int j = 0; j < kPreSteps + DCONV - 2; ++j) {
+            const int ts = t0 - (DCONV - 2) + j;
+            flags |= (ts >= 0 && ts < s.L && rv[j] != 0) ? (1u << j) : 0u;
+        }
+    }
     float w[8][DCONV], bias[8];
     {   // the taps of 8 consecutive channels are 8*DCONV consecutive floats
         float wf[8 * DCONV];
@@ -73,31 +104,21 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
             for (int k = 0; k < DCONV; ++k) w[i][k] = wf[i * DCONV + k];
         }
     }
-    // win[k] = input row t - (DCONV-1) + k for the current t; the last slot is loaded per timestep
+    // win[k] = input row t - (DCONV-1) + k for the current t; the last slot is filled per timestep
     float win[DCONV][8];
 #pragma unroll
     for (int k = 0; k < DCONV - 1; ++k) {
         const int ts = t0 - (DCONV - 1) + k;
+        const bool have = ts >= 0 || state_in != nullptr;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) win[k][i] = 0.f;
-        if (ts >= 0) {
-            const Pack8<T> v = Pack8<T>::load(row0 + (size_t)ts * s.ld + DI + c0);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) win[k][i] = v.get(i);
-        } else if (state_in != nullptr) {
-            const Pack8<T> v = Pack8<T>::load(state_in + ((size_t)b * (DCONV - 1) + (DCONV - 1 + ts)) * C + c0);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) win[k][i] = v.get(i);
-        }
+        for (int i = 0; i < 8; ++i) win[k][i] = have ? hist[k].get(i) : 0.f;
     }
-    const unsigned char *rs = reset ? reset + (size_t)b * s.L : nullptr;
-    if (rs != nullptr) {
+    {
         // a restart at one of the d_conv-2 timesteps before this run cuts the window rows before it
         bool cut = false;
 #pragma unroll
-        for (int k = DCONV - 2; k >= 1; --k) {  // window row k is timestep t0 - (DCONV-1) + k
-            const int ts = t0 - (DCONV - 1) + k;
-            cut = cut || (ts >= 0 && rs[ts] != 0);
+        for (int k = DCONV - 2; k >= 1; --k) {  // window row k is timestep t0 - (DCONV-1) + k: flag bit k - 1
+            cut = cut || ((flags >> (k - 1)) & 1u) != 0;
             if (cut) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) win[k - 1][i] = 0.f;
@@ -116,17 +137,12 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
         dst = Cm + ((size_t)b * s.L) * GN + (c0 - DI - GN);
         dst_stride = GN;
     }
-    // all of the run's input rows are requested before the first is used
-    Pack8<T> in[kPreSteps];
-#pragma unroll
-    for (int j = 0; j < kPreSteps; ++j)
-        if (t0 + j < t1) in[j] = Pack8<T>::load(row0 + (size_t)(t0 + j) * s.ld + DI + c0);
 #pragma unroll
     for (int j = 0; j < kPreSteps; ++j) {
         const int t = t0 + j;
         if (t >= t1) break;
         const Pack8<T> v = in[j];
-        if (rs != nullptr && rs[t] != 0) {
+        if ((flags >> (j + DCONV - 2)) & 1u) {
 #pragma unroll
             for (int k = 0; k < DCONV - 1; ++k) {
 #pragma unroll
@@ -160,9 +176,12 @@ __global__ __launch_bounds__(256) void block_pre_kernel(const T *__restrict__ zx
 }
 
 // LPR lanes per (b, t) row, 64 / LPR rows per wave: out = rmsnorm(y * silu(z)) * weight over the H*P channels.
-// LPR is the smallest of 16, 32, 64 whose lanes cover the row with at most MAXP pieces of 8 channels each, so that
-// narrow rows (256 channels are 32 pieces) leave no lane idle.
-template <typename T, typename TY, int LPR>
+// LPR is the smallest of 16, 32, 64 whose lanes cover the row with at most 4 pieces of 8 channels each, so that
+// narrow rows (256 channels are 32 pieces) leave no lane idle; PPL is the number of pieces a lane holds.  All of a
+// lane's loads are issued before the first is used and none is under a condition -- a conditional load is a branch,
+// and the compiler waits for every earlier load at each one: a piece past the row's end reads the row's last piece
+// and counts as zeros, a row past the tensor reads row 0 and is not stored.
+template <typename T, typename TY, int LPR, int PPL>
 __global__ __launch_bounds__(256) void block_post_kernel(const TY *__restrict__ y, const T *__restrict__ zxbcdt,
                                                          const float *__restrict__ norm_w, float eps,
                                                          T *__restrict__ out, BlockShape s) {
@@ -172,33 +191,51 @@ __global__ __launch_bounds__(256) void block_post_kernel(const TY *__restrict__ 
     const bool live = row < (long long)s.B * s.L;  // (whole waves stay for the lane exchanges)
     const TY *yr = y + (size_t)(live ? row : 0) * DI;
     const T *zr = zxbcdt + (size_t)(live ? row : 0) * s.ld;
-    constexpr int MAXP = 4;  // pieces of 8 channels per lane kept in registers: 64 lanes cover H*P <= 2048
-    float v[MAXP][8];
+    Pack8<TY> yv[PPL];
+    Pack8<T> zv[PPL];
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    f4 wa[PPL], wb[PPL];
+#pragma unroll
+    for (int u = 0; u < PPL; ++u) {
+        const int c0 = min((u * LPR + lane) * 8, DI - 8);
+        yv[u] = Pack8<TY>::load(yr + c0);
+        zv[u] = Pack8<T>::load(zr + c0);
+    }
+#pragma unroll
+    for (int u = 0; u < PPL; ++u) {
+        const int c0 = min((u * LPR + lane) * 8, DI - 8);
+        wa[u] = *reinterpret_cast<const f4 *>(norm_w + c0);
+        wb[u] = *reinterpret_cast<const f4 *>(norm_w + c0 + 4);
+    }
+    // (named as inputs of one statement here, the weights cannot be requested later than this: left alone, the
+    // compiler moves their loads behind the arithmetic on y and z, a second trip to memory)
+    if constexpr (PPL == 1) asm volatile("" ::"v"(wa[0]), "v"(wb[0]));
+    if constexpr (PPL == 2) asm volatile("" ::"v"(wa[0]), "v"(wb[0]), "v"(wa[1]), "v"(wb[1]));
+    if constexpr (PPL == 3) asm volatile("" ::"v"(wa[0]), "v"(wb[0]), "v"(wa[1]), "v"(wb[1]), "v"(wa[2]), "v"(wb[2]));
+    if constexpr (PPL == 4)
+        asm volatile("" ::"v"(wa[0]), "v"(wb[0]), "v"(wa[1]), "v"(wb[1]), "v"(wa[2]), "v"(wb[2]), "v"(wa[3]), "v"(wb[3]));
+    float v[PPL][8];
     float ss = 0.f;
 #pragma unroll
-    for (int u = 0; u < MAXP; ++u) {
-        const int c0 = (u * LPR + lane) * 8;
-        if (c0 < DI) {
-            const Pack8<TY> yv = Pack8<TY>::load(yr + c0);
-            const Pack8<T> zv = Pack8<T>::load(zr + c0);
+    for (int u = 0; u < PPL; ++u) {
+        // (a factor, not a select: a select would put every element's exponential under a branch of its own)
+        const float in = (u * LPR + lane) * 8 < DI ? 1.f : 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                v[u][i] = yv.get(i) * silu(zv.get(i));
-                ss += v[u][i] * v[u][i];
-            }
+        for (int i = 0; i < 8; ++i) {
+            v[u][i] = in * yv[u].get(i) * silu(zv[u].get(i));
+            ss += v[u][i] * v[u][i];
         }
     }
     ss = group_sum<LPR>(ss);
     const float scale = rsqrtf(ss / (float)DI + eps);
 #pragma unroll
-    for (int u = 0; u < MAXP; ++u) {
+    for (int u = 0; u < PPL; ++u) {
         const int c0 = (u * LPR + lane) * 8;
-        if (c0 < DI && live) {
-            float o[8];
+        const float w[8] = {wa[u].x, wa[u].y, wa[u].z, wa[u].w, wb[u].x, wb[u].y, wb[u].z, wb[u].w};
+        float o[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = v[u][i] * scale * norm_w[c0 + i];
-            Pack8<T>::store(out + (size_t)row * DI + c0, o);
-        }
+        for (int i = 0; i < 8; ++i) o[i] = v[u][i] * scale * w[i];
+        if (c0 < DI && live) Pack8<T>::store(out + (size_t)row * DI + c0, o);
     }
 }
 
@@ -240,15 +277,20 @@ static hipError_t post_dispatch(const BlockShape &s, const void *y, const void *
     const TY *yy = static_cast<const TY *>(y);
     const T *zz = static_cast<const T *>(zxbcdt);
     T *oo = static_cast<T *>(out);
-    // the fewest lanes per row that keep a lane's pieces within what the kernel holds in registers for 64 lanes (4)
-    if (pieces <= 16 * 4) {
-        block_post_kernel<T, TY, 16><<<dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st>>>(yy, zz, norm_w, eps, oo, s);
-    } else if (pieces <= 32 * 4) {
-        block_post_kernel<T, TY, 32><<<dim3((unsigned)((rows * 32 + 255) / 256)), dim3(256), 0, st>>>(yy, zz, norm_w, eps, oo, s);
-    } else {
-        block_post_kernel<T, TY, 64><<<dim3((unsigned)((rows * 64 + 255) / 256)), dim3(256), 0, st>>>(yy, zz, norm_w, eps, oo, s);
+    // the fewest lanes per row that keep a lane's pieces within four, and the pieces a lane then holds
+    const int lpr = pieces <= 16 * 4 ? 16 : pieces <= 32 * 4 ? 32 : 64;
+    const int ppl = (pieces + lpr - 1) / lpr;
+    const dim3 grid((unsigned)((rows * lpr + 255) / 256)), block(256);
+#define SSD_POST_CASE(LPRv, PPLv)                                                                        \
+    if (lpr == LPRv && ppl == PPLv) {                                                                    \
+        block_post_kernel<T, TY, LPRv, PPLv><<<grid, block, 0, st>>>(yy, zz, norm_w, eps, oo, s);         \
+        return hipGetLastError();                                                                        \
     }
-    return hipGetLastError();
+    SSD_POST_CASE(16, 1) SSD_POST_CASE(16, 2) SSD_POST_CASE(16, 3) SSD_POST_CASE(16, 4)
+    SSD_POST_CASE(32, 3) SSD_POST_CASE(32, 4)
+    SSD_POST_CASE(64, 3) SSD_POST_CASE(64, 4)
+#undef SSD_POST_CASE
+    return hipErrorInvalidValue;
 }
 
 hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,

@@ -233,6 +233,25 @@ template <int NL> __device__ inline float group_sum(float v) {
     return v;
 }
 
+// The value lane u (0..7) of this lane's aligned group of NL lanes holds.  A group that is a whole row of 16 lanes
+// takes it by DPP (row_newbcast: lane u of every row to all of the row), any other by a lane exchange.
+template <int NL> __device__ inline float group_lane(float v, int u) {
+    if constexpr (NL == 16) {
+        switch (u) {  // u is a constant after unrolling
+            case 0: return dpp_move_f<0x150>(v);
+            case 1: return dpp_move_f<0x151>(v);
+            case 2: return dpp_move_f<0x152>(v);
+            case 3: return dpp_move_f<0x153>(v);
+            case 4: return dpp_move_f<0x154>(v);
+            case 5: return dpp_move_f<0x155>(v);
+            case 6: return dpp_move_f<0x156>(v);
+            default: return dpp_move_f<0x157>(v);
+        }
+    } else {
+        return __shfl(v, (int)(threadIdx.x & 63) / NL * NL + u, 64);
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Output columns of a transposed 32x32 accumulator tile, stored 16 bytes at a time
 // ------------------------------------------------------------------------------------------

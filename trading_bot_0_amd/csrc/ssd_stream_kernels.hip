@@ -164,60 +164,68 @@ __global__ __launch_bounds__(256) void step_kernel(float *__restrict__ state, co
                                                    const float *__restrict__ D, TO *__restrict__ y, StepShape s) {
     constexpr int N = NL * 4;
     constexpr int RPP = 64 / NL;  // rows per pass
-    // passes whose loads are issued together: a whole [32, 64] state (8 against 4: 86.4 against 88.0 us at batch
-    // 4096, 8 heads); never more than NL, so that lane u of a row's group can keep pass u's result
+    // passes whose loads are issued together: a whole [32, 64] state; never more than NL, so that lane u of a
+    // row's group can keep pass u's result
     constexpr int UN = NL < 8 ? NL : 8;
     const int lane = threadIdx.x & 63;
-    const long long bh = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (bh >= (long long)s.B * s.H) return;
-    const int b = (int)(bh / s.H), h = (int)(bh % s.H);
+    // the wave's (b, h), in scalar registers (the launcher keeps B * H below 2^31)
+    const int bh = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
+    if (bh >= s.B * s.H) return;
+    const int b = bh / s.H, h = bh - b * s.H;
     const int g = h / (s.H / s.G);
     const int nl = lane % NL, rl = lane / NL;
-    const float dtv = (float)dt[bh];
-    const float decay = expf(dtv * A[h]);
-    const float dh = D ? D[h] : 0.f;
-    float bv[4], cv[4];
-    load4(Bm + ((size_t)b * s.G + g) * N + nl * 4, bv);  // this lane's four state columns: one load each
-    load4(Cm + ((size_t)b * s.G + g) * N + nl * 4, cv);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) bv[i] *= dtv;
     float4 *st = reinterpret_cast<float4 *>(state) + (size_t)bh * s.P * NL;
     const T *xr = x + (size_t)bh * s.P;
     TO *yr = y + (size_t)bh * s.P;
-    for (int p0 = 0; p0 < s.P; p0 += RPP * UN) {
-        float4 hv[UN];
-        float xv[UN];
-        // the block's rows of x in one load: lane (rl, nl < UN) takes row p0 + nl * RPP + rl (the lane that stores
-        // that row's y below), and every pass fetches its row's value from that lane
-        const int pq = p0 + nl * RPP + rl;
-        const float xq = (nl < UN && pq < s.P) ? (float)xr[pq] : 0.f;
+    // Every load of a block of rows is issued before the first result is needed, none of them under a condition (a
+    // conditional load is a branch, and the compiler waits for all earlier loads at every one): rows past the state
+    // are read as its last row and never stored.  The block's rows of x are one load: lane (rl, nl < UN) takes row
+    // p0 + nl * RPP + rl (the lane that stores that row's y), and every pass fetches its row's value from that lane.
+    float4 hv[UN];
+    float xq;
+    auto load_block = [&](int p0) {
+        const bool whole = p0 + RPP * UN <= s.P;  // uniform
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const int p = p0 + u * RPP + rl;
-            if (p < s.P) hv[u] = st[(size_t)p * NL + nl];
+            hv[u] = st[(size_t)(whole ? p : min(p, s.P - 1)) * NL + nl];
         }
+        xq = (float)xr[min(p0 + nl * RPP + rl, s.P - 1)];
+    };
+    // the step's scalars and this lane's four columns of B and C are requested first and used after the first block
+    // of the state has been requested, so that the state's loads do not wait for them
+    const T dt_raw = dt[bh];
+    const float a_h = A[h];
+    const float dh = D ? D[h] : 0.f;
+    float bv[4], cv[4];
+    load4(Bm + ((size_t)b * s.G + g) * N + nl * 4, bv);
+    load4(Cm + ((size_t)b * s.G + g) * N + nl * 4, cv);
+    load_block(0);
+    const float dtv = (float)dt_raw;
+    const float decay = expf(dtv * a_h);
 #pragma unroll
-        for (int u = 0; u < UN; ++u) xv[u] = __shfl(xq, rl * NL + u, 64);
+    for (int i = 0; i < 4; ++i) bv[i] *= dtv;
+    for (int p0 = 0; p0 < s.P; p0 += RPP * UN) {
+        if (p0 != 0) load_block(p0);
+        const bool whole = p0 + RPP * UN <= s.P;
+        float xv[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) xv[u] = group_lane<NL>(xq, u);
         float keep = 0.f;  // lane u of a row's group: y of the row of pass u
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const int p = p0 + u * RPP + rl;
-            float part = 0.f;
-            if (p < s.P) {
-                float4 v = hv[u];
-                v.x = decay * v.x + xv[u] * bv[0];
-                v.y = decay * v.y + xv[u] * bv[1];
-                v.z = decay * v.z + xv[u] * bv[2];
-                v.w = decay * v.w + xv[u] * bv[3];
-                st[(size_t)p * NL + nl] = v;
-                part = v.x * cv[0] + v.y * cv[1] + v.z * cv[2] + v.w * cv[3];
-            }
-            part = group_sum<NL>(part);
+            float4 v = hv[u];
+            v.x = decay * v.x + xv[u] * bv[0];
+            v.y = decay * v.y + xv[u] * bv[1];
+            v.z = decay * v.z + xv[u] * bv[2];
+            v.w = decay * v.w + xv[u] * bv[3];
+            if (whole || p < s.P) st[(size_t)p * NL + nl] = v;
+            const float part = group_sum<NL>(v.x * cv[0] + v.y * cv[1] + v.z * cv[2] + v.w * cv[3]);
             if (nl == u) keep = part + dh * xv[u];
         }
-        // one store for the block's rows: lane (rl, nl < UN) holds row p0 + nl * RPP + rl
-        const int p = p0 + nl * RPP + rl;
-        if (nl < UN && p < s.P) yr[p] = (TO)keep;
+        const int pq = p0 + nl * RPP + rl;
+        if (nl < UN && pq < s.P) yr[pq] = (TO)keep;
     }
 }
 
@@ -339,6 +347,7 @@ static hipError_t step_dispatch(const StepShape &s, float *state, const void *x,
                                 const float *A, const void *Bm, const void *Cm, const float *D, void *y,
                                 hipStream_t st) {
     const long long pairs = (long long)s.B * s.H;
+    if (pairs > 0x7fffffffLL) return hipErrorInvalidValue;  // the kernel counts (b, h) pairs in an int
     const dim3 grid((unsigned)((pairs + 3) / 4)), block(256);
     const T *xx = static_cast<const T *>(x), *dd = static_cast<const T *>(dt);
     const T *bb = static_cast<const T *>(Bm), *cc = static_cast<const T *>(Cm);
