@@ -42,9 +42,16 @@ template <> struct PackCh<float> {
 constexpr int kPostBlocks = 1024;    // workgroups of post_bwd (each walks rows with a grid stride)
 
 // ---- post ----------------------------------------------------------------------------------------------------
-// LPR lanes per (b, t) row as in the forward; v = y silu(z), r = (mean v^2 + eps)^-1/2, g = dout w:
+// LPR lanes per (b, t) row as in the forward, PPL pieces of 8 channels per lane; v = y silu(z),
+// r = (mean v^2 + eps)^-1/2, g = dout w:
 //   dv = r g - r^3 v mean(g v);  dy = dv silu(z);  dz = dv y silu'(z);  dw += dout v r
-template <typename T, typename TY, int LPR>
+// No load is under a condition (a piece past the row's end reads the row's last piece and counts as zeros, a row past
+// the tensor reads the last row and is not stored), and a lane's next row is requested before this row's arithmetic
+// and stores: behind a conditional load the compiler waits for every earlier load and store.
+// EXACT: the lanes' pieces cover the row exactly.  Whole passes of the workgroup's rows then store without a
+// condition, so that the compiler can count the stores between a row's loads and their use instead of waiting for
+// all of them (the last, partial pass of the tensor runs the guarded code).
+template <typename T, typename TY, int LPR, int PPL, bool EXACT>
 __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restrict__ y, const T *__restrict__ zxbcdt,
                                                              const float *__restrict__ norm_w, float eps,
                                                              const T *__restrict__ dout, T *__restrict__ dy,
@@ -52,42 +59,69 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
                                                              BlockShape s) {
     const int DI = s.H * s.P;
     const int lane = threadIdx.x & (LPR - 1);
-    constexpr int MAXP = 4;
+    constexpr int MAXP = PPL;
     constexpr int RPB = 256 / LPR;  // rows per workgroup and pass
     const long long rows = (long long)s.B * s.L;
-    float wv[MAXP][8], dwacc[MAXP][8];
+    float wv[MAXP][8], dwacc[MAXP][8], in[MAXP];
+    int cc[MAXP];  // the piece this lane reads for slot u (the row's last piece where the slot lies past the row)
 #pragma unroll
     for (int u = 0; u < MAXP; ++u) {
         const int c0 = (u * LPR + lane) * 8;
+        in[u] = c0 < DI ? 1.f : 0.f;
+        cc[u] = min(c0, DI - 8);
+        const float4 wa = *reinterpret_cast<const float4 *>(norm_w + cc[u]), wb = *reinterpret_cast<const float4 *>(norm_w + cc[u] + 4);
+        const float wq[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            wv[u][i] = c0 < DI ? norm_w[c0 + i] : 0.f;
+            wv[u][i] = in[u] * wq[i];
             dwacc[u][i] = 0.f;
         }
     }
+    struct RowIn {
+        Pack8<TY> y[MAXP];
+        Pack8<T> z[MAXP], d[MAXP];
+    };
+    auto fetch = [&](long long row) {
+        RowIn o;
+        const size_t r_ = (size_t)min(row, rows - 1);
+#pragma unroll
+        for (int u = 0; u < MAXP; ++u) {
+            o.y[u] = Pack8<TY>::load(y + r_ * DI + cc[u]);
+            o.z[u] = Pack8<T>::load(zxbcdt + r_ * s.ld + cc[u]);
+            o.d[u] = Pack8<T>::load(dout + r_ * DI + cc[u]);
+        }
+        return o;
+    };
     const float inv_di = 1.f / (float)DI;
-    for (long long row0 = (long long)blockIdx.x * RPB; row0 < rows; row0 += (long long)gridDim.x * RPB) {
+    const long long stride = (long long)gridDim.x * RPB;
+    RowIn cur = fetch((long long)blockIdx.x * RPB + threadIdx.x / LPR);
+    auto pass = [&](long long row0, auto whole_tag) {
+        constexpr bool WHOLE = decltype(whole_tag)::value;  // every row of the pass exists
         const long long row = row0 + threadIdx.x / LPR;
-        const bool live = row < rows;  // (whole waves stay for the lane exchanges)
-        const size_t r_ = live ? (size_t)row : 0;
+        const bool live = WHOLE || row < rows;  // (whole waves stay for the lane exchanges)
         float yy[MAXP][8], zz[MAXP][8], dd[MAXP][8];
+#pragma unroll
+        for (int u = 0; u < MAXP; ++u) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                yy[u][i] = EXACT ? cur.y[u].get(i) : in[u] * cur.y[u].get(i);
+                zz[u][i] = cur.z[u].get(i);
+                dd[u][i] = cur.d[u].get(i);
+                // (the unpacked values exist from here on: left alone, the compiler unpacks where they are used, keeps
+                // the packed registers alive until then and moves the next row's loads behind the arithmetic)
+                asm volatile("" : "+v"(yy[u][i]), "+v"(zz[u][i]), "+v"(dd[u][i]));
+            }
+        }
+        cur = fetch(row + stride);  // (after the values have been taken out: the loads go into the same registers)
+        __builtin_amdgcn_sched_barrier(0);  // (and are not moved behind the arithmetic)
         float ss = 0.f, gv = 0.f;
 #pragma unroll
         for (int u = 0; u < MAXP; ++u) {
-            const int c0 = (u * LPR + lane) * 8;
-            if (c0 < DI) {
-                const Pack8<TY> yv = Pack8<TY>::load(y + r_ * DI + c0);
-                const Pack8<T> zv = Pack8<T>::load(zxbcdt + r_ * s.ld + c0);
-                const Pack8<T> dv = Pack8<T>::load(dout + r_ * DI + c0);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    yy[u][i] = yv.get(i);
-                    zz[u][i] = zv.get(i);
-                    dd[u][i] = dv.get(i);
-                    const float v = yy[u][i] * silu(zz[u][i]);
-                    ss += v * v;
-                    gv += dd[u][i] * wv[u][i] * v;
-                }
+            for (int i = 0; i < 8; ++i) {
+                const float v = yy[u][i] * silu(zz[u][i]);  // (zero in a slot past the row: y counts as zero there)
+                ss += v * v;
+                gv += dd[u][i] * wv[u][i] * v;
             }
         }
         ss = group_sum<LPR>(ss);
@@ -97,7 +131,7 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
 #pragma unroll
         for (int u = 0; u < MAXP; ++u) {
             const int c0 = (u * LPR + lane) * 8;
-            if (c0 < DI && live) {
+            if ((EXACT || c0 < DI) && live) {
                 float oy[8], oz[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
@@ -112,7 +146,15 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
                 Pack8<T>::store(dzxbcdt + (size_t)row * s.ld + c0, oz);
             }
         }
+    };
+    // (the first pass stands outside the loop: entered from code with no stores in flight, the loop's first wait would
+    // be counted for that case and wait for the stores of the pass before on every later round)
+    long long row0 = (long long)blockIdx.x * RPB;
+    if (row0 + RPB <= rows) {
+        pass(row0, std::true_type{});
+        for (row0 += stride; row0 + RPB <= rows; row0 += stride) pass(row0, std::true_type{});
     }
+    if (row0 < rows) pass(row0, std::false_type{});
     // the workgroup's partial of dw: the RPB row slots of every channel, added in slot order
     __shared__ float red[256 * 8];
 #pragma unroll
@@ -181,7 +223,11 @@ static hipError_t launch_column_sums(const float *part, int nparts, int cols, fl
 // two rings of registers (the loop is unrolled by K, so ring positions are compile-time): dpre[t] is formed at step t
 // and din[t-(K-1)] leaves at the same step.  A gradient on the returned conv state joins din of the last K-1
 // timesteps; the gradient of the incoming conv state is block_pre_bwd_state_kernel's.
-template <typename T, int K>
+// Every load is unconditional (rows outside the sequence read a row inside it and count as zeros) and a step's rows
+// are requested K steps before they are used, into the ring slot the step K before has just emptied: a conditional
+// load is a branch at which the compiler waits for every earlier load and store, which made each step wait for the
+// store of the step before.  RS: the call has a reset mask.
+template <typename T, int K, bool RS>
 __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict__ zxbcdt, const float *__restrict__ conv_w,
                                                             const float *__restrict__ conv_b, const T *__restrict__ state_in,
                                                             const unsigned char *__restrict__ reset, const T *__restrict__ dx,
@@ -207,13 +253,23 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
         const int t1 = min(t0 + kBwdSteps, s.L);
         const int c0 = piece * kBwdCh;
         const T *row0 = zxbcdt + ((size_t)b * s.L) * s.ld + DI + c0;
-        const unsigned char *rs = reset ? reset + (size_t)b * s.L : nullptr;
+        const unsigned char *rs = RS ? reset + (size_t)b * s.L : nullptr;
+        static_assert(kBwdCh == 4, "a thread's taps are K float4, its biases one");
         float w[kBwdCh][K], bias[kBwdCh];
+        {
+            float wf[kBwdCh * K];
 #pragma unroll
-        for (int i = 0; i < kBwdCh; ++i) {
-            bias[i] = conv_b[c0 + i];
+            for (int q = 0; q < K; ++q) {
+                const float4 v = *reinterpret_cast<const float4 *>(conv_w + (size_t)c0 * K + 4 * q);
+                wf[4 * q] = v.x; wf[4 * q + 1] = v.y; wf[4 * q + 2] = v.z; wf[4 * q + 3] = v.w;
+            }
+            const float4 bq = *reinterpret_cast<const float4 *>(conv_b + c0);
+            bias[0] = bq.x; bias[1] = bq.y; bias[2] = bq.z; bias[3] = bq.w;
 #pragma unroll
-            for (int k = 0; k < K; ++k) w[i][k] = conv_w[(size_t)(c0 + i) * K + k];
+            for (int i = 0; i < kBwdCh; ++i) {
+#pragma unroll
+                for (int k = 0; k < K; ++k) w[i][k] = wf[i * K + k];
+            }
         }
         // where the gradient of the scan's input for these channels comes from
         const T *gsrc;
@@ -228,20 +284,37 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
             gsrc = dC + ((size_t)b * s.L) * GN + (c0 - DI - GN);
             gstride = GN;
         }
-        // input row of timestep ts (history before 0 from the conv state, zero without one)
-        auto in_row = [&](int ts, float (&v)[kBwdCh]) {
-#pragma unroll
-            for (int i = 0; i < kBwdCh; ++i) v[i] = 0.f;
-            if (ts >= 0) {
-                const PackCh<T> p = PackCh<T>::load(row0 + (size_t)ts * s.ld);
-#pragma unroll
-                for (int i = 0; i < kBwdCh; ++i) v[i] = p.get(i);
-            } else if (state_in != nullptr) {
-                const PackCh<T> p = PackCh<T>::load(state_in + ((size_t)b * (K - 1) + (K - 1 + ts)) * C + c0);
-#pragma unroll
-                for (int i = 0; i < kBwdCh; ++i) v[i] = p.get(i);
-            }
+        // what step j (timestep t0 + j) reads: its input row, its gradient row, its restart flag
+        struct StepIn {
+            PackCh<T> p, g;
+            unsigned char r;
         };
+        auto fetch = [&](int j) {
+            StepIn o;
+            const int tc = min(t0 + j, s.L - 1);
+            o.p = PackCh<T>::load(row0 + (size_t)tc * s.ld);
+            o.g = PackCh<T>::load(gsrc + (size_t)tc * gstride);
+            o.r = RS ? rs[tc] : (unsigned char)0;
+            return o;
+        };
+        // the K-1 input rows before the run (history before 0 from the conv state, zero without one) and the restart
+        // flags of the K-2 timesteps before it
+        PackCh<T> hist[K - 1];
+#pragma unroll
+        for (int m = 1; m <= K - 1; ++m) {
+            const int ts = t0 - m;
+            const T *own = row0 + (size_t)max(ts, 0) * s.ld;
+            const T *old = state_in != nullptr ? state_in + ((size_t)b * (K - 1) + max(K - 1 + ts, 0)) * C + c0 : own;
+            hist[m - 1] = PackCh<T>::load(ts >= 0 ? own : old);
+        }
+        unsigned char rb[K > 2 ? K - 2 : 1] = {};
+        if constexpr (RS) {
+#pragma unroll
+            for (int back = 1; back <= K - 2; ++back) rb[back - 1] = rs[max(t0 - back, 0)];
+        }
+        StepIn cur[K];
+#pragma unroll
+        for (int u = 0; u < K; ++u) cur[u] = fetch(u);
         // rings: step j (timestep t0 + j) uses position j % K; position of step j - m is (j - m) mod K
         float win[K][kBwdCh], dq[K][kBwdCh];
         bool fl[K];
@@ -252,13 +325,16 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
             for (int i = 0; i < kBwdCh; ++i) dq[k][i] = 0.f;
         }
 #pragma unroll
-        for (int m = 1; m <= K - 1; ++m) in_row(t0 - m, win[K - m]);
-        if (rs != nullptr) {
+        for (int m = 1; m <= K - 1; ++m) {
+            const bool have = t0 - m >= 0 || state_in != nullptr;
+#pragma unroll
+            for (int i = 0; i < kBwdCh; ++i) win[K - m][i] = have ? hist[m - 1].get(i) : 0.f;
+        }
+        if constexpr (RS) {
             // a restart at one of the K-2 timesteps before the run cuts the rows before it
 #pragma unroll
             for (int back = 1; back <= K - 2; ++back) {
-                const int ts = t0 - back;
-                if (ts >= 0 && rs[ts] != 0) {
+                if (t0 - back >= 0 && rb[back - 1] != 0) {
 #pragma unroll
                     for (int m = back + 1; m <= K - 1; ++m) {
 #pragma unroll
@@ -275,7 +351,7 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
             for (int u = 0; u < K; ++u) {  // ring position of this step: u
                 const int t = t0 + jb + u;
                 const bool exists = t < s.L && jb + u < NT;
-                const bool r = exists && rs != nullptr && rs[t] != 0;
+                const bool r = RS && exists && cur[u].r != 0;
                 if (r) {  // the rows before a restart do not reach it
 #pragma unroll
                     for (int m = 1; m <= K - 1; ++m) {
@@ -286,18 +362,12 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
                 float gin[kBwdCh];
 #pragma unroll
                 for (int i = 0; i < kBwdCh; ++i) {
-                    gin[i] = 0.f;
-                    win[u][i] = 0.f;
+                    win[u][i] = exists ? cur[u].p.get(i) : 0.f;
+                    gin[i] = exists ? cur[u].g.get(i) : 0.f;
                 }
-                if (exists) {
-                    const PackCh<T> p = PackCh<T>::load(row0 + (size_t)t * s.ld);
-                    const PackCh<T> g = PackCh<T>::load(gsrc + (size_t)t * gstride);
-#pragma unroll
-                    for (int i = 0; i < kBwdCh; ++i) {
-                        win[u][i] = p.get(i);
-                        gin[i] = g.get(i);
-                    }
-                }
+                // (after the slot's values have been taken out, so that the load can go into the same registers: a
+                // copy at the loop's end would have to wait for it)
+                cur[u] = fetch(jb + u + K);
                 const bool own = exists && t < t1;  // this thread's own timesteps: the parameter gradients
 #pragma unroll
                 for (int i = 0; i < kBwdCh; ++i) {
@@ -331,7 +401,7 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
                     // those before the window's last restart zeroed
                     if (dstate_out != nullptr && sidx >= s.L - (K - 1)) {
                         bool kept = true;
-                        for (int tt = sidx + 1; tt < s.L; ++tt) kept = kept && !(rs != nullptr && rs[tt] != 0);
+                        for (int tt = sidx + 1; tt < s.L; ++tt) kept = kept && !(RS && rs[tt] != 0);
                         if (kept) {
                             const PackCh<T> p = PackCh<T>::load(dstate_out + ((size_t)b * (K - 1) + (sidx - (s.L - (K - 1)))) * C + c0);
 #pragma unroll
@@ -513,17 +583,24 @@ static hipError_t post_bwd_dispatch(const BlockShape &s, const void *y, const vo
     const TY *yy = static_cast<const TY *>(y);
     const T *zz = static_cast<const T *>(zxbcdt), *dd = static_cast<const T *>(dout);
     T *oy = static_cast<T *>(dy), *oz = static_cast<T *>(dzxbcdt);
-    int blocks;
-    if (pieces <= 16 * 4) {
-        blocks = (int)std::min<long long>(kPostBlocks, (rows + 15) / 16);
-        block_post_bwd_kernel<T, TY, 16><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, s);
-    } else if (pieces <= 32 * 4) {
-        blocks = (int)std::min<long long>(kPostBlocks, (rows + 7) / 8);
-        block_post_bwd_kernel<T, TY, 32><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, s);
-    } else {
-        blocks = (int)std::min<long long>(kPostBlocks, (rows + 3) / 4);
-        block_post_bwd_kernel<T, TY, 64><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, s);
+    // lanes per row and pieces per lane as in the forward
+    const int lpr = pieces <= 16 * 4 ? 16 : pieces <= 32 * 4 ? 32 : 64;
+    const int ppl = (pieces + lpr - 1) / lpr;
+    const int blocks = (int)std::min<long long>(kPostBlocks, (rows + 256 / lpr - 1) / (256 / lpr));
+    bool launched = false;
+#define SSD_POST_BWD_CASE(LPRv, PPLv)                                                                                       \
+    if (lpr == LPRv && ppl == PPLv) {                                                                                       \
+        if (pieces == LPRv * PPLv)                                                                                          \
+            block_post_bwd_kernel<T, TY, LPRv, PPLv, true><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, s); \
+        else                                                                                                                \
+            block_post_bwd_kernel<T, TY, LPRv, PPLv, false><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, s); \
+        launched = true;                                                                                                    \
     }
+    SSD_POST_BWD_CASE(16, 1) SSD_POST_BWD_CASE(16, 2) SSD_POST_BWD_CASE(16, 3) SSD_POST_BWD_CASE(16, 4)
+    SSD_POST_BWD_CASE(32, 3) SSD_POST_BWD_CASE(32, 4)
+    SSD_POST_BWD_CASE(64, 3) SSD_POST_BWD_CASE(64, 4)
+#undef SSD_POST_BWD_CASE
+    if (!launched) return hipErrorInvalidValue;
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     return launch_column_sums(part, blocks, DI, part + (size_t)kPostBlocks * DI, dnorm_w, st);
@@ -558,15 +635,24 @@ static hipError_t pre_bwd_dispatch(const BlockShape &s, const void *zxbcdt, cons
     const dim3 sgrid((unsigned)(((long long)s.B * (C / 8) + 255) / 256));
     switch (K) {
         case 2:
-            block_pre_bwd_kernel<T, 2><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            if (reset != nullptr)
+                block_pre_bwd_kernel<T, 2, true><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            else
+                block_pre_bwd_kernel<T, 2, false><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
             if (gsi) block_pre_bwd_state_kernel<T, 2><<<sgrid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, gsi, s);
             break;
         case 3:
-            block_pre_bwd_kernel<T, 3><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            if (reset != nullptr)
+                block_pre_bwd_kernel<T, 3, true><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            else
+                block_pre_bwd_kernel<T, 3, false><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
             if (gsi) block_pre_bwd_state_kernel<T, 3><<<sgrid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, gsi, s);
             break;
         case 4:
-            block_pre_bwd_kernel<T, 4><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            if (reset != nullptr)
+                block_pre_bwd_kernel<T, 4, true><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
+            else
+                block_pre_bwd_kernel<T, 4, false><<<grid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, out, part, s);
             if (gsi) block_pre_bwd_state_kernel<T, 4><<<sgrid, dim3(256), 0, st>>>(in, conv_w, conv_b, si, reset, gx, gb, gc, gso, gsi, s);
             break;
         default: return hipErrorInvalidValue;
