@@ -477,22 +477,26 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // tile nc - j begins where this one's tile j does; this scan's initial state meets the other's final state and
     // the other way round.  The piece goes to out[b, k, h, slice] with k counted in forward time.
     constexpr bool ANCH = KIND == 3 || KIND == 7;
-    auto adjoint_state = [&](int j) -> const float * {
+    // (where the other scan has no state to meet -- no initial state, no gradient on the final state -- the anchor is
+    // zero: the loads then read the other scan's first tile state, so that none of them stands under a condition, and
+    // `zero` drops the result.  A load under a condition sits in a block of its own with its first use, and the wave
+    // waits for it there instead of during the phase it was meant to overlap.)
+    auto adjoint_state = [&](int j, bool &zero) -> const float * {
         const float *g = j == 0 ? an.other_final : j == s.nc ? an.other_init : an.other_tiles;
-        if (g == nullptr) return nullptr;
-        const size_t bh = j == 0 || j == s.nc ? (size_t)b * s.H + h : ((size_t)b * s.nc + (s.nc - j)) * s.H + h;
-        return g + (bh * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
+        zero = g == nullptr;
+        const bool tiles = zero || (j != 0 && j != s.nc);
+        const size_t bh = tiles ? ((size_t)b * s.nc + (zero ? 0 : s.nc - j)) * s.H + h : (size_t)b * s.H + h;
+        return (zero ? an.other_tiles : g) + (bh * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
     };
     // one slice at a time, so that at most one slice of the other scan's state is held in registers
     auto load_other = [&](const float *g, int sl, float4 (&gq)[NB][4]) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4)
-                gq[nb][q4] = g ? *reinterpret_cast<const float4 *>(g + sl * 32 * N + 32 * nb + 8 * q4) : make_float4(0, 0, 0, 0);
+            for (int q4 = 0; q4 < 4; ++q4) gq[nb][q4] = *reinterpret_cast<const float4 *>(g + sl * 32 * N + 32 * nb + 8 * q4);
         }
     };
-    auto write_anchor = [&](int k, int sl, const float4 (&gq)[NB][4]) {
+    auto write_anchor = [&](int k, int sl, const float4 (&gq)[NB][4], bool zero) {
         double part = 0.0;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
@@ -502,17 +506,19 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 part += (double)st[sn][4 * q4] * gq[nb][q4].x + (double)st[sn][4 * q4 + 1] * gq[nb][q4].y +
                         (double)st[sn][4 * q4 + 2] * gq[nb][q4].z + (double)st[sn][4 * q4 + 3] * gq[nb][q4].w;
         }
-        part = wave_inclusive_scan(part);
+        part = wave_inclusive_scan(zero ? 0.0 : part);
         if (lane0 == 63) an.out[(((size_t)b * (s.nc + 1) + (ADJ ? s.nc - k : k)) * s.H + h) * PBn + pb + sl] = part;
     };
     if constexpr (ANCH) {
         if (an.out != nullptr) {
-            const float *g0 = init ? adjoint_state(0) : nullptr;  // no initial state: a zero anchor
+            bool zero0;
+            const float *g0 = adjoint_state(0, zero0);
+            zero0 = zero0 || init == nullptr;  // no initial state: a zero anchor
 #pragma unroll
             for (int sl = 0; sl < SL; ++sl) {
                 float4 gq[NB][4];
                 load_other(g0, sl, gq);
-                write_anchor(0, sl, gq);
+                write_anchor(0, sl, gq, zero0);
             }
         }
     }
@@ -683,14 +689,20 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 // the epilogue (lane = (row l, half): elements 8 vg + 4 half .. + 3 of the head's row)
                 uint2 aq[4] = {make_uint2(0, 0), make_uint2(0, 0), make_uint2(0, 0), make_uint2(0, 0)};
                 float wt = 1.f;
+                if constexpr (TR_ADJ) {
+                    // the heads' dt of this block's rows (dB sums the heads' outputs weighted by it), requested here and
+                    // used in the epilogue; a row outside the sequence reads a row inside it and weighs zero
+                    const int trow = s.L - 1 - (t0 + l);
+                    wt = (float)dt[((size_t)b * trows + min(max(trow, 0), trows - 1)) * s.H + h];
+                }
                 if constexpr (ROWS) {
-                    const int arow = s.L - 1 - (t0 + l);
-                    if (l < rows && arow >= 0 && arow < trows) {
-                        const T *ar = aux + ((size_t)b * trows + arow) * HP + h * s.P + pb * 32 + 4 * half;
+                    // (no condition on the loads: a row outside the sequence reads a row inside it, and nothing of it is
+                    // stored -- under a condition the loads sit in a block of their own where the wave waits for them)
+                    const int arow = min(max(s.L - 1 - (t0 + l), 0), trows - 1);
+                    const T *ar = aux + ((size_t)b * trows + arow) * HP + h * s.P + pb * 32 + 4 * half;
 #pragma unroll
-                        for (int vg = 0; vg < 4; ++vg) aq[vg] = *reinterpret_cast<const uint2 *>(ar + 8 * vg);
-                        wt = (float)dt[((size_t)b * trows + arow) * s.H + h];
-                    }
+                    for (int vg = 0; vg < 4; ++vg) aq[vg] = *reinterpret_cast<const uint2 *>(ar + 8 * vg);
+                    wt = (float)dt[((size_t)b * trows + arow) * s.H + h];
                 }
                 Frag<T> Cf[NK];
 #pragma unroll
@@ -778,8 +790,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     const int le = phase_tid() & 63, he = le >> 5, ll = lb * 32 + (le & 31);
                     const int trow = ADJ ? s.L - 1 - (t0 + ll) : t0 + ll;
                     const bool live = ll < rows && trow >= 0 && trow < trows;
-                    // adjoint: dB sums the heads' outputs weighted by their dt
-                    if (TR_ADJ) wt = live ? (float)dt[((size_t)b * trows + trow) * s.H + h] : 0.f;
+                    if (TR_ADJ) wt = live ? wt : 0.f;
 #pragma unroll
                     for (int sl = 0; sl < SL; ++sl) {
                         float part = 0.f;  // forward: this slice's part of C_t . y_t
@@ -900,8 +911,13 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         // the other scan's state where this tile ends: the first slice in flight during phase 2, the second (two
         // slices per wave leave no registers to hold both) requested after it
         float4 gq[ANCH ? NB : 1][4];
+        bool gzero = false;
+        const float *gnext = nullptr;
         if constexpr (ANCH) {
-            if (an.out != nullptr) load_other(adjoint_state(c + 1), 0, gq);
+            if (an.out != nullptr) {
+                gnext = adjoint_state(c + 1, gzero);
+                load_other(gnext, 0, gq);
+            }
         }
         seg_total *= a_end;
         const int lane = phase_tid() & 63, half = lane >> 5;
@@ -958,10 +974,25 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         }
         if constexpr (ANCH) {
             if (an.out != nullptr) {
-                write_anchor(c + 1, 0, gq);
+                // (the other scan's values are used from here on, not before: left alone, the compiler converts them to
+                // float64 right behind their loads, in front of phase 2, and the wave waits for them there)
+                auto pin = [&](float4 (&q)[NB][4]) {
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; ++q4)
+                            asm volatile("" : "+v"(q[nb][q4].x), "+v"(q[nb][q4].y), "+v"(q[nb][q4].z), "+v"(q[nb][q4].w));
+                    }
+                };
+                pin(gq);
+                // the second slice is requested here and arrives during the first slice's sums (requested ahead of phase
+                // 2 with the first, the compiler copies registers right behind the loads and waits for them there)
+                float4 gq1[SL == 2 ? NB : 1][4];
+                if constexpr (SL == 2) load_other(gnext, 1, gq1);
+                write_anchor(c + 1, 0, gq, gzero);
                 if constexpr (SL == 2) {
-                    load_other(adjoint_state(c + 1), 1, gq);
-                    write_anchor(c + 1, 1, gq);
+                    pin(gq1);
+                    write_anchor(c + 1, 1, gq1, gzero);
                 }
             }
         }

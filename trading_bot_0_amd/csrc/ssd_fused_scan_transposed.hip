@@ -29,6 +29,7 @@ hipError_t launch_transposed_scan(const ScanShape &sT, bool adjoint, const void 
     t.Q = kOnePassTile;
     t.nc = (sT.L + kOnePassTile - 1) / kOnePassTile;
     if (an.out != nullptr && adjoint != wide(sT)) return hipErrorInvalidValue;
+    if (an.out != nullptr && an.other_tiles == nullptr) return hipErrorInvalidValue;  // (the kernel reads it without asking)
     if (wide(sT))
         return adjoint ? fused_launch_transposed<__bf16, 7>(t, x, dt, A, Bm, Cm, nullptr, init, reset, out, final_states,
                                                             tile_states, nullptr, an, st)
