@@ -11,6 +11,8 @@
 // collected in an LDS tile of the wave's own and written out with adjacent lanes on adjacent 16-byte pieces of a
 // row (stores scattered over 32 rows straight from the accumulators' layout run at a fraction of the memory
 // system's rate).
+#include <algorithm>
+
 #include "ssd_device.h"
 
 namespace ssd {
@@ -22,7 +24,14 @@ constexpr int kProjBlockCols = 160;   // most output columns per workgroup (thei
 constexpr int kProjChunk = 32;        // output columns per MFMA tile
 constexpr int kProjTiles = 8;         // tiles of 32 rows per wave
 
-template <int KS>  // K = 16 * KS
+// CH: 32-column chunks of the widest block of columns (1..5; a block takes CH or CH - 1 chunks, and its last chunk
+// may hold fewer columns than it covers).  The chunk count is a template parameter and every store goes out without a condition -- a
+// buffer store whose offset is put out of range for rows past M and columns past the block, which the hardware then
+// drops -- because loads and stores share one counter per wave, in order: only in straight-line code with every
+// store counted does the compiler wait for a tile's rows of u by their exact position in that order.  With a loop of
+// unknown length or a guarded store in between it waits for everything outstanding -- the next tile's rows, requested
+// a moment ago, and the last stores -- and the tile's loads, products and stores ran one after the other.
+template <int KS, int CH>  // K = 16 * KS
 __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf16 *__restrict__ u,
                                                                       const __bf16 *__restrict__ w,
                                                                       __bf16 *__restrict__ out, long long M, int N,
@@ -30,7 +39,7 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
     constexpr int K = 16 * KS, NTHR = 64 * kProjWaves;
     constexpr int ROWB = K * 2 + 16;        // bytes of a staged row of w: 16 bytes of padding shift the banks
     constexpr int kTileRowB = 64 * 2 + 16;  // a row of a wave's output tile: 64 columns and 16 bytes of padding
-    __shared__ __attribute__((aligned(16))) unsigned char wsm[kProjBlockCols * ROWB];
+    __shared__ __attribute__((aligned(16))) unsigned char wsm[CH * kProjChunk * ROWB];
     __shared__ __attribute__((aligned(16))) unsigned char otile[kProjWaves][32 * kTileRowB];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // Workgroups go to the eight XCDs in turn, each XCD with an L2 of its own: the column blocks of a range of rows
@@ -41,30 +50,33 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
     const long long rg = (long long)(within / col_blocks) * 8 + xcd;
     const int n0 = cb * block_cols;                 // this workgroup's first column
     const int ncols = cb == col_blocks - 1 ? N - n0 : block_cols;  // a multiple of 8; the last block takes the rest
-    const int chunks = (ncols + kProjChunk - 1) / kProjChunk;
     const long long row0 = rg * kProjTiles * (32LL * kProjWaves);
     if (row0 >= M) return;  // the grid is padded to whole rounds of XCDs
 
-    {   // rows n0 .. n0 + 32 * chunks - 1 of w, all requested before the first is written to LDS (rows past N repeat
-        // the last one; their columns are never stored)
-        constexpr int FILL = (kProjBlockCols * (K / 8) + NTHR - 1) / NTHR;
-        const int pieces = chunks * kProjChunk * (K / 8);
+    {   // rows n0 .. n0 + 32 * CH - 1 of w, all requested before the first is written to LDS (rows past N repeat the
+        // last one, and pieces past the block are the block's last piece once more: neither loads nor writes stand
+        // under a condition; the surplus columns are never stored)
+        constexpr int PIECES = CH * kProjChunk * (K / 8);
+        constexpr int FILL = (PIECES + NTHR - 1) / NTHR;
         uint4 q[FILL];
 #pragma unroll
         for (int i = 0; i < FILL; ++i) {
-            const int p = min(tid + i * NTHR, pieces - 1);
+            const int p = min(tid + i * NTHR, PIECES - 1);
             q[i] = *reinterpret_cast<const uint4 *>(w + (size_t)min(n0 + p / (K / 8), N - 1) * K + (p % (K / 8)) * 8);
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < FILL; ++i) {
-            const int p = tid + i * NTHR;
-            if (p < pieces) *reinterpret_cast<uint4 *>(wsm + (p / (K / 8)) * ROWB + (p % (K / 8)) * 16) = q[i];
+            const int p = min(tid + i * NTHR, PIECES - 1);
+            *reinterpret_cast<uint4 *>(wsm + (p / (K / 8)) * ROWB + (p % (K / 8)) * 16) = q[i];
         }
     }
     __syncthreads();
 
     const int r = lane & 31, half = lane >> 5;
     unsigned char *tile = otile[wave];
+    // the workgroup's rows of `out` as a range-checked buffer: 2 048 rows of at most ldo elements
+    const __amdgpu_buffer_rsrc_t obuf = make_buffer(out + (size_t)row0 * ldo, (unsigned)min((long long)kProjTiles * 32 * kProjWaves, M - row0) * (unsigned)ldo * 2u);
     auto tile_row0 = [&](int t) { return row0 + (long long)t * (32 * kProjWaves) + wave * 32; };
     // this lane's part of its row of u: K elements 16 ks + 8 half .. + 7 for every K step (rows past M repeat the
     // last row; they are never stored)
@@ -73,13 +85,19 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) uf[ks].v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(ur + 16 * ks));
     };
+    // (a block takes CH chunks or one fewer -- 648 columns are 4 x 128 + 136 -- and the last chunk is the only piece
+    // of a tile's work under a condition, a uniform one)
+    const bool last_chunk = ncols > (CH - 1) * kProjChunk;
     auto tile_product = [&](int t, const Frag<__bf16>(&uf)[KS]) {
+        const unsigned trow = (unsigned)(t * (32 * kProjWaves) + wave * 32);  // the tile's first row within the workgroup's
         const long long m0 = tile_row0(t);
-        for (int c0 = 0; c0 < chunks; c0 += 2) {
+#pragma unroll
+        for (int c0 = 0; c0 < CH; c0 += 2) {
+            if (c0 == CH - 1 && !last_chunk) break;  // (an odd CH: the last pair is the last chunk alone)
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub) {
                 const int c = c0 + sub;
-                if (c >= chunks) break;
+                if (c >= CH || (c == CH - 1 && !last_chunk)) break;
                 const unsigned char *wb = wsm + (c * kProjChunk + r) * ROWB + half * 16;
                 f32x16 acc = {0}, acc_odd = {0};  // two chains of dependent MFMAs instead of one
 #pragma unroll
@@ -104,9 +122,10 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
 #pragma unroll
             for (int pass = 0; pass < 4; ++pass) {
                 const int row = pass * 8 + (lane >> 3), col = c0 * kProjChunk + (lane & 7) * 8;
-                const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kTileRowB + (lane & 7) * 16);
-                if (m0 + row < M && col < ncols)
-                    *reinterpret_cast<uint4 *>(out + (size_t)(m0 + row) * ldo + n0 + col) = v;
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + row * kTileRowB + (lane & 7) * 16);
+                const bool ok = m0 + row < M && col < ncols;
+                const unsigned off = ((trow + (unsigned)row) * (unsigned)ldo + (unsigned)(n0 + col)) * 2u;
+                __builtin_amdgcn_raw_buffer_store_b128(v, obuf, ok ? off : kBufferDropOffset, 0, 0);
             }
             asm volatile("" ::: "memory");
             __builtin_amdgcn_wave_barrier();
@@ -114,13 +133,13 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
     };
     // Two sets of row fragments: the next tile's rows are requested before this tile's products, because loads and
     // stores complete in order per wave -- requested after, they would wait for this tile's stores to reach memory.
+    // (Tiles past M load the last row and store nothing, so that the loop has no exit in its middle.)
     Frag<__bf16> ua[KS], ub[KS];
     load_rows(0, ua);
+#pragma unroll
     for (int t = 0; t < kProjTiles; t += 2) {
-        if (tile_row0(t) >= M) break;
         load_rows(t + 1, ub);
         tile_product(t, ua);
-        if (tile_row0(t + 1) >= M) break;
         if (t + 2 < kProjTiles) load_rows(t + 2, ua);
         tile_product(t + 1, ub);
     }
@@ -162,11 +181,18 @@ hipError_t launch_block_proj(long long rows, int in_features, int out_features, 
     const dim3 grid((unsigned)groups), block(64 * kProjWaves);
     const __bf16 *uu = static_cast<const __bf16 *>(u), *ww = static_cast<const __bf16 *>(w);
     __bf16 *oo = static_cast<__bf16 *>(out);
-    if (in_features == 128)
-        block_proj_kernel<8><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, out_ld, col_blocks, block_cols);
-    else
-        block_proj_kernel<16><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, out_ld, col_blocks, block_cols);
-    return hipGetLastError();
+    // the chunks of 32 columns the widest block takes
+    const int widest = std::max(block_cols, out_features - (col_blocks - 1) * block_cols);
+    const int ch = (widest + kProjChunk - 1) / kProjChunk;
+#define SSD_PROJ_CASE(KSv, CHv)                                                                                        \
+    if (in_features == 16 * KSv && ch == CHv) {                                                                        \
+        block_proj_kernel<KSv, CHv><<<grid, block, 0, st>>>(uu, ww, oo, rows, out_features, out_ld, col_blocks, block_cols); \
+        return hipGetLastError();                                                                                      \
+    }
+    SSD_PROJ_CASE(8, 1) SSD_PROJ_CASE(8, 2) SSD_PROJ_CASE(8, 3) SSD_PROJ_CASE(8, 4) SSD_PROJ_CASE(8, 5)
+    SSD_PROJ_CASE(16, 1) SSD_PROJ_CASE(16, 2) SSD_PROJ_CASE(16, 3) SSD_PROJ_CASE(16, 4) SSD_PROJ_CASE(16, 5)
+#undef SSD_PROJ_CASE
+    return hipErrorInvalidValue;
 }
 
 }  // namespace ssd
