@@ -384,7 +384,9 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
 // The same for chunks of 64 steps and NH = 4, 8 or 16 heads with one wave per (b, c) and all its heads: lane =
 // (step % TL) * NH + head with TL = 64 / NH, register r = step / TL, so that every load and store of the wave is one
 // contiguous run of 64 elements of a [B, L, H] array (a wave per head touches a cache line per lane instead).
-template <typename T, int NH>
+// NP: the pieces of C . yC per element when they are 1..4 (then e1 holds the (e1, dd) pairs and the loads are
+// straight-line code); 0: any other form of the inputs, through conditions uniform over the launch.
+template <typename T, int NH, int NP>
 __global__ __launch_bounds__(256) void bwd_ddt_heads_kernel(const T *__restrict__ dt, const float *__restrict__ A,
                                                             const float *__restrict__ e1, const float *__restrict__ u,
                                                             const float *__restrict__ dd, const double *__restrict__ anchor,
@@ -399,46 +401,92 @@ __global__ __launch_bounds__(256) void bwd_ddt_heads_kernel(const T *__restrict_
     const int c = (int)(id % s.nc);
     const long long b = id / s.nc;
     const int h = lane % NH, tl = lane / NH;
-    const double a = (double)A[h];
-    auto anchor_at = [&](int k) {
-        const size_t at = ((size_t)b * (s.nc + 1) + k) * NH + h;
-        if (raw_anchors == 0) return anchor[at];
-        double v = 0.0;
-        for (int i = 0; i < raw_anchors; ++i) v += anchor[at * raw_anchors + i];
-        if (k < s.nc) {
-            const size_t t = (size_t)b * s.L + (size_t)k * 64;
-            v *= (reset != nullptr && reset[t] != 0) ? 0.0 : exp((double)(float)dt[t * NH + h] * a);
-        }
-        return v;
-    };
-    const double q0 = anchor_at(c), q1 = anchor_at(c + 1);
     const int t0 = c * 64, len = min(64, s.L - t0);
     const size_t row0 = ((size_t)b * s.L + t0) * NH;  // this chunk's first element of a [B, L, H] array
+    // Every load of the wave is requested here, before the first is used, and none stands under a condition (a step
+    // past the sequence reads the chunk's last step and counts as zero; a piece past nparts or raw_anchors reads the
+    // last piece and counts as zero): under conditions and in loops of unknown length the compiler put a wait behind
+    // every one of them.
+    constexpr int kMaxPieces = 4;  // pieces per element read without a loop (more take the loops below)
+    const size_t last = row0 + (size_t)len * NH - 1;
+    T dt_q[R];
+    float2 pr_q[R];
+    float pk_q[R][kMaxPieces], u_q[R];
+    const bool few_parts = NP > 0 || (parts != nullptr && nparts <= kMaxPieces);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const size_t at = min(row0 + (size_t)r * 64 + lane, last);
+        dt_q[r] = dt[at];
+        if constexpr (NP > 0) {
+            pr_q[r] = *reinterpret_cast<const float2 *>(e1 + 2 * at);
+#pragma unroll
+            for (int k = 0; k < NP; ++k) pk_q[r][k] = parts[at * NP + k];
+        } else if (parts != nullptr) {  // (uniform)
+            pr_q[r] = *reinterpret_cast<const float2 *>(e1 + 2 * at);
+            if (few_parts) {
+#pragma unroll
+                for (int k = 0; k < kMaxPieces; ++k) pk_q[r][k] = parts[at * nparts + min(k, nparts - 1)];
+            }
+        } else {
+            pr_q[r] = make_float2(e1[at], dd[at]);
+            u_q[r] = u[at];
+        }
+    }
+    // the anchors: the inner product of the two states where chunk k starts.  raw_anchors > 0: `anchor` holds that
+    // many pieces per (b, k, h), still without the first step's decay (zero where the sequence restarts there)
+    const double a = (double)A[h];
+    double an_q[2][kMaxPieces];
+    T an_dt[2];
+    unsigned char an_rs[2];
+    const int ra = max(raw_anchors, 1);  // (the launcher keeps raw_anchors within kMaxPieces)
+    const unsigned char *rs_or_any = reset != nullptr ? reset : reinterpret_cast<const unsigned char *>(dt);
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const size_t at = ((size_t)b * (s.nc + 1) + c + e) * NH + h;
+#pragma unroll
+        for (int i = 0; i < kMaxPieces; ++i) an_q[e][i] = anchor[at * ra + min(i, ra - 1)];
+        const size_t t = (size_t)b * s.L + (size_t)min(c + e, s.nc - 1) * 64;
+        an_dt[e] = dt[t * NH + h];
+        an_rs[e] = rs_or_any[t];
+    }
+    auto anchor_at = [&](int e) {
+        double v = 0.0;
+#pragma unroll
+        for (int i = 0; i < kMaxPieces; ++i) v += i < ra ? an_q[e][i] : 0.0;
+        const double first = (reset != nullptr && an_rs[e] != 0) ? 0.0 : exp((double)(float)an_dt[e] * a);
+        return (raw_anchors != 0 && c + e < s.nc) ? v * first : v;
+    };
+    const double q0 = anchor_at(0), q1 = anchor_at(1);
     float e1v[R], ddv[R], dtv[R];
     double uv[R], before[R];  // u_t and the sum of u over the chunk's earlier steps
     double carry = 0.0;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int t = r * TL + tl;
-        const size_t at = row0 + (size_t)r * 64 + lane;
-        e1v[r] = ddv[r] = dtv[r] = 0.f;
-        float uf = 0.f;
-        if (t < len) {
-            dtv[r] = (float)dt[at];
-            if (parts != nullptr) {
-                const float2 pr = *reinterpret_cast<const float2 *>(e1 + 2 * at);
-                e1v[r] = pr.x;
-                ddv[r] = pr.y;
-                float sc = 0.f;
-                for (int k = 0; k < nparts; ++k) sc += parts[at * nparts + k];
-                uf = sc - dtv[r] * e1v[r];
+        const bool in = t < len;
+        dtv[r] = in ? (float)dt_q[r] : 0.f;
+        e1v[r] = in ? pr_q[r].x : 0.f;
+        ddv[r] = in ? pr_q[r].y : 0.f;
+        float uf;
+        if constexpr (NP > 0) {
+            float sc = 0.f;
+#pragma unroll
+            for (int k = 0; k < NP; ++k) sc += pk_q[r][k];
+            uf = sc - dtv[r] * e1v[r];
+        } else if (parts != nullptr) {
+            float sc = 0.f;
+            if (few_parts) {
+#pragma unroll
+                for (int k = 0; k < kMaxPieces; ++k) sc += k < nparts ? pk_q[r][k] : 0.f;
             } else {
-                e1v[r] = e1[at];
-                ddv[r] = dd[at];
-                uf = u[at];
+                const size_t at = min(row0 + (size_t)r * 64 + lane, last);
+                for (int k = 0; k < nparts; ++k) sc += parts[at * nparts + k];
             }
+            uf = sc - dtv[r] * e1v[r];
+        } else {
+            uf = u_q[r];
         }
-        uv[r] = (double)uf;
+        uv[r] = in ? (double)uf : 0.0;
         double v = uv[r];  // inclusive sum over this register's steps of the same head (lanes NH apart)
 #pragma unroll
         for (int d = NH; d < 64; d <<= 1) {
@@ -576,17 +624,24 @@ hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float
                  const double *anchor, void *ddt, double *dA_part, double *dD_part, const float *parts, int nparts,
                  const unsigned char *reset, int raw_anchors, hipStream_t st) {
     if (s.Q > 64) return hipErrorInvalidValue;  // one pass of the wave per chunk
-    if (s.Q == 64 && (s.H == 4 || s.H == 8 || s.H == 16)) {
+    if (s.Q == 64 && (s.H == 4 || s.H == 8 || s.H == 16) && raw_anchors <= 4) {
         const long long chunks = (long long)s.B * s.nc;
         const dim3 grid((unsigned)((chunks + 3) / 4)), block(256);
-#define SSD_DDT_HEADS(NH)                                                                                              \
-    bwd_ddt_heads_kernel<T, NH><<<grid, block, 0, st>>>(static_cast<const T *>(dt), A, e1, u, dd, anchor,               \
-                                                        static_cast<T *>(ddt), dA_part, dD_part, s, parts, nparts, reset, \
-                                                        raw_anchors)
+#define SSD_DDT_HEADS_NP(NH, NP)                                                                                       \
+    bwd_ddt_heads_kernel<T, NH, NP><<<grid, block, 0, st>>>(static_cast<const T *>(dt), A, e1, u, dd, anchor,           \
+                                                            static_cast<T *>(ddt), dA_part, dD_part, s, parts, nparts,   \
+                                                            reset, raw_anchors)
+#define SSD_DDT_HEADS(NH)                                           \
+    do {                                                            \
+        if (parts != nullptr && nparts == 1) SSD_DDT_HEADS_NP(NH, 1); \
+        else if (parts != nullptr && nparts == 2) SSD_DDT_HEADS_NP(NH, 2); \
+        else SSD_DDT_HEADS_NP(NH, 0);                               \
+    } while (0)
         if (s.H == 4) SSD_DDT_HEADS(4);
         else if (s.H == 8) SSD_DDT_HEADS(8);
         else SSD_DDT_HEADS(16);
 #undef SSD_DDT_HEADS
+#undef SSD_DDT_HEADS_NP
         return hipGetLastError();
     }
     const long long waves = (long long)s.B * s.nc * s.H;
