@@ -422,17 +422,31 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
 #pragma unroll
     for (int sl = 0; sl < SL; ++sl) {
         const size_t lane_off = (size_t)((pb + sl) * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
-        const float *ib = init && !fresh ? init + (((size_t)b * (folded ? 1 : S) + (folded ? 0 : seg)) * s.H + h) * s.P * N + lane_off
-                                         : nullptr;
+        // (one uniform branch around all of the state's loads: with a condition on each, the compiler waits for every
+        // load before the next -- eight or sixteen trips to memory before the first tile)
+        const bool have_init = init != nullptr && !fresh;
+        float4 iq[NB][4];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) iq[nb][gq] = make_float4(0, 0, 0, 0);
+        }
+        if (have_init) {
+            const float *ib = init + (((size_t)b * (folded ? 1 : S) + (folded ? 0 : seg)) * s.H + h) * s.P * N + lane_off;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) iq[nb][gq] = *reinterpret_cast<const float4 *>(ib + 32 * nb + 8 * gq);
+            }
+        }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
             for (int gq = 0; gq < 4; ++gq) {
-                const float4 v = ib ? *reinterpret_cast<const float4 *>(ib + 32 * nb + 8 * gq) : make_float4(0, 0, 0, 0);
-                st[sl * NB + nb][4 * gq + 0] = v.x;
-                st[sl * NB + nb][4 * gq + 1] = v.y;
-                st[sl * NB + nb][4 * gq + 2] = v.z;
-                st[sl * NB + nb][4 * gq + 3] = v.w;
+                st[sl * NB + nb][4 * gq + 0] = iq[nb][gq].x;
+                st[sl * NB + nb][4 * gq + 1] = iq[nb][gq].y;
+                st[sl * NB + nb][4 * gq + 2] = iq[nb][gq].z;
+                st[sl * NB + nb][4 * gq + 3] = iq[nb][gq].w;
             }
         }
         if constexpr (KIND == 0) {
