@@ -419,6 +419,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     // a restart before the first step: the initial state is not read at all (it may hold anything)
     const bool folded = KIND == 0 && s.seg_local != nullptr;  // the entering state comes from the recurrence below
     const bool fresh = !ADJ && rsb != nullptr && (seg == 0 || folded) && rsb[0] != 0;
+    // the first tile's inputs are requested ahead of the state's, so that the two trips to memory overlap (and behind
+    // the restart flag's, which the state's loads branch on)
+    prefetch(c_first);
 #pragma unroll
     for (int sl = 0; sl < SL; ++sl) {
         const size_t lane_off = (size_t)((pb + sl) * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
@@ -451,18 +454,38 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         }
         if constexpr (KIND == 0) {
             if (folded) {  // enter[j+1] = decay[j] * enter[j] + local[j] over the segments before this one
-                for (int j = 0; j < seg; ++j) {
-                    const float a = s.seg_local_decay[((size_t)b * S + j) * s.H + h];
-                    const float *lb = s.seg_local + (((size_t)b * S + j) * s.H + h) * s.P * N + lane_off;
+                // two segments per round, both requested before the first is used: half the trips to memory
+                for (int j = 0; j < seg; j += 2) {
+                    const int j1 = min(j + 1, seg - 1);
+                    const float a0 = s.seg_local_decay[((size_t)b * S + j) * s.H + h];
+                    const float a1 = s.seg_local_decay[((size_t)b * S + j1) * s.H + h];
+                    const float *l0 = s.seg_local + (((size_t)b * S + j) * s.H + h) * s.P * N + lane_off;
+                    const float *l1 = s.seg_local + (((size_t)b * S + j1) * s.H + h) * s.P * N + lane_off;
+                    float4 v0[NB][4], v1[NB][4];
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
                         for (int gq = 0; gq < 4; ++gq) {
-                            const float4 v = *reinterpret_cast<const float4 *>(lb + 32 * nb + 8 * gq);
-                            st[sl * NB + nb][4 * gq + 0] = a * st[sl * NB + nb][4 * gq + 0] + v.x;
-                            st[sl * NB + nb][4 * gq + 1] = a * st[sl * NB + nb][4 * gq + 1] + v.y;
-                            st[sl * NB + nb][4 * gq + 2] = a * st[sl * NB + nb][4 * gq + 2] + v.z;
-                            st[sl * NB + nb][4 * gq + 3] = a * st[sl * NB + nb][4 * gq + 3] + v.w;
+                            v0[nb][gq] = *reinterpret_cast<const float4 *>(l0 + 32 * nb + 8 * gq);
+                            v1[nb][gq] = *reinterpret_cast<const float4 *>(l1 + 32 * nb + 8 * gq);
+                        }
+                    }
+                    const bool two = j + 1 < seg;  // (uniform)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            f32x16 &t = st[sl * NB + nb];
+                            t[4 * gq + 0] = a0 * t[4 * gq + 0] + v0[nb][gq].x;
+                            t[4 * gq + 1] = a0 * t[4 * gq + 1] + v0[nb][gq].y;
+                            t[4 * gq + 2] = a0 * t[4 * gq + 2] + v0[nb][gq].z;
+                            t[4 * gq + 3] = a0 * t[4 * gq + 3] + v0[nb][gq].w;
+                            if (two) {
+                                t[4 * gq + 0] = a1 * t[4 * gq + 0] + v1[nb][gq].x;
+                                t[4 * gq + 1] = a1 * t[4 * gq + 1] + v1[nb][gq].y;
+                                t[4 * gq + 2] = a1 * t[4 * gq + 2] + v1[nb][gq].z;
+                                t[4 * gq + 3] = a1 * t[4 * gq + 3] + v1[nb][gq].w;
+                            }
                         }
                     }
                 }
@@ -538,7 +561,6 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     }
 
     float seg_total = 1.f;  // product of the tiles' decays (KIND 2)
-    prefetch(c_first);
     // one tile; `set` (a compile-time 0 or 1) is the set of LDS tiles it uses; false when the scan ends inside it
     auto tile = [&](const int c, auto set) -> bool {
         constexpr int SET = decltype(set)::value;
