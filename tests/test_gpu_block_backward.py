@@ -49,7 +49,8 @@ def check_sum(out, ref, scale, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(2, 50, 8, 32, 64, 1), (3, 7, 8, 16, 16, 2), (1, 33, 16, 64, 128, 2), (5, 300, 8, 32, 64, 1)])
+@pytest.mark.parametrize("shape", [(2, 50, 8, 32, 64, 1), (3, 7, 8, 16, 16, 2), (1, 33, 16, 64, 128, 2), (5, 300, 8, 32, 64, 1),
+                                   (2, 9, 8, 24, 16, 1), (1, 21, 24, 24, 16, 1), (3, 70, 40, 40, 16, 1)])  # rows the lanes do not cover exactly
 def test_post_backward(shape, dtype):
     Bsz, L, H, P, N, G = shape
     p = params(H, P, N, G, 4)
