@@ -526,9 +526,23 @@ __global__ __launch_bounds__(256) void bwd_head_sums_kernel(const double *__rest
     __shared__ double red[2][256];
     const int h = blockIdx.x;
     double sa = 0.0, sd = 0.0;
-    for (long long i = threadIdx.x; i < (long long)s.B * s.nc; i += blockDim.x) {
-        sa += dA_part[(size_t)h * ((size_t)s.B * s.nc) + i];
-        sd += dD_part[(size_t)h * ((size_t)s.B * s.nc) + i];
+    const long long n = (long long)s.B * s.nc;
+    const double *pa = dA_part + (size_t)h * (size_t)n, *pd = dD_part + (size_t)h * (size_t)n;
+    // eight parts per round, requested together (an index past the end reads the last part and adds zero)
+    for (long long i0 = threadIdx.x; i0 < n; i0 += 8LL * blockDim.x) {
+        double qa[8], qd[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const long long i = min(i0 + (long long)u * blockDim.x, n - 1);
+            qa[u] = pa[i];
+            qd[u] = pd[i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const bool in = i0 + (long long)u * blockDim.x < n;
+            sa += in ? qa[u] : 0.0;
+            sd += in ? qd[u] : 0.0;
+        }
     }
     red[0][threadIdx.x] = sa;
     red[1][threadIdx.x] = sd;

@@ -534,11 +534,27 @@ __global__ __launch_bounds__(256) void block_dt_bwd_kernel(const T *__restrict__
         float acc = 0.f;
         if (slot < slots) {
             const float bias = dt_bias[h];
-            for (long long row = (long long)blockIdx.x * slots + slot; row < rows; row += (long long)gridDim.x * slots) {
-                const float raw = (float)zxbcdt[(size_t)row * s.ld + off + h] + bias;
-                const float g = (float)ddt[(size_t)row * s.H + h] * sigmoidf(raw);
-                dzxbcdt[(size_t)row * s.ld + off + h] = (T)g;
-                acc += g;
+            // four rows per round, their loads requested together and without a condition (a row past the tensor
+            // reads the last row and is not stored): one trip to memory per round instead of one per row
+            constexpr int kRound = 4;
+            const long long stride = (long long)gridDim.x * slots;
+            for (long long row0 = (long long)blockIdx.x * slots + slot; row0 < rows; row0 += kRound * stride) {
+                T raw_q[kRound], ddt_q[kRound];
+#pragma unroll
+                for (int u = 0; u < kRound; ++u) {
+                    const size_t row = (size_t)min(row0 + u * stride, rows - 1);
+                    raw_q[u] = zxbcdt[row * s.ld + off + h];
+                    ddt_q[u] = ddt[row * s.H + h];
+                }
+#pragma unroll
+                for (int u = 0; u < kRound; ++u) {
+                    const long long row = row0 + u * stride;
+                    const float g = (float)ddt_q[u] * sigmoidf((float)raw_q[u] + bias);
+                    if (row < rows) {
+                        dzxbcdt[(size_t)row * s.ld + off + h] = (T)g;
+                        acc += g;
+                    }
+                }
             }
         }
         __syncthreads();
