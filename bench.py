@@ -21,16 +21,23 @@ fp32 accumulation, final states returned).  Prints ONE JSON line:
                compulsory traffic of the whole op.  Staged forward: the slowest stage.
   stages       the staged kernels issued one by one through their own entry points, each with
                its algorithmic bytes, GB/s and (stages 2, 4) dense MFMA rate; measured in both cases
-  stream_step  the single-timestep update at batch 4096: latency and GB/s; stream_steps_one_launch: the same
+  stream_step  the single-timestep update at batch 4096: latency and GB/s over the 64 steps, and over a loop of 1 000
+               steps with an event per step (mean and median); stream_steps_one_launch: the same
                64 steps as one call of ssd_steps_fwd (which runs 16 steps or more on the one-pass scan)
   reference_suite  the reference's historical benchmark cases for this path (batch 4, seq_len 4096,
                BFloat16) in the reference's result schema: mamba2_* rows time this library's whole Mamba-2 block
                (sizes in each row's config), ssd_scan_* rows the scan op alone
+  forward_float32_y  the float32-y instance of the headline kernel (bf16 inputs, y stored as float32): the output
+               err_y is measured on, timed beside the bf16-y instance, against its own compulsory traffic
+  workloads    the other configurations at full size (plumbing, long lookback, decay-extreme in bf16 and float32):
+               forward time (mean and median of 100 calls), path, HBM and MFMA fractions, errors of this run against
+               the oracle on the first batch row; --no-workloads skips them
   forward_float32  the same workload with float32 inputs (the other parity mode): time per call, which path ran (the
                float one-pass kernel on three bf16 terms per operand, or the staged kernels on float MFMAs), its
-               compulsory traffic against the HBM peak and the op's dense flops against the 157.3 TFLOP/s float MFMA
-               peak (the one-pass kernel multiplies on the bf16 matrix pipe, so that fraction may pass 1), and its
-               parity errors against the oracle on the first batch rows
+               compulsory traffic against the HBM peak, and its matrix-core rate against the pipe it multiplies on
+               (the one-pass kernel executes six bf16 products per float product: 6 x the dense flops against the
+               bf16 peak; the staged kernels the dense flops against the float MFMA peak), and its parity errors
+               against the oracle on the first batch rows
   backward     the backward pass of the scan at the same shape: time per call, and its compulsory traffic
                (x, dt, B, C, dy read; dx, ddt, dB, dC written) against the HBM peak
   mamba2_block the block around the scan at the policy shape (d_model = nheads*headdim): whole block, and the
@@ -66,6 +73,10 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MEASURED_TRAFFIC_BYTES = {("policy_bf16", 256): 491.9e6,          # 201 100 + 279 300 KiB, one launch
                           ("long_lookback_bf16", 32): 2012.4e6,   # 900 200 + 1 065 000 KiB, one launch
                           ("decay_extreme", 64): 325.0e6}         # states only 63 060 + 12 290, forward 106 700 + 135 400 KiB
+TRAFFIC_MEASURED_AT = "c6b6689"   # the library revision the counter runs in profiles/ were made at
+# matrix-pipe busy fraction of the same kernels from the same counter runs (SQ_VALU_MFMA_BUSY_CYCLES over
+# SQ_BUSY_CU_CYCLES): what the north star's "MFMA utilisation" reads as on the hardware's own counters
+MEASURED_MFMA_PIPE_BUSY = {("policy_bf16", 256): 0.27, ("long_lookback_bf16", 32): 0.238}
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 
@@ -83,6 +94,7 @@ def parse_args():
     ap.add_argument("--no-block", action="store_true")
     ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--no-float32", action="store_true")
+    ap.add_argument("--no-workloads", action="store_true", help="skip the other workloads' rows (full size, forward only)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise kernel over 256 MiB in / 256 MiB out three times, the known-size "
@@ -91,6 +103,18 @@ def parse_args():
 
 
 SPIN_SECONDS = 0.25
+
+
+def f32_mfma(dense_flops, seconds, on_bf16_pipe):
+    """The float32 mode's matrix-core figures against the pipe the path multiplies on: the float one-pass kernel forms
+    every product from six bf16 MFMAs (three bf16 terms per operand), so it executes 6 x the op's dense flops on the
+    bf16 pipe; the staged float kernels use float MFMAs."""
+    if on_bf16_pipe:
+        executed = 6.0 * dense_flops
+        return {"mfma_pipe": "bf16 (six bf16 products per float product)", "executed_TFLOPs": round(executed / seconds / 1e12, 1),
+                "peak_TFLOPs": MFMA_BF16_PEAK_TFLOPS, "mfma_frac": round(executed / seconds / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    return {"mfma_pipe": "float32", "executed_TFLOPs": round(dense_flops / seconds / 1e12, 1),
+            "peak_TFLOPs": MFMA_F32_PEAK_TFLOPS, "mfma_frac": round(dense_flops / seconds / 1e12 / MFMA_F32_PEAK_TFLOPS, 4)}
 
 
 def spin(fn, torch, seconds=SPIN_SECONDS):
@@ -300,16 +324,39 @@ def main():
             forward()
             oe[i][1].record()
         torch.cuda.synchronize()
-        ms = sum(a.elapsed_time(b) for a, b in oe) / args.steps
+        per_call = sorted(a.elapsed_time(b) for a, b in oe)
+        ms = sum(per_call) / args.steps
+        ms_median = per_call[len(per_call) // 2]
         ab = algorithmic_bytes_fwd(w)
         gbs = ab / (ms * 1e-3) / 1e9
         tf = sum(sf[k] for k in ("chunk_state", "chunk_scan")) / (ms * 1e-3) / 1e12
-        onepass_info = {"ms": round(ms, 5), "alg_bytes": ab, "GBps": round(gbs, 1),
+        onepass_info = {"ms": round(ms, 5), "ms_median": round(ms_median, 5), "calls": args.steps, "alg_bytes": ab,
+                        "GBps": round(gbs, 1),
                         "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "dense_TFLOPs": round(tf, 1),
                         "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)}
         roofline = {"kernel": "onepass_scan" if onepass else f"onepass_scan on {segments} segments", "bound": "hbm", "achieved": onepass_info["GBps"],
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": onepass_info["hbm_frac"],
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, w.batch))}
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, w.batch)),
+                    "traffic_measured_at": TRAFFIC_MEASURED_AT if (w.name, w.batch) in MEASURED_TRAFFIC_BYTES else None,
+                    "mfma_pipe_busy": MEASURED_MFMA_PIPE_BUSY.get((w.name, w.batch)),
+                    "mfma_pipe_busy_note": "SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CU_CYCLES of the same kernel, from the "
+                                           "rocprofv3 --pmc run of the same revision (profiles/)"}
+        if w.dtype == "bf16":
+            # the float32-y instance of the same kernel: the output err_y is measured on (bf16 inputs, y in float32,
+            # so its compulsory traffic holds y at four bytes per element)
+            y32buf = torch.empty(x.shape, dtype=torch.float32, device="cuda")
+            fwd32 = ssd.PreparedChunkScan(x, dt, A, Bm, Cm, D, chunk=w.chunk, initial_states=init, workspace=ws, out=y32buf,
+                                          final_out=final)
+            spin(fwd32, torch)
+            t32y, _ = event_time_steps(fwd32, args.steps, torch)
+            ab32 = ab + 2 * x.numel()
+            y32_info = {"ms": round(t32y * 1e3, 5), "alg_bytes": ab32, "GBps": round(ab32 / t32y / 1e9, 1),
+                        "hbm_frac": round(ab32 / t32y / 1e9 / HBM_PEAK_GBS, 4),
+                        "units_per_s": round(w.units / t32y, 1),
+                        "note": "the instance err_y is measured on; the headline instance stores the same y rounded to bf16"}
+            del y32buf, fwd32
+        else:
+            y32_info = None
     else:
         dom = max(stages, key=lambda k: stages[k]["ms"])
         roofline = {"kernel": dom, "bound": "hbm", "achieved": stages[dom]["GBps"], "peak": HBM_PEAK_GBS,
@@ -336,6 +383,9 @@ def main():
     }
     if onepass or segments > 1:
         out["onepass_scan"] = onepass_info
+        out["ms_per_call_median"] = onepass_info["ms_median"]
+        if y32_info is not None:
+            out["forward_float32_y"] = y32_info
 
     # ---- the same workload in float32 mode (the north star's other parity mode): bound by the float MFMAs ----
     if not args.no_float32 and w.dtype == "bf16":
@@ -374,8 +424,8 @@ def main():
                                       else (f"one-pass on {f32_segments} segments (three bf16 terms per operand)" if f32_segments > 1 else "staged"),
                                       "compulsory_io_bytes": io32,
                                       "hbm_frac": round(io32 / t32 / 1e9 / HBM_PEAK_GBS, 4),
-                                      "dense_TFLOPs": round(fl / t32 / 1e12, 1), "peak_TFLOPs": MFMA_F32_PEAK_TFLOPS,
-                                      "mfma_frac": round(fl / t32 / 1e12 / MFMA_F32_PEAK_TFLOPS, 4),
+                                      "dense_TFLOPs": round(fl / t32 / 1e12, 1),
+                                      **f32_mfma(fl, t32, f32_onepass or f32_segments > 1),
                                       "units_per_s": round(w.batch * w.seqlen / t32, 1),
                                       "err_y": e32[0], "err_final": e32[1], "tolerance": 1e-4}
             del y32o, f32o
@@ -400,6 +450,69 @@ def main():
                            "hbm_frac": round(bwd_bytes / t_bwd / 1e9 / HBM_PEAK_GBS, 4),
                            "workspace_bytes": wsb.numel(), "units_per_s": round(BL / t_bwd, 1)}
         del dyb, wsb
+
+    # ---- the other workloads at full size: forward only, one row each -----------------------------------
+    # (the configurations beside the headline one: parity for them is in the tests; here their time, path, traffic
+    # fractions and this run's errors against the oracle on the first batch row, so that one run covers them all)
+    if not args.no_workloads and args.workload == "policy_bf16" and not args.batch:
+        rows_out = []
+        for wname, wdtype in (("plumbing_f32", "f32"), ("long_lookback_bf16", "bf16"), ("decay_extreme", "bf16"),
+                              ("decay_extreme", "f32")):
+            ww = WORKLOADS[wname].with_dtype(wdtype)
+            wi = make_inputs(ww, seed=0, device="cuda")
+            call = ssd.PreparedChunkScan(wi["x"], wi["dt"], wi["A"], wi["B"], wi["C"], wi["D"], chunk=ww.chunk,
+                                         initial_states=wi["init"])
+            spin(call, torch, 0.1)
+            n_calls = 100
+            we = [torch.cuda.Event(enable_timing=True) for _ in range(n_calls + 1)]
+            torch.cuda.synchronize()
+            we[0].record()
+            for i in range(n_calls):
+                call()
+                we[i + 1].record()
+            torch.cuda.synchronize()
+            per = sorted(we[i].elapsed_time(we[i + 1]) for i in range(n_calls))
+            t_w = we[0].elapsed_time(we[n_calls]) * 1e-3 / n_calls
+            wy, wf = call()
+            if wdtype == "bf16":   # judged on the float32 y of the same kernel, as the headline
+                wy32, _ = ssd.ssd_chunk_scan(wi["x"], wi["dt"], wi["A"], wi["B"], wi["C"], wi["D"], chunk=ww.chunk,
+                                             initial_states=wi["init"], y_dtype=torch.float32)
+                stored_ok = bool(torch.equal(wy, wy32.to(torch.bfloat16)))
+            else:
+                wy32, stored_ok = wy, None
+            torch.cuda.synchronize()
+
+            def one(t):
+                return None if t is None else t[:1].float().cpu().numpy().astype(np.float64)
+
+            yr, fr = c_oracle.ssd_sequential_c(one(wi["x"]), one(wi["dt"]), wi["A"].cpu().numpy().astype(np.float64),
+                                               one(wi["B"]), one(wi["C"]), wi["D"].cpu().numpy().astype(np.float64),
+                                               one(wi["init"]), nthreads=min(16, os.cpu_count() or 1))
+            segs = ssd.chunk_scan_segments(ww.batch, ww.seqlen, ww.nheads, ww.headdim, ww.dstate, ww.ngroups, ww.chunk,
+                                           ww.torch_dtype)
+            one_launch = ssd.chunk_scan_is_onepass(ww.batch, ww.seqlen, ww.nheads, ww.headdim, ww.dstate, ww.ngroups,
+                                                   ww.chunk, ww.torch_dtype)
+            wab = algorithmic_bytes_fwd(ww)
+            wfl = sum(stage_flops(ww)[k] for k in ("chunk_state", "chunk_scan"))
+            row = {"workload": wname, "dtype": wdtype, "batch": ww.batch, "seqlen": ww.seqlen, "nheads": ww.nheads,
+                   "headdim": ww.headdim, "dstate": ww.dstate, "ngroups": ww.ngroups, "chunk": ww.chunk,
+                   "ms": round(t_w * 1e3, 5), "ms_median": round(per[n_calls // 2], 5), "calls": n_calls,
+                   "path": "onepass" if one_launch else (f"onepass on {segs} segments" if segs > 1 else "staged"),
+                   "alg_bytes": wab, "hbm_frac": round(wab / t_w / 1e9 / HBM_PEAK_GBS, 4),
+                   "units_per_s": round(ww.units / t_w, 1), "dense_TFLOPs": round(wfl / t_w / 1e12, 1),
+                   "err_y": orc.rel_err(wy32[:1].float().cpu().numpy(), yr), "err_final": orc.rel_err(wf[:1].cpu().numpy(), fr),
+                   "err_rows": 1, "tolerance": 2e-2 if wdtype == "bf16" else 1e-4}
+            if wdtype == "bf16":
+                row["mfma_frac"] = round(wfl / t_w / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
+                row["stored_y_is_rounded_f32_y"] = stored_ok
+                row["mfma_pipe_busy"] = MEASURED_MFMA_PIPE_BUSY.get((wname, ww.batch))
+                row["traffic"] = MEASURED_TRAFFIC_BYTES.get((wname, ww.batch))
+            else:
+                row.update(f32_mfma(wfl, t_w, one_launch or segs > 1))
+            rows_out.append(row)
+            del wi, call, wy, wf, wy32, yr, fr
+            torch.cuda.empty_cache()
+        out["workloads"] = rows_out
 
     # ---- streaming step at batch 4096 ---------------------------------------------------------
     if not args.no_stream_step:
@@ -427,6 +540,22 @@ def main():
         out["stream_step"] = {"batch": sw.batch, "steps": sw.stream_steps, "us_per_step": round(us, 2),
                               "alg_bytes": step_bytes(sw), "GBps": round(gbs, 1),
                               "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
+        # a 1 000-step loop of the same update (the 64 steps' inputs in turn), an event around every step: mean and median
+        n_loop = 1000
+        le = [torch.cuda.Event(enable_timing=True) for _ in range(n_loop + 1)]
+        torch.cuda.synchronize()
+        le[0].record()
+        for t in range(n_loop):
+            k = t % sw.stream_steps
+            ssd.ssd_step(state, xs[k], ds[k], si["A"], bs[k], cs[k], si["D"], out=ys)
+            le[t + 1].record()
+        torch.cuda.synchronize()
+        per_step = sorted(le[t].elapsed_time(le[t + 1]) * 1e3 for t in range(n_loop))
+        us_loop = le[0].elapsed_time(le[n_loop]) * 1e3 / n_loop
+        out["stream_step"]["loop_1000"] = {"us_per_step": round(us_loop, 2), "us_median": round(per_step[n_loop // 2], 2),
+                                           "GBps": round(step_bytes(sw) / (us_loop * 1e-6) / 1e9, 1),
+                                           "hbm_frac": round(step_bytes(sw) / (us_loop * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+        del le
         # the same 64 steps as ONE launch (state in registers between the steps): per-step latency, and the
         # traffic of the launch = state in and out once plus the 64 steps' inputs and outputs
         xs64, ds64 = si["x"].contiguous(), si["dt"].contiguous()

@@ -157,6 +157,40 @@ fn opt_u8(t: Option<&Tensor>) -> *const u8 {
     t.map_or(std::ptr::null(), |t| t.data_ptr() as *const u8)
 }
 
+/// A raw HIP stream handle (`hipStream_t`) as the library takes it; `None` is the legacy default stream.
+pub type StreamHandle = Option<*mut c_void>;
+
+fn stream_ptr(stream: StreamHandle) -> *mut c_void {
+    stream.unwrap_or(std::ptr::null_mut())
+}
+
+extern "C" {
+    /// The getter this binding needs from the vendored torch shim (`vendor/torch-sys-0.25.0/libtch/torch_api.{h,cpp}`,
+    /// next to the graph stream-scope helpers at `torch_api.cpp:408-464`): the raw handle of the calling thread's
+    /// current stream on `device_index`, i.e. the capture stream while `at_cuda_graph_stream_begin` is in scope.
+    /// INTEGRATION.md gives the patch.  Errors go to the shim's thread-local `torch_last_err`, as for its other calls.
+    pub fn at_cuda_current_stream(device_index: i64) -> *mut c_void;
+}
+
+/// The current stream of `device` for the calling thread: pass it to the wrappers below so that the kernels land
+/// on the stream torch's own work is on (and inside a graph capture, `train/update.rs:206-330`).
+pub fn current_stream(device: tch::Device) -> Result<StreamHandle> {
+    match device {
+        tch::Device::Cuda(index) => {
+            let handle = unsafe { at_cuda_current_stream(index as i64) };
+            // the shim's own error slot, read the way `torch/cuda/graph.rs:107-119` reads it
+            let err = unsafe { torch_sys::get_and_reset_last_err() };
+            if !err.is_null() {
+                let msg = unsafe { CStr::from_ptr(err) }.to_string_lossy().into_owned();
+                unsafe { libc::free(err.cast()) };
+                bail!("at_cuda_current_stream: {msg}");
+            }
+            Ok(Some(handle))
+        }
+        other => bail!("SSD runs on a GPU stream, got device {other:?}"),
+    }
+}
+
 fn require(name: &str, t: &Tensor, shape: &[i64], kind: Kind) -> Result<()> {
     if !t.device().is_cuda() {
         bail!("SSD {name} must be on the GPU, got {:?}", t.device());
@@ -206,9 +240,11 @@ fn validate_scan(dims: &SsdDims, x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor
 
 /// SSD chunk-scan forward: y `[B,L,H,P]` (x's kind) and final states `[B,H,P,N]` f32.
 /// `reset` `[B,L]` u8: a non-zero entry restarts that row's state from zero before the timestep.
-/// The stream is NULL (the legacy default stream): the vendored torch-sys exposes no current-stream getter.
+/// `stream`: where the kernels are issued -- `current_stream(x.device())?` for torch's current stream (what a caller
+/// inside the captured update must pass), `None` for the legacy default stream.
 pub fn ssd_chunk_scan(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tensor, d: Option<&Tensor>, chunk: i64,
-                      initial_states: Option<&Tensor>, reset: Option<&Tensor>) -> Result<(Tensor, Tensor)> {
+                      initial_states: Option<&Tensor>, reset: Option<&Tensor>, stream: StreamHandle)
+                      -> Result<(Tensor, Tensor)> {
     let dims = scan_dims(x, b, chunk)?;
     validate_scan(&dims, x, dt, a, b, c, d, initial_states, reset)?;
     let mut need = 0usize;
@@ -219,7 +255,7 @@ pub fn ssd_chunk_scan(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tenso
     check(unsafe {
         ssd_chunk_scan_reset_fwd(&dims, dtype_code(x)?, x.data_ptr(), dt.data_ptr(), a.data_ptr() as *const f32,
                                  b.data_ptr(), c.data_ptr(), opt_f32(d), opt_f32(initial_states), opt_u8(reset),
-                                 y.data_ptr(), fin.data_ptr() as *mut f32, ws.data_ptr(), need, std::ptr::null_mut())
+                                 y.data_ptr(), fin.data_ptr() as *mut f32, ws.data_ptr(), need, stream_ptr(stream))
     })?;
     Ok((y, fin))
 }
@@ -229,7 +265,7 @@ pub fn ssd_chunk_scan(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tenso
 /// unless they run as one launch of the one-pass kernel.  Calls that overlap on one GPU race on that array.
 pub fn ssd_chunk_scan_noalloc(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tensor, d: Option<&Tensor>,
                               chunk: i64, initial_states: Option<&Tensor>, reset: Option<&Tensor>, y: &mut Tensor,
-                              final_states: &mut Tensor) -> Result<()> {
+                              final_states: &mut Tensor, stream: StreamHandle) -> Result<()> {
     let dims = scan_dims(x, b, chunk)?;
     validate_scan(&dims, x, dt, a, b, c, d, initial_states, reset)?;
     require("y", y, &x.size(), x.kind())?;
@@ -237,13 +273,13 @@ pub fn ssd_chunk_scan_noalloc(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c
     check(unsafe {
         ssd_chunk_scan_noalloc_fwd(&dims, dtype_code(x)?, x.data_ptr(), dt.data_ptr(), a.data_ptr() as *const f32,
                                    b.data_ptr(), c.data_ptr(), opt_f32(d), opt_f32(initial_states), opt_u8(reset),
-                                   y.data_ptr(), final_states.data_ptr() as *mut f32, std::ptr::null_mut())
+                                   y.data_ptr(), final_states.data_ptr() as *mut f32, stream_ptr(stream))
     })
 }
 
 /// Advances `state` `[B,H,P,N]` f32 in place by one timestep; returns y `[B,H,P]`.
 pub fn ssd_step(state: &mut Tensor, x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tensor,
-                d: Option<&Tensor>) -> Result<Tensor> {
+                d: Option<&Tensor>, stream: StreamHandle) -> Result<Tensor> {
     let (ss, bs) = (state.size(), b.size());
     if ss.len() != 4 || bs.len() != 3 {
         bail!("SSD state must be [B,H,P,N] and B [B,G,N], got {ss:?} and {bs:?}");
@@ -255,7 +291,7 @@ pub fn ssd_step(state: &mut Tensor, x: &Tensor, dt: &Tensor, a: &Tensor, b: &Ten
     check(unsafe {
         ssd_step_fwd(&dims, dtype_code(x)?, state.data_ptr() as *mut f32, x.data_ptr(), dt.data_ptr(),
                      a.data_ptr() as *const f32, b.data_ptr(), c.data_ptr(), opt_f32(d), y.data_ptr(),
-                     std::ptr::null_mut())
+                     stream_ptr(stream))
     })?;
     Ok(y)
 }
@@ -263,7 +299,7 @@ pub fn ssd_step(state: &mut Tensor, x: &Tensor, dt: &Tensor, a: &Tensor, b: &Ten
 /// `nsteps` timesteps in one launch (inputs `[B,T,...]`), `reset` `[B,T]` u8 marking rows to zero right before a
 /// step: the rollout's advance -> reset slots -> forward (`train/rollout.rs:209-235`) as one call.
 pub fn ssd_steps(state: &mut Tensor, x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tensor, d: Option<&Tensor>,
-                 reset: Option<&Tensor>) -> Result<Tensor> {
+                 reset: Option<&Tensor>, stream: StreamHandle) -> Result<Tensor> {
     let (ss, xs, bs) = (state.size(), x.size(), b.size());
     if ss.len() != 4 || xs.len() != 4 || bs.len() != 4 {
         bail!("SSD steps: state [B,H,P,N], x [B,T,H,P], B [B,T,G,N], got {ss:?}, {xs:?}, {bs:?}");
@@ -273,7 +309,7 @@ pub fn ssd_steps(state: &mut Tensor, x: &Tensor, dt: &Tensor, a: &Tensor, b: &Te
     check(unsafe {
         ssd_steps_fwd(&dims, xs[1], dtype_code(x)?, state.data_ptr() as *mut f32, opt_u8(reset), x.data_ptr(),
                       dt.data_ptr(), a.data_ptr() as *const f32, b.data_ptr(), c.data_ptr(), opt_f32(d), y.data_ptr(),
-                      std::ptr::null_mut())
+                      stream_ptr(stream))
     })?;
     Ok(y)
 }
@@ -291,7 +327,8 @@ pub struct SsdGrads {
 
 pub fn ssd_chunk_scan_backward(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, c: &Tensor, d: Option<&Tensor>,
                                dy: &Tensor, chunk: i64, initial_states: Option<&Tensor>, reset: Option<&Tensor>,
-                               dfinal_states: Option<&Tensor>, need_dinitial_states: bool) -> Result<SsdGrads> {
+                               dfinal_states: Option<&Tensor>, need_dinitial_states: bool, stream: StreamHandle)
+                               -> Result<SsdGrads> {
     let dims = scan_dims(x, b, chunk)?;
     validate_scan(&dims, x, dt, a, b, c, d, initial_states, reset)?;
     require("dy", dy, &x.size(), x.kind())?;
@@ -316,7 +353,7 @@ pub fn ssd_chunk_scan_backward(x: &Tensor, dt: &Tensor, a: &Tensor, b: &Tensor, 
                            c.data_ptr(), opt_f32(d), opt_f32(initial_states), opt_u8(reset), dy.data_ptr(),
                            opt_f32(dfinal_states), g.dx.data_ptr(), g.ddt.data_ptr(), g.da.data_ptr() as *mut f32,
                            g.db.data_ptr(), g.dc.data_ptr(), opt_mut(&g.dd), opt_mut(&g.dinitial_states),
-                           ws.data_ptr(), need, std::ptr::null_mut())
+                           ws.data_ptr(), need, stream_ptr(stream))
     })?;
     Ok(g)
 }

@@ -150,7 +150,11 @@ int ssd_chunk_scan_reset_fwd(const ssd_dims *dims, int dtype, const void *x, con
  * (ssd_chunk_scan_is_onepass), at any size.  Calls no hipMalloc/hipFree or any other allocating
  * routine.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different streams or
  * threads) race on it; calls on one stream are ordered and safe.  Nothing in the array has to start at zero (every
- * kernel writes what it later reads), so it is not cleared between calls. */
+ * kernel writes what it later reads), so it is not cleared between calls.
+ * Under graph capture: the first call on a device places the array there and looks its address up, and the first call
+ * for a shape asks the runtime for occupancy figures and raises LDS limits -- none of that may run inside a capture.
+ * Make one call per device and shape outside the capture first; every later call of that shape issues kernel launches
+ * only and can be captured and replayed. */
 #define SSD_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 int ssd_chunk_scan_noalloc_fwd(const ssd_dims *dims, int dtype, const void *x, const void *dt, const float *A,
                                const void *Bm, const void *Cm, const float *D, const float *initial_states,

@@ -102,6 +102,29 @@ def test_rust_binding_matches_the_header():
             assert a == b, f"{name}: parameter {i} is {a} in ssd.rs, {b} in the header"
 
 
+def test_rust_wrappers_pass_the_callers_stream():
+    """Every public wrapper that launches kernels takes a `stream: StreamHandle` and hands `stream_ptr(stream)` to the
+    library as the last argument of its call; none passes a NULL stream of its own.  The getter the binding needs from
+    the torch shim is declared with the shim's calling convention (a device index in, a raw handle out)."""
+    text = re.sub(r"//[^\n]*", "", (REPO / "bindings" / "rust" / "ssd.rs").read_text())
+    launching = {"ssd_chunk_scan": "ssd_chunk_scan_reset_fwd", "ssd_chunk_scan_noalloc": "ssd_chunk_scan_noalloc_fwd",
+                 "ssd_step": "ssd_step_fwd", "ssd_steps": "ssd_steps_fwd", "ssd_chunk_scan_backward": "ssd_chunk_scan_bwd"}
+    for wrapper, entry in launching.items():
+        m = re.search(r"pub fn " + wrapper + r"\s*\(([^)]*)\)[^{]*\{(.*?)\n\}\n", text, flags=re.S)
+        assert m, wrapper
+        params, body = m.group(1), m.group(2)
+        assert re.search(r"\bstream\s*:\s*StreamHandle\s*$", params.strip()), f"{wrapper} must end in stream: StreamHandle"
+        call = re.search(entry + r"\s*\((.*?)\)\s*\}\)", body, flags=re.S)
+        assert call, f"{wrapper} does not call {entry}"
+        assert call.group(1).rstrip().endswith("stream_ptr(stream)"), f"{wrapper} must pass the caller's stream to {entry}"
+    assert re.search(r"fn\s+stream_ptr\s*\(\s*stream\s*:\s*StreamHandle\s*\)\s*->\s*\*mut\s+c_void", text)
+    assert re.search(r"pub type StreamHandle\s*=\s*Option<\*mut c_void>", text)
+    assert re.search(r"pub fn at_cuda_current_stream\s*\(\s*device_index\s*:\s*i64\s*\)\s*->\s*\*mut c_void", text)
+    # the patch for the shim that INTEGRATION.md gives declares the same function
+    integ = (REPO / "INTEGRATION.md").read_text()
+    assert "void *at_cuda_current_stream(int64_t device_index);" in integ
+
+
 def test_rust_structs_match_the_header():
     htext = re.sub(r"/\*.*?\*/", "", (REPO / "include" / "ssd_hip.h").read_text(), flags=re.S)
     rtext = re.sub(r"//[^\n]*", "", (REPO / "bindings" / "rust" / "ssd.rs").read_text())

@@ -178,3 +178,52 @@ def test_block_backward_is_the_directional_derivative_of_the_gpu_forward():
     num = float((up - dn) / (2 * h))
     ana = float((du.double() * v.double()).sum())
     assert abs(num - ana) <= 2e-3 * max(abs(ana), 1.0), (num, ana)
+
+
+@pytest.mark.parametrize("d_conv", [2, 3])
+def test_block_backward_with_short_filters_at_training_size(d_conv):
+    """A block with a filter shorter than four taps at 32 768 rows: the two backward stages share one scratch buffer
+    sized from the filter length, and from this many rows on its conv part is the larger one, so both stages must be
+    told the same length.  The size also sends the weight gradients through their slabbed path and the projections
+    through the library's kernel."""
+    b = Mamba2Block(d_model=128, nheads=8, headdim=16, dstate=16, ngroups=1, d_conv=d_conv, seed=5)
+    Bsz, L = 8, 4096
+    g = torch.Generator().manual_seed(25 + d_conv)
+    u = torch.randn(Bsz, L, 128, generator=g).to(torch.bfloat16).cuda()
+    dout = torch.randn(Bsz, L, 128, generator=g).to(torch.bfloat16).cuda()
+    out, ctx = b.forward(u, save_for_backward=True)
+    got = b.backward(ctx, dout)
+    torch.cuda.synchronize()
+    from test_gpu_block import oracle_params
+    ref = blk.block_backward(np64(u), oracle_params(b), np64(dout))
+    for key in ("du", "din_proj", "dconv_w", "dconv_b", "ddt_bias", "dA", "dD", "dnorm_w", "dout_proj"):
+        o = got[key].detach().float().cpu().numpy().astype(np.float64)
+        r = ref[key]
+        assert o.shape == r.shape, key
+        # the small block test's bar (1.5e-1 rms for the chain's eight or so bf16 roundings) plus, for du -- four
+        # million elements stored in bf16, the largest of them ten rms out -- a share of the element itself
+        rms = max(np.sqrt(np.mean(r * r)), 1e-30)
+        over = np.abs(o - r) - (1.5e-1 * rms + (2.0 ** -6 * np.abs(r) if key == "du" else 0.0))
+        assert np.isfinite(o).all() and over.max() <= 0, f"{key}: over the bar by {over.max() / rms:.3e} rms"
+        assert np.corrcoef(o.ravel(), r.ravel())[0, 1] > 0.999, key
+
+
+@pytest.mark.parametrize("rows,e,ld,d", [(16384, 648, 704, 256), (32768, 256, 256, 64), (8192, 40, 64, 128)])
+def test_weight_gradient_slabs_against_float64(rows, e, ld, d):
+    """a^T b over many rows (bf16): the slabbed batched product with float32 partial sums, fed a view into wider
+    rows as the block's backward does, against the float64 product of the same bf16 values.  Each output is a sum of
+    `rows` products rounded once each to float32 at most: within 1e-3 of the summed terms' 2-norm."""
+    from trading_bot_0_amd.block import _weight_gradient
+    g = torch.Generator().manual_seed(rows + e)
+    buf = torch.randn(rows, ld, generator=g).to(torch.bfloat16).cuda()
+    a = buf[:, :e]
+    bm = torch.randn(rows, d, generator=g).to(torch.bfloat16).cuda()
+    got = _weight_gradient(a, bm)
+    torch.cuda.synchronize()
+    assert got.shape == (e, d) and got.dtype == torch.float32
+    a64, b64 = a.double().cpu().numpy(), bm.double().cpu().numpy()
+    ref = a64.T @ b64
+    scale = np.sqrt((a64 * a64).sum(0))[:, None] * np.abs(b64).max()
+    err = (np.abs(got.double().cpu().numpy() - ref) / scale).max()
+    assert err <= 1e-3, f"{err:.3e}"
+    assert torch.equal(got, _weight_gradient(a, bm)), "the same bits on a second run"

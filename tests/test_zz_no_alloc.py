@@ -2,7 +2,12 @@
 against ssd_chunk_scan_reset_fwd with a caller-owned workspace: the same kernels on a different scratch buffer, so
 y and the final states must be equal bit for bit.  Each case makes two calls in a row on the library's static
 scratch array, the second with a smaller input (the array still holds the first call's intermediates), and checks
-that the device's free memory does not move across the calls."""
+that the device's free memory does not move across the calls.
+
+The comparison is with the workspace entry point, not with the oracle: the two run the same kernels and differ only in
+the base pointer of the scratch they are handed (same layout behind it), so a bug in that layout would corrupt both
+alike and is what the workspace entry point's own tests against the oracle (tests/test_gpu_scan.py) are for; what this
+file can catch is what is particular to the static array: its address, its size limit, stale contents."""
 from ctypes import byref, c_size_t
 
 import pytest
@@ -109,3 +114,56 @@ def test_noalloc_forward_takes_the_full_policy_shape_and_refuses_what_does_not_f
     rc = lib.ssd_chunk_scan_noalloc_fwd(byref(dims), ssd.SSD_DTYPE_BF16, x16.data_ptr(), inp["dt"].data_ptr(), inp["A"].data_ptr(),
                                         inp["B"].data_ptr(), inp["C"].data_ptr(), None, None, None, y.data_ptr(), None, None)
     assert rc == 3 and "static scratch" in ssd.last_error(lib)
+
+
+@pytest.mark.parametrize("name,batch,seqlen", [("policy_bf16", 4, 300), ("policy_bf16", 32, 2048)])
+def test_noalloc_forward_captured_in_a_graph(name, batch, seqlen):
+    """One staged and one segmented shape: a call outside the capture first (it places the array, asks for occupancy
+    figures and raises LDS limits), then the same call captured in a graph and replayed twice with eager work and
+    synchronisation between the replays; every replay must equal the workspace entry point bit for bit."""
+    lib = ssd.load_library()
+    torch.cuda.set_device(0)
+    prime(lib)
+    w = WORKLOADS[name].with_batch(batch)
+    inp = make_inputs(w, seed=5, device="cuda", seqlen=seqlen)
+    x, dt, A, Bm, Cm, D = (inp[k] for k in ("x", "dt", "A", "B", "C", "D"))
+    Bsz, L, H, P = x.shape
+    G, N = Bm.shape[2], Bm.shape[3]
+    segments = ssd.chunk_scan_segments(Bsz, L, H, P, N, G, w.chunk)
+    assert (segments > 1) == (batch == 32)
+    dims = ssd.SsdDims(Bsz, L, H, P, N, G, w.chunk)
+    reset = torch.zeros(Bsz, L, dtype=torch.uint8, device="cuda")
+    reset[1, L // 2] = 1
+    need = c_size_t(0)
+    ssd._check(lib, lib.ssd_workspace_bytes(byref(dims), byref(need)))
+    ws = torch.empty(need.value, dtype=torch.uint8, device="cuda")
+    y_ref, f_ref = torch.empty_like(x), torch.empty(Bsz, H, P, N, device="cuda")
+    y_new, f_new = torch.empty_like(x), torch.empty(Bsz, H, P, N, device="cuda")
+
+    def common(xx):
+        return (xx.data_ptr(), dt.data_ptr(), A.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), D.data_ptr(), None,
+                reset.data_ptr())
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):   # the call of this shape outside the capture
+        ssd._check(lib, lib.ssd_chunk_scan_noalloc_fwd(byref(dims), ssd.SSD_DTYPE_BF16, *common(x), y_new.data_ptr(),
+                                                       f_new.data_ptr(), side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ssd._check(lib, lib.ssd_chunk_scan_noalloc_fwd(byref(dims), ssd.SSD_DTYPE_BF16, *common(x), y_new.data_ptr(),
+                                                       f_new.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    for replay in range(2):
+        x.copy_(torch.randn(x.shape, device="cuda").to(x.dtype))   # eager work between the replays: new inputs
+        y_new.fill_(float("nan"))
+        f_new.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        ssd._check(lib, lib.ssd_chunk_scan_reset_fwd(byref(dims), ssd.SSD_DTYPE_BF16, *common(x), y_ref.data_ptr(),
+                                                     f_ref.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                     torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert not torch.isnan(y_new.float()).any()
+        assert torch.equal(y_new, y_ref) and torch.equal(f_new, f_ref), f"replay {replay}"

@@ -167,9 +167,11 @@ def block_bwd_workspace(batch, seqlen, nheads, headdim, dstate, ngroups, d_conv=
     return torch.empty(need.value, dtype=torch.uint8, device=device)
 
 
-def block_post_bwd(y, zxbcdt, norm_w, dout, dzxbcdt, nheads, headdim, dstate, ngroups, eps=1e-5, workspace=None):
+def block_post_bwd(y, zxbcdt, norm_w, dout, dzxbcdt, nheads, headdim, dstate, ngroups, eps=1e-5, workspace=None,
+                   d_conv=4):
     """Gradients of block_post: returns (dy [B,L,H,P], dnorm_w [H*P]) and writes dz into the z channels of dzxbcdt
-    (a tensor laid out like zxbcdt, same row stride)."""
+    (a tensor laid out like zxbcdt, same row stride).  `d_conv` is the block's filter length: the library sizes the
+    scratch both backward calls of a pass share from it, so it must be the one `workspace` was sized with."""
     lib = _lib()
     Bsz, L, E = zxbcdt.shape
     H, P, N, G = nheads, headdim, dstate, ngroups
@@ -188,8 +190,8 @@ def block_post_bwd(y, zxbcdt, norm_w, dout, dzxbcdt, nheads, headdim, dstate, ng
     dy = torch.empty((Bsz, L, H, P), dtype=dtype, device=zxbcdt.device)
     dnorm_w = torch.empty(H * P, dtype=torch.float32, device=zxbcdt.device)
     if workspace is None:
-        workspace = block_bwd_workspace(Bsz, L, H, P, N, G, 4, dtype, zxbcdt.device)
-    dims = SsdBlockDims(Bsz, L, H, P, N, G, 4, ld)
+        workspace = block_bwd_workspace(Bsz, L, H, P, N, G, d_conv, dtype, zxbcdt.device)
+    dims = SsdBlockDims(Bsz, L, H, P, N, G, d_conv, ld)
     ssd._check(lib, lib.ssd_block_post_bwd(byref(dims), code, y.data_ptr(), zxbcdt.data_ptr(), norm_w.data_ptr(), c_float(eps),
                                            dout.data_ptr(), dy.data_ptr(), dzxbcdt.data_ptr(), dnorm_w.data_ptr(),
                                            workspace.data_ptr(), workspace.numel(), ssd._stream_ptr(zxbcdt)))
@@ -371,7 +373,8 @@ class Mamba2Block:
         dbuf = torch.empty((Bsz, L, ld), dtype=act, device=u.device)
         dzx = dbuf[..., :E] if ld != E else dbuf
         ws = block_bwd_workspace(Bsz, L, self.H, self.P, self.N, self.G, self.d_conv, act, u.device)
-        dy, dnorm_w = block_post_bwd(y, zxbcdt, self.norm_w, dyn, dzx, self.H, self.P, self.N, self.G, self.eps, workspace=ws)
+        dy, dnorm_w = block_post_bwd(y, zxbcdt, self.norm_w, dyn, dzx, self.H, self.P, self.N, self.G, self.eps, workspace=ws,
+                                     d_conv=self.d_conv)
         g = ssd.ssd_chunk_scan_backward(x, dt, self.A, Bm, Cm, self.D, dy, chunk=self.chunk, reset=reset)
         dconv_w, dconv_b, ddt_bias, _ = block_pre_bwd(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, g["dx"], g["dB"],
                                                       g["dC"], g["ddt"], dzx, self.H, self.P, self.N, self.G, reset=reset,

@@ -238,8 +238,11 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
     const int CP = C / kBwdCh;
     const int runs = (s.L + kBwdSteps - 1) / kBwdSteps;
     const int pl = threadIdx.x % kPiecesPerBlock, rl = threadIdx.x / kPiecesPerBlock;
-    const int piece = blockIdx.x * kPiecesPerBlock + pl;
-    const long long br = (long long)blockIdx.y * kRunsPerBlock + rl;
+    // one linear grid, piece blocks fastest (the grid's second dimension stops at 65 535 run blocks)
+    const unsigned piece_blocks = (CP + kPiecesPerBlock - 1) / kPiecesPerBlock;
+    const unsigned run_block = blockIdx.x / piece_blocks;
+    const int piece = (blockIdx.x % piece_blocks) * kPiecesPerBlock + pl;
+    const long long br = (long long)run_block * kRunsPerBlock + rl;
     const bool active = piece < CP && br < (long long)s.B * runs;
     float dwacc[kBwdCh][K], dbacc[kBwdCh];
 #pragma unroll
@@ -429,7 +432,7 @@ __global__ __launch_bounds__(256) void block_pre_bwd_kernel(const T *__restrict_
             for (int k = 0; k <= K; ++k) {
                 float acc = 0.f;
                 for (int q = 0; q < kRunsPerBlock; ++q) acc += red[(q * kPiecesPerBlock + pl) * (K + 1) + k];
-                part[(size_t)blockIdx.y * cols + (size_t)c * (K + 1) + k] = acc;
+                part[(size_t)run_block * cols + (size_t)c * (K + 1) + k] = acc;
             }
         }
     }
@@ -642,8 +645,9 @@ static hipError_t pre_bwd_dispatch(const BlockShape &s, const void *zxbcdt, cons
     const int DI = s.H * s.P, C = DI + 2 * s.G * s.N, CP = C / kBwdCh, K = s.d_conv;
     const long long runs = (s.L + kBwdSteps - 1) / kBwdSteps;
     const long long run_blocks = ((long long)s.B * runs + kRunsPerBlock - 1) / kRunsPerBlock;
-    if (run_blocks > 65535LL * 32768LL) return hipErrorInvalidValue;
-    const dim3 grid((CP + kPiecesPerBlock - 1) / kPiecesPerBlock, (unsigned)run_blocks);
+    const long long piece_blocks = (CP + kPiecesPerBlock - 1) / kPiecesPerBlock;
+    if (run_blocks * piece_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)(run_blocks * piece_blocks));
     const T *in = static_cast<const T *>(zxbcdt), *si = static_cast<const T *>(state_in);
     const T *gx = static_cast<const T *>(dx), *gb = static_cast<const T *>(dB), *gc = static_cast<const T *>(dC);
     const T *gso = static_cast<const T *>(dstate_out);

@@ -567,16 +567,19 @@ static inline hipError_t persistent_grid(K kernel, int block, size_t lds, int ti
     return hipSuccess;
 }
 
-// Raises a kernel's dynamic LDS limit to `bytes` (needed above 64 KiB), once per kernel, device and size.
+// Raises a kernel's dynamic LDS limit (needed above 64 KiB) to the CU's whole LDS, once per kernel and device.  The
+// attribute holds the last value set, so a limit set per size would be left at a smaller size by a later call that
+// found its own size already noted; the CU's limit serves every size a launcher can ask for.
 template <typename K> static inline hipError_t allow_lds(K kernel, size_t bytes) {
     if (bytes <= 64 * 1024) return hipSuccess;
+    if (bytes > kLdsLimitBytes) return hipErrorInvalidValue;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     const void *kp = reinterpret_cast<const void *>(kernel);
-    const uint64_t key = launch_config_key(2, dev, 0, bytes);
+    const uint64_t key = launch_config_key(2, dev, 0, 0);
     if (launch_facts().find(kp, key) == 1) return hipSuccess;
-    e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimitBytes);
     if (e == hipSuccess) launch_facts().keep(kp, key, 1);
     return e;
 }
