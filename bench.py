@@ -346,7 +346,7 @@ def main():
             # so its compulsory traffic holds y at four bytes per element)
             y32buf = torch.empty(x.shape, dtype=torch.float32, device="cuda")
             fwd32 = ssd.PreparedChunkScan(x, dt, A, Bm, Cm, D, chunk=w.chunk, initial_states=init, workspace=ws, out=y32buf,
-                                          final_out=final)
+                                          final_out=final, y_dtype=torch.float32)
             spin(fwd32, torch)
             t32y, _ = event_time_steps(fwd32, args.steps, torch)
             ab32 = ab + 2 * x.numel()
@@ -694,6 +694,9 @@ def main():
         t_in = timed(lambda: block_proj(u, w_in, pad_rows=True))   # as the block calls it: rows of whole 128-byte lines
         t_in_dense = timed(lambda: block_proj(u, w_in))
         t_out = timed(lambda: block_proj(yn, w_out))
+        from trading_bot_0_amd import block_post_proj
+        t_post_out = timed(lambda: block_post_proj(ys_, zx, blk.norm_w, w_out, blk.H, blk.P, blk.N, blk.G))
+        post_out_bytes = e * rows * (2 * blk.d_inner + blk.d_model)               # reads y and z, writes out
         t_in_blas = timed(lambda: torch.matmul(u, w_in.t()))
         t_out_blas = timed(lambda: torch.matmul(yn, w_out.t()))
         out["mamba2_block"] = {"d_model": blk.d_model, "ms": round(t_block, 4),
@@ -702,7 +705,9 @@ def main():
                                "pre_ms": round(t_pre, 4), "pre_GBps": round(pre_bytes / t_pre / 1e6, 1),
                                "post_ms": round(t_post, 4), "post_GBps": round(post_bytes / t_post / 1e6, 1),
                                "out_proj_ms": round(t_out, 4), "out_proj_GBps": round(out_bytes / t_out / 1e6, 1),
-                               "out_proj_blas_ms": round(t_out_blas, 4)}
+                               "out_proj_blas_ms": round(t_out_blas, 4),
+                               "post_out_proj_fused_ms": round(t_post_out, 4),
+                               "post_out_proj_fused_GBps": round(post_out_bytes / t_post_out / 1e6, 1)}
         if hasattr(blk, "backward") and not args.no_backward:
             # forward with what the backward needs kept, then the block's backward (stage kernels of this library,
             # the scan's backward, four GEMMs)

@@ -114,6 +114,9 @@ extern "C" {
         u: *const c_void, w: *const c_void, out: *mut c_void, hip_stream: *mut c_void) -> c_int;
     pub fn ssd_block_post_fwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
         norm_w: *const f32, eps: f32, out: *mut c_void, hip_stream: *mut c_void) -> c_int;
+    pub fn ssd_block_post_proj_fwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
+        norm_w: *const f32, eps: f32, w: *const c_void, out_features: i64, out_ld: i64, out: *mut c_void,
+        hip_stream: *mut c_void) -> c_int;
     pub fn ssd_block_bwd_workspace_bytes(dims: *const SsdBlockDims, dtype: c_int, out_bytes: *mut usize) -> c_int;
     pub fn ssd_block_post_bwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
         norm_w: *const f32, eps: f32, dout: *const c_void, dy: *mut c_void, dzxbcdt: *mut c_void, dnorm_w: *mut f32,

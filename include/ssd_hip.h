@@ -277,6 +277,16 @@ int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, 
 int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,
                        const float *norm_w, float eps, void *out, void *hip_stream);
 
+/* ssd_block_post_fwd and the out-projection behind it as one kernel: out [B*L, out_features] (row stride out_ld
+ * elements, 0 = out_features) = rmsnorm(y * silu(z)) * norm_w . w [out_features, H*P]^T, so that the normalised rows
+ * never reach memory (the reference's counterpart is the output linear layer of its temporal mixer,
+ * trading_bots/src/torch/model/blocks/gqa.rs:82-109).  bfloat16 only (dtype 1: y, zxbcdt, w and out bf16, float32
+ * accumulation), H*P 128 or 256, out_features a multiple of 8 up to 256; SSD_ERR_UNSUPPORTED otherwise (run the two
+ * stages).  Rounding differs from the two stages' by where it happens: the gated row and the weights times norm_w
+ * are rounded to bf16 once each, the row's rsqrt factor is applied to the float32 sums. */
+int ssd_block_post_proj_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                            float eps, const void *w, int64_t out_features, int64_t out_ld, void *out, void *hip_stream);
+
 /* ---- Backward pass of the block's two stages -------------------------------------------------------------------
  * With ssd_chunk_scan_bwd between them and two GEMMs per projection (the caller's BLAS), these make the block
  * trainable: the reference's historical benchmark case for it is mamba2_fwd_bwd_train

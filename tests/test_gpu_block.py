@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import mamba2_block_oracle as blk
-from trading_bot_0_amd import Mamba2Block, SsdError, block_post, block_pre, block_proj
+from trading_bot_0_amd import Mamba2Block, SsdError, block_post, block_post_proj, block_pre, block_proj
 
 from _util import np64, rel_err
 
@@ -126,6 +126,41 @@ def test_stages_take_padded_rows(shape, dtype):
         block_pre(buf[:, :, 1:E + 1], p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G)
     with pytest.raises(ValueError):       # elements of a row not adjacent
         block_pre(buf[:, :, :2 * E:2], p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G)
+
+
+@pytest.mark.parametrize("shape", [(2, 50, 8, 32, 64, 1, 256), (3, 700, 8, 32, 64, 1, 256), (1, 2049, 8, 16, 16, 1, 128),
+                                   (5, 33, 16, 16, 16, 2, 72), (1, 1, 8, 32, 64, 1, 8), (2, 4100, 8, 32, 128, 1, 200)])
+@pytest.mark.parametrize("padded", [False, True])
+def test_post_scan_with_out_projection_in_one_kernel(shape, padded):
+    """rmsnorm(y silu(z)) norm_w . w^T as one kernel against the float64 value of the same bf16 inputs.  The kernel
+    rounds the gated row and the weights times norm_w to bf16 once each and the sum once more on the way out, so
+    every element lies within 2^-8 of the sum of its terms' magnitudes plus one bf16 rounding of itself -- a bound
+    on rounding alone; a misplaced row, channel or factor is off by the terms' 2-norm, an order of magnitude more.
+    Ragged row counts (rows past the last tile), column counts off the chunks of 32, rows of whole lines."""
+    Bsz, L, H, P, N, G, dm = shape
+    p = params(H, P, N, G, 4)
+    DI, E = H * P, 2 * H * P + 2 * G * N + H
+    g = torch.Generator().manual_seed(L + dm)
+    z = torch.randn(Bsz, L, E, generator=g).to(torch.bfloat16).cuda()
+    if padded:
+        buf = torch.full((Bsz, L, (E + 63) // 64 * 64), float("nan"), dtype=torch.bfloat16, device="cuda")
+        buf[..., :E] = z
+        z = buf[..., :E]
+    y = (torch.randn(Bsz, L, H, P, generator=g) * 3).to(torch.bfloat16).cuda()
+    w = (torch.randn(dm, DI, generator=g) / DI ** 0.5).to(torch.bfloat16).cuda()
+    out = block_post_proj(y, z, p["norm_w"], w, H, P, N, G)
+    torch.cuda.synchronize()
+    assert out.shape == (Bsz, L, dm) and out.dtype == torch.bfloat16
+    yn = blk.block_post(np64(y), np64(z), np64(p["norm_w"]), 1e-5).reshape(Bsz * L, DI)
+    w64 = np64(w)
+    ref = yn @ w64.T
+    mag = np.abs(yn) @ np.abs(w64).T
+    o = np64(out).reshape(Bsz * L, dm)
+    over = np.abs(o - ref) - (1.05 * 2.0 ** -8 * mag + 2.0 ** -8 * np.abs(ref) + 1e-30)
+    assert np.isfinite(o).all() and over.max() <= 0, f"over the rounding bound by {over.max():.3e}"
+    # and next to the two stages run one after the other (their bf16 roundings fall elsewhere, within the same bound)
+    two = np64(block_proj(block_post(y, z, p["norm_w"], H, P, N, G), w)).reshape(Bsz * L, dm)
+    assert (np.abs(o - two) <= 2 * (1.05 * 2.0 ** -8 * mag + 2.0 ** -8 * np.abs(ref)) + 1e-30).all()
 
 
 @pytest.mark.parametrize("rows,k,n", [(300, 256, 648), (4099, 256, 256), (2049, 128, 168), (33, 256, 8), (5000, 256, 768)])

@@ -200,11 +200,16 @@ def test_block_backward_with_short_filters_at_training_size(d_conv):
         o = got[key].detach().float().cpu().numpy().astype(np.float64)
         r = ref[key]
         assert o.shape == r.shape, key
-        # the small block test's bar (1.5e-1 rms for the chain's eight or so bf16 roundings) plus, for du -- four
-        # million elements stored in bf16, the largest of them ten rms out -- a share of the element itself
+        # The chain rounds to bf16 about eight times forward and back; the small block test's bar (1.5e-1 rms on the
+        # worst of a few thousand elements) is a tail bound, and du here has four million elements: its worst element
+        # lies further out in the same error distribution.  So: the error's own rms within 5e-2 of the reference's,
+        # and its worst element within six times that (plus a share of the element for du, which is stored in bf16).
         rms = max(np.sqrt(np.mean(r * r)), 1e-30)
-        over = np.abs(o - r) - (1.5e-1 * rms + (2.0 ** -6 * np.abs(r) if key == "du" else 0.0))
-        assert np.isfinite(o).all() and over.max() <= 0, f"{key}: over the bar by {over.max() / rms:.3e} rms"
+        err = np.abs(o - r)
+        assert np.isfinite(o).all(), key
+        assert np.sqrt(np.mean(err * err)) <= 5e-2 * rms, f"{key}: rms error {np.sqrt(np.mean(err * err)) / rms:.3e} rms"
+        over = err - (3e-1 * rms + (2.0 ** -6 * np.abs(r) if key == "du" else 0.0))
+        assert over.max() <= 0, f"{key}: over the bar by {over.max() / rms:.3e} rms"
         assert np.corrcoef(o.ravel(), r.ravel())[0, 1] > 0.999, key
 
 

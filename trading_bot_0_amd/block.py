@@ -35,6 +35,8 @@ def _lib():
         lib.ssd_block_pre_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_block_post_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, P]
         lib.ssd_block_proj_fwd.argtypes = [c_int64, c_int64, c_int64, c_int64, c_int, P, P, P, P]
+        lib.ssd_block_post_proj_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, c_int64, c_int64, P, P]
+        lib.ssd_block_post_proj_fwd.restype = c_int
         lib.ssd_block_pre_reset_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_block_pre_reset_fwd.restype = c_int
         lib.ssd_block_bwd_workspace_bytes.argtypes = [POINTER(SsdBlockDims), c_int, POINTER(c_size_t)]
@@ -154,6 +156,35 @@ def block_post(y, zxbcdt, norm_w, nheads, headdim, dstate, ngroups, eps=1e-5):
     dims = SsdBlockDims(Bsz, L, H, P, N, G, 4, ld)
     ssd._check(lib, lib.ssd_block_post_fwd(byref(dims), code, y.data_ptr(), zxbcdt.data_ptr(), norm_w.data_ptr(),
                                            c_float(eps), out.data_ptr(), ssd._stream_ptr(zxbcdt)))
+    return out
+
+
+def block_post_proj_supported(y: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `block_post_proj` takes these tensors (else `block_post`, then the projection)."""
+    return (y.is_cuda and y.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.dim() == 2
+            and weight.shape[1] in (128, 256) and weight.shape[0] % 8 == 0 and weight.shape[0] <= 256)
+
+
+def block_post_proj(y, zxbcdt, norm_w, weight, nheads, headdim, dstate, ngroups, eps=1e-5):
+    """out [B,L,out_features] = (rmsnorm(y * silu(z)) * norm_w) . weight^T as one kernel (bf16; weight
+    [out_features, H*P]): `block_post` and the out-projection without the normalised rows going to memory between."""
+    lib = _lib()
+    Bsz, L, E = zxbcdt.shape
+    H, P, N, G = nheads, headdim, dstate, ngroups
+    if not zxbcdt.is_cuda or E != in_proj_width(H, P, N, G):
+        raise ValueError(f"zxbcdt must be a GPU tensor with {in_proj_width(H, P, N, G)} channels, got {tuple(zxbcdt.shape)}")
+    if zxbcdt.dtype != torch.bfloat16 or y.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError("block_post_proj takes bfloat16 tensors")
+    ld = _row_stride(zxbcdt)
+    ssd._require(y, "y", (Bsz, L, H, P), torch.bfloat16)
+    ssd._require(norm_w, "norm_w", (H * P,), torch.float32)
+    if weight.dim() != 2 or weight.shape[1] != H * P or not weight.is_contiguous():
+        raise ValueError(f"weight must be contiguous [out_features, {H * P}], got {tuple(weight.shape)}")
+    out = torch.empty((Bsz, L, weight.shape[0]), dtype=torch.bfloat16, device=zxbcdt.device)
+    dims = SsdBlockDims(Bsz, L, H, P, N, G, 4, ld)
+    ssd._check(lib, lib.ssd_block_post_proj_fwd(byref(dims), ssd.SSD_DTYPE_BF16, y.data_ptr(), zxbcdt.data_ptr(),
+                                                norm_w.data_ptr(), c_float(eps), weight.data_ptr(), weight.shape[0], 0,
+                                                out.data_ptr(), ssd._stream_ptr(zxbcdt)))
     return out
 
 
@@ -347,8 +378,13 @@ class Mamba2Block:
                                             self.G, conv_state=state.conv, return_conv_state=True)
             state.conv = conv
             y = state.ssm.init_from_prefix(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk)
+        w_out = self._weights(u.dtype)[1]
+        if not save_for_backward and block_post_proj_supported(y, w_out) and y.numel() // self.d_inner >= 8192:
+            # gate, norm and out-projection as one kernel: the normalised rows never reach memory (the backward pass
+            # needs them, so a forward that keeps its tensors for it runs the two stages)
+            return block_post_proj(y, zxbcdt, self.norm_w, w_out, self.H, self.P, self.N, self.G, self.eps)
         yn = block_post(y, zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
-        out = self._project(yn, self._weights(u.dtype)[1])
+        out = self._project(yn, w_out)
         if save_for_backward:
             if state is not None:
                 raise ValueError("backward through a window that continues a carried state is not supported")

@@ -951,4 +951,31 @@ int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, con
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block post-scan launch");
 }
 
+int ssd_block_post_proj_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                            float eps, const void *w, int64_t out_features, int64_t out_ld, void *out, void *hip_stream) {
+    ssd::BlockShape s;
+    if (int rc = make_block_shape(dims, dtype, &s)) return rc;
+    if (dtype != SSD_DTYPE_BF16)
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: the fused post-scan + out-projection takes dtype 1 (bfloat16), got %d", dtype);
+    if (out_features <= 0 || out_features > 0x7fffffff)
+        return fail(SSD_ERR_INVALID, "ssd: out_features must be positive, got %lld", (long long)out_features);
+    if (!ssd::block_post_proj_supported(s, (int)out_features))
+        return fail(SSD_ERR_UNSUPPORTED,
+                    "ssd: the fused post-scan + out-projection needs nheads*headdim 128 or 256 and out_features a multiple "
+                    "of 8 up to 256, got %d and %lld", s.H * s.P, (long long)out_features);
+    if (out_ld == 0) out_ld = out_features;
+    if (out_ld < out_features || out_ld > 0x7ffff || out_ld % 8 != 0)
+        return fail(SSD_ERR_INVALID, "ssd: out_ld must be 0 or at least out_features (%lld), a multiple of 8 and below 524288, got %lld",
+                    (long long)out_features, (long long)out_ld);
+    REQUIRE_PTR(y);
+    REQUIRE_PTR(zxbcdt);
+    REQUIRE_PTR(norm_w);
+    REQUIRE_PTR(w);
+    REQUIRE_PTR(out);
+    if (!(eps > 0.f)) return fail(SSD_ERR_INVALID, "ssd: eps must be positive");
+    hipError_t e = ssd::launch_block_post_proj(s, y, zxbcdt, norm_w, eps, w, (int)out_features, (int)out_ld, out,
+                                               (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "block post-scan + out-projection launch");
+}
+
 }  // extern "C"

@@ -13,6 +13,7 @@
 // system's rate).
 #include <algorithm>
 
+#include "ssd_block_common.h"
 #include "ssd_device.h"
 
 namespace ssd {
@@ -145,6 +146,152 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------------------------
+// Gate + RMSNorm + out-projection in one pass: out[m, n] = sum_k yn[m, k] w[n, k] with
+// yn[m, k] = v[m, k] rsqrt(mean_k v[m, k]^2 + eps) norm_w[k], v = y silu(z) -- the normalised row never reaches
+// memory (it would be written by one kernel and read back by the next: two thirds of the bytes of a row's y and z).
+// A row of the inner width K (128 or 256 channels) is exactly the MFMA's K axis, which a lane pair (r, r + 32) holds
+// entirely in its operand fragments: the prologue turns a tile's rows of y and z into fragments of bf16(v) and the
+// pair's sum of squares; the norm's weights are folded into the staged matrix (w[n, k] norm_w[k], rounded to bf16)
+// and the row's rsqrt factor scales the accumulators, whose lanes hold one row each.  One workgroup takes all
+// out_features (at most 256) columns, so that the prologue runs once per row: its rows of w fill 132 KB of LDS, and a
+// wave's output tile covers 16 rows at a time to fit beside them.
+// ------------------------------------------------------------------------------------------------------------------
+constexpr int kPostProjMaxCols = 256;
+
+template <int KS, int CH>  // K = 16 * KS inner channels, CH chunks of 32 output columns
+__global__ __launch_bounds__(64 * kProjWaves) void block_post_proj_kernel(
+    const __bf16 *__restrict__ y, const __bf16 *__restrict__ zxbcdt, const float *__restrict__ norm_w, float eps,
+    const __bf16 *__restrict__ w, __bf16 *__restrict__ out, long long M, int N, int ld_z, int ldo, int tiles) {
+    constexpr int K = 16 * KS, NTHR = 64 * kProjWaves, PPR = K / 8;  // 16-byte pieces per row of w
+    constexpr int ROWB = K * 2 + 16;  // a staged row of w: 16 bytes of padding shift the banks from row to row
+    constexpr int kTileRowB = 64 * 2 + 16;
+    __shared__ __attribute__((aligned(16))) unsigned char wsm[CH * kProjChunk * ROWB];
+    __shared__ __attribute__((aligned(16))) unsigned char otile[kProjWaves][16 * kTileRowB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const long long row0 = (long long)blockIdx.x * tiles * (32LL * kProjWaves);  // tiles: 32-row tiles per wave, 1 .. kProjTiles
+    const int r = lane & 31, half = lane >> 5;
+    // this lane's K elements are 16 ks + 8 half .. + 7 for every K step
+    auto tile_row0 = [&](int t) { return row0 + (long long)t * (32 * kProjWaves) + wave * 32; };
+    // A tile's rows of y are requested one tile ahead (they are in flight during the products and stores of the tile
+    // before); its rows of z only at the top of the tile: both sets a tile ahead would not fit the registers beside
+    // the operand fragments, and the workgroup's other waves fill the SIMD during the wait.
+    uint4 yq[KS], zq[KS];
+    auto tile_row = [&](int t) { return min(tile_row0(t) + r, M - 1); };  // rows past M repeat the last row; never stored
+    auto load_y = [&](int t) {
+        const __bf16 *yr = y + (size_t)tile_row(t) * K + 8 * half;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) yq[ks] = *reinterpret_cast<const uint4 *>(yr + 16 * ks);
+    };
+    auto load_z = [&](int t) {
+        const __bf16 *zr = zxbcdt + (size_t)tile_row(t) * ld_z + 8 * half;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) zq[ks] = *reinterpret_cast<const uint4 *>(zr + 16 * ks);
+    };
+    load_y(0);  // in flight while w is staged
+    {   // rows 0 .. 32 CH - 1 of w times norm_w, rounded to bf16 (rows past N repeat the last one: never stored)
+        constexpr int PIECES = CH * kProjChunk * PPR;
+        constexpr int FILL = (PIECES + NTHR - 1) / NTHR;
+#pragma unroll 4
+        for (int i = 0; i < FILL; ++i) {
+            const int p = min(tid + i * NTHR, PIECES - 1);
+            const int row = p / PPR, piece = p % PPR;
+            const Pack8<__bf16> q = Pack8<__bf16>::load(w + (size_t)min(row, N - 1) * K + piece * 8);
+            const float4 na = *reinterpret_cast<const float4 *>(norm_w + piece * 8);
+            const float4 nb = *reinterpret_cast<const float4 *>(norm_w + piece * 8 + 4);
+            uint4 o;
+            o.x = pack_bf16x2(q.get(0) * na.x, q.get(1) * na.y);
+            o.y = pack_bf16x2(q.get(2) * na.z, q.get(3) * na.w);
+            o.z = pack_bf16x2(q.get(4) * nb.x, q.get(5) * nb.y);
+            o.w = pack_bf16x2(q.get(6) * nb.z, q.get(7) * nb.w);
+            *reinterpret_cast<uint4 *>(wsm + row * ROWB + piece * 16) = o;
+        }
+    }
+    __syncthreads();
+    if (row0 >= M) return;
+    unsigned char *tile = otile[wave];
+    const __amdgpu_buffer_rsrc_t obuf = make_buffer(out + (size_t)row0 * ldo, (unsigned)min((long long)tiles * 32 * kProjWaves, M - row0) * (unsigned)ldo * 2u);
+    const float inv_k = 1.f / (float)K;
+#pragma unroll 1
+    for (int t = 0; t < tiles; ++t) {
+        // ---- prologue: this tile's rows of y and z -> fragments of bf16(y silu(z)) and the rows' rsqrt factor ----
+        load_z(t);
+        Frag<__bf16> uf[KS];
+        float ss = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const Pack8<__bf16> yy{yq[ks]}, zz{zq[ks]};
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                v[i] = yy.get(i) * silu(zz.get(i));
+                ss += v[i] * v[i];
+            }
+            uint4 o;
+            o.x = pack_bf16x2(v[0], v[1]);
+            o.y = pack_bf16x2(v[2], v[3]);
+            o.z = pack_bf16x2(v[4], v[5]);
+            o.w = pack_bf16x2(v[6], v[7]);
+            uf[ks].v = __builtin_bit_cast(bf16x8, o);
+        }
+        ss += __shfl_xor(ss, 32, 64);
+        const float rstd = rsqrtf(ss * inv_k + eps);
+        // the next tile's rows of y: requested before this tile's products and stores (loads and stores complete in
+        // order per wave: requested behind the stores they would wait for those to reach memory)
+        if (t + 1 < tiles) load_y(t + 1);
+        const unsigned trow = (unsigned)(t * (32 * kProjWaves) + wave * 32);
+        const long long m0 = tile_row0(t);
+#pragma unroll
+        for (int c0 = 0; c0 < CH; c0 += 2) {
+            f32x16 acc[2];
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                const int c = c0 + sub;
+                acc[sub] = f32x16{0};
+                if (c >= CH) break;
+                const unsigned char *wb = wsm + (c * kProjChunk + r) * ROWB + half * 16;
+                f32x16 acc_odd = {0};
+#pragma unroll
+                for (int ks = 0; ks < KS; ks += 2) {
+                    Frag<__bf16> wf0, wf1;
+                    wf0.v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(wb + ks * 32));
+                    wf1.v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(wb + ks * 32 + 32));
+                    acc[sub] = mma32(wf0, uf[ks], acc[sub]);
+                    acc_odd = mma32(wf1, uf[ks + 1], acc_odd);
+                }
+                acc[sub] = (acc[sub] + acc_odd) * rstd;
+            }
+            // acc[sub][4 vg + i] = out[m0 + r, 32 (c0 + sub) + 8 vg + 4 half + i]; the wave's tile holds 16 rows, so
+            // the rows go out in two halves (rows r < 16, then the others)
+#pragma unroll
+            for (int rh = 0; rh < 2; ++rh) {
+                if ((r >> 4) == rh) {
+#pragma unroll
+                    for (int sub = 0; sub < 2; ++sub) {
+#pragma unroll
+                        for (int vg = 0; vg < 4; ++vg)
+                            *reinterpret_cast<uint2 *>(tile + (r & 15) * kTileRowB + (sub * 32 + 8 * vg + 4 * half) * 2) = make_uint2(
+                                pack_bf16x2(acc[sub][4 * vg], acc[sub][4 * vg + 1]), pack_bf16x2(acc[sub][4 * vg + 2], acc[sub][4 * vg + 3]));
+                    }
+                }
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int pass = 0; pass < 2; ++pass) {
+                    const int trw = pass * 8 + (lane >> 3), row = rh * 16 + trw, col = c0 * kProjChunk + (lane & 7) * 8;
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + trw * kTileRowB + (lane & 7) * 16);
+                    const bool ok = m0 + row < M && col < N;
+                    const unsigned off = ((trow + (unsigned)row) * (unsigned)ldo + (unsigned)col) * 2u;
+                    __builtin_amdgcn_raw_buffer_store_b128(v, obuf, ok ? off : kBufferDropOffset, 0, 0);
+                }
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    }
+}
+
 }  // namespace
 
 bool block_proj_supported(long long rows, int in_features, int out_features) {
@@ -192,6 +339,46 @@ hipError_t launch_block_proj(long long rows, int in_features, int out_features, 
     SSD_PROJ_CASE(8, 1) SSD_PROJ_CASE(8, 2) SSD_PROJ_CASE(8, 3) SSD_PROJ_CASE(8, 4) SSD_PROJ_CASE(8, 5)
     SSD_PROJ_CASE(16, 1) SSD_PROJ_CASE(16, 2) SSD_PROJ_CASE(16, 3) SSD_PROJ_CASE(16, 4) SSD_PROJ_CASE(16, 5)
 #undef SSD_PROJ_CASE
+    return hipErrorInvalidValue;
+}
+
+bool block_post_proj_supported(const BlockShape &s, int out_features) {
+    const int DI = s.H * s.P;
+    return (DI == 128 || DI == 256) && out_features > 0 && out_features <= kPostProjMaxCols && out_features % 8 == 0;
+}
+
+// out [B*L, out_features] (row stride out_ld) = rmsnorm(y silu(z)) norm_w . w^T; y [B*L, H*P] bf16, z the first H*P
+// channels of zxbcdt's rows (stride s.ld), w [out_features, H*P] bf16.
+hipError_t launch_block_post_proj(const BlockShape &s, const void *y, const void *zxbcdt, const float *norm_w, float eps,
+                                  const void *w, int out_features, int out_ld, void *out, hipStream_t st) {
+    if (!block_post_proj_supported(s, out_features) || out_ld < out_features || out_ld % 8 != 0) return hipErrorInvalidValue;
+    const int K = s.H * s.P;
+    const long long rows = (long long)s.B * s.L;
+    // rows per workgroup: up to kProjTiles tiles of 32 rows per wave, fewer when that would leave CUs without a
+    // workgroup (each workgroup stages all of w, as much as 256 of its rows, so more than one tile where rows allow)
+    int dev = 0, cus = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = device_cu_count(dev, &cus);
+    if (e != hipSuccess) return e;
+    const long long per_tile = 32LL * kProjWaves;
+    const int tiles = (int)std::max<long long>(1, std::min<long long>(kProjTiles, rows / (per_tile * cus)));
+    const long long rows_per_group = per_tile * tiles;
+    const long long groups = (rows + rows_per_group - 1) / rows_per_group;
+    if (groups > 0x7fffffffLL || (unsigned long long)rows_per_group * out_ld * 2 > 0x7fffffffULL) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)groups), block(64 * kProjWaves);
+    const __bf16 *yy = static_cast<const __bf16 *>(y), *zz = static_cast<const __bf16 *>(zxbcdt), *ww = static_cast<const __bf16 *>(w);
+    __bf16 *oo = static_cast<__bf16 *>(out);
+    const int ch = (out_features + kProjChunk - 1) / kProjChunk;
+#define SSD_POST_PROJ_CASE(KSv, CHv)                                                                                   \
+    if (K == 16 * KSv && ch == CHv) {                                                                                  \
+        block_post_proj_kernel<KSv, CHv><<<grid, block, 0, st>>>(yy, zz, norm_w, eps, ww, oo, rows, out_features, s.ld, out_ld, tiles); \
+        return hipGetLastError();                                                                                      \
+    }
+    SSD_POST_PROJ_CASE(8, 1) SSD_POST_PROJ_CASE(8, 2) SSD_POST_PROJ_CASE(8, 3) SSD_POST_PROJ_CASE(8, 4)
+    SSD_POST_PROJ_CASE(8, 5) SSD_POST_PROJ_CASE(8, 6) SSD_POST_PROJ_CASE(8, 7) SSD_POST_PROJ_CASE(8, 8)
+    SSD_POST_PROJ_CASE(16, 1) SSD_POST_PROJ_CASE(16, 2) SSD_POST_PROJ_CASE(16, 3) SSD_POST_PROJ_CASE(16, 4)
+    SSD_POST_PROJ_CASE(16, 5) SSD_POST_PROJ_CASE(16, 6) SSD_POST_PROJ_CASE(16, 7) SSD_POST_PROJ_CASE(16, 8)
+#undef SSD_POST_PROJ_CASE
     return hipErrorInvalidValue;
 }
 

@@ -52,6 +52,7 @@ EXPORTED_SYMBOLS = (
     "ssd_block_bwd_workspace_bytes",
     "ssd_block_post_bwd",
     "ssd_block_pre_bwd",
+    "ssd_block_post_proj_fwd",
 )
 
 
