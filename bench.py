@@ -634,14 +634,19 @@ def main():
                 t_prefill = event_time_steps(lambda: rblk.forward(ru, state=rst), 100, torch)[0] * 1e3
                 ru_t = ru[:, 0].contiguous()
                 spin(lambda: rblk.step(ru_t, rst), torch, 0.1)
-                t_bstep = event_time_steps(lambda: rblk.step(ru_t, rst), 100, torch)[0] * 1e3
+                t_bstep = event_time_steps(lambda: rblk.step(ru_t, rst), 200, torch)[0] * 1e3
+                spin(lambda: rblk.step(ru_t, rst, fused=False), torch, 0.1)
+                t_bstep_stages = event_time_steps(lambda: rblk.step(ru_t, rst, fused=False), 100, torch)[0] * 1e3
                 gstep = rblk.graphed_step(rst)
                 spin(lambda: gstep(ru_t), torch, 0.1)
                 t_gstep = event_time_steps(lambda: gstep(ru_t), 200, torch)[0] * 1e3
             suite += [{"name": "mamba2_forward_train", "time_ms": t_train, "config": {**cfg, **bsizes}},
                       {"name": "mamba2_infer_prefill", "time_ms": t_prefill, "config": {**cfg, **bsizes}},
                       {"name": "mamba2_infer_step", "time_ms": t_bstep,
-                       "config": {"batch": 4, "seq_len": 1, "dtype": "BFloat16", **bsizes}},
+                       "config": {"batch": 4, "seq_len": 1, "dtype": "BFloat16", "launches": "one (ssd_block_step_fwd)", **bsizes}},
+                      {"name": "mamba2_infer_step_stage_kernels", "time_ms": t_bstep_stages,
+                       "config": {"batch": 4, "seq_len": 1, "dtype": "BFloat16",
+                                  "launches": "five stage kernels, two library products", **bsizes}},
                       {"name": "mamba2_infer_step_graph", "time_ms": t_gstep,
                        "config": {"batch": 4, "seq_len": 1, "dtype": "BFloat16", "captured": "one HIP graph per step", **bsizes}}]
             if hasattr(rblk, "backward") and not args.no_backward:

@@ -117,6 +117,10 @@ extern "C" {
     pub fn ssd_block_post_proj_fwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
         norm_w: *const f32, eps: f32, w: *const c_void, out_features: i64, out_ld: i64, out: *mut c_void,
         hip_stream: *mut c_void) -> c_int;
+    pub fn ssd_block_step_fwd(dims: *const SsdBlockDims, dtype: c_int, d_model: i64, u: *const c_void, w_in: *const c_void,
+        conv_w: *const f32, conv_b: *const f32, dt_bias: *const f32, a: *const f32, d: *const f32, norm_w: *const f32,
+        eps: f32, w_out: *const c_void, conv_state: *mut c_void, ssm_state: *mut f32, out: *mut c_void,
+        hip_stream: *mut c_void) -> c_int;
     pub fn ssd_block_bwd_workspace_bytes(dims: *const SsdBlockDims, dtype: c_int, out_bytes: *mut usize) -> c_int;
     pub fn ssd_block_post_bwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
         norm_w: *const f32, eps: f32, dout: *const c_void, dy: *mut c_void, dzxbcdt: *mut c_void, dnorm_w: *mut f32,

@@ -287,6 +287,21 @@ int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, con
 int ssd_block_post_proj_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                             float eps, const void *w, int64_t out_features, int64_t out_ld, void *out, void *hip_stream);
 
+/* One timestep of the whole block for every stream as ONE launch: in-projection, conv window update + SiLU,
+ * softplus(dt), SSM state update and readout, gate + RMSNorm, out-projection (the per-bar update of
+ * trading_bots/src/torch/model/stream/live.rs:228-244, called from trading_bots/src/torch/infer/offline.rs:124-125:
+ * at a few streams the step's cost is the host's time to issue launches, so the chain of stage kernels and library
+ * products is one kernel here).  dims->seqlen must be 1.  u [B,d_model], w_in [2*H*P+2*G*N+H, d_model] and w_out
+ * [d_model, H*P] in the activation type (dtype 0: float32, 1: bfloat16), conv_w [C,d_conv], conv_b [C], dt_bias [H],
+ * A [H], D [H] or NULL, norm_w [H*P] float32; conv_state [B,d_conv-1,C] (activation type) and ssm_state [B,H,P,N]
+ * (float32) advance in place; out [B,d_model].  d_model and H*P must each be 128 or 256 and dstate a multiple of 16
+ * (SSD_ERR_UNSUPPORTED otherwise: run the stages).  A workgroup per stream reads both weight matrices whole, so the
+ * call is meant for small batches (up to a few dozen streams); large ones are faster through the stage kernels. */
+int ssd_block_step_fwd(const ssd_block_dims *dims, int dtype, int64_t d_model, const void *u, const void *w_in,
+                       const float *conv_w, const float *conv_b, const float *dt_bias, const float *A, const float *D,
+                       const float *norm_w, float eps, const void *w_out, void *conv_state, float *ssm_state, void *out,
+                       void *hip_stream);
+
 /* ---- Backward pass of the block's two stages -------------------------------------------------------------------
  * With ssd_chunk_scan_bwd between them and two GEMMs per projection (the caller's BLAS), these make the block
  * trainable: the reference's historical benchmark case for it is mamba2_fwd_bwd_train

@@ -379,6 +379,57 @@ def test_block_stages_inside_a_captured_graph():
         assert all(torch.equal(a, b) for a, b in zip(captured, eager)), f"replay {i}"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cfg", [(256, 8, 32, 64, 1, 4, 4), (128, 8, 16, 16, 2, 3, 3), (256, 16, 16, 128, 2, 2, 5),
+                                 (128, 8, 32, 32, 1, 4, 1), (256, 8, 16, 32, 1, 4, 2)])
+def test_block_step_as_one_launch(cfg, dtype):
+    """The whole step as one kernel (ssd_block_step_fwd), three steps in a row from random states, against the float64
+    oracle block run one timestep at a time from the same states, and against the stage kernels' step: outputs and
+    both states.  float32: 1e-3 of the rms (the bar of the streamed block test); bf16: the block test's 1e-1 for the
+    output (about five bf16 roundings in the chain) and for the SSM state (its increment dt x B is a product of three
+    rounded factors, and the largest elements of it are many rms of the state); next to the stage kernels, which round
+    at the same points, 1e-2."""
+    d_model, H, P, N, G, K, Bsz = cfg
+    b = Mamba2Block(d_model=d_model, nheads=H, headdim=P, dstate=N, ngroups=G, d_conv=K, seed=7)
+    p = oracle_params(b)
+    g = torch.Generator().manual_seed(31)
+    C = H * P + 2 * G * N
+    conv0 = torch.randn(Bsz, K - 1, C, generator=g).to(dtype).cuda()
+    ssm0 = torch.randn(Bsz, H, P, N, generator=g).cuda()
+    us = torch.randn(3, Bsz, d_model, generator=g).to(dtype).cuda()
+    st_f, st_s = b.new_state(Bsz, dtype=dtype), b.new_state(Bsz, dtype=dtype)
+    for st in (st_f, st_s):
+        st.conv.copy_(conv0)
+        st.ssm.state.copy_(ssm0)
+    conv_ref, ssm_ref = np64(conv0), np64(ssm0)
+    tol_out, tol_state = (1e-3, 1e-3) if dtype == torch.float32 else (1e-1, 1e-1)
+    for i in range(3):
+        out_f = b.step(us[i], st_f, fused=True)
+        out_s = b.step(us[i], st_s, fused=False)
+        torch.cuda.synchronize()
+        ref, conv_ref, ssm_ref = blk.block_forward(np64(us[i]).reshape(Bsz, 1, d_model), p, conv_state=conv_ref, ssm_state=ssm_ref)
+        assert out_f.shape == (Bsz, d_model) and out_f.dtype == dtype
+        assert rel_err(out_f, ref[:, 0]) <= tol_out, f"step {i}: output {rel_err(out_f, ref[:, 0]):.3e}"
+        assert rel_err(st_f.ssm.state, ssm_ref) <= tol_state, f"step {i}: SSM state"
+        assert rel_err(st_f.conv, conv_ref) <= (1e-5 if dtype == torch.float32 else 2.0 ** -7 * 6), f"step {i}: conv state"
+        # beside the stage kernels' step (same rounding points, other summation orders)
+        assert rel_err(out_f, np64(out_s)) <= (1e-4 if dtype == torch.float32 else 5e-2), f"step {i}: fused vs stages"
+        assert rel_err(st_f.ssm.state, np64(st_s.ssm.state)) <= (1e-5 if dtype == torch.float32 else 1e-2)
+        # the oracle continues from its own states; the conv state it returns is the raw in-projection rows, which
+        # the GPU holds rounded to the activation type: continue the oracle from the GPU's rows so that the three steps
+        # test three steps, not the drift of a rounding
+        conv_ref = np64(st_f.conv)
+
+
+def test_block_step_as_one_launch_refuses_what_it_does_not_take():
+    b = Mamba2Block(d_model=64, nheads=8, headdim=32, dstate=64, seed=1)
+    st = b.new_state(2, dtype=torch.float32)
+    with pytest.raises(SsdError):
+        b.step(torch.randn(2, 64).cuda(), st, fused=True)
+    out = b.step(torch.randn(2, 64).cuda(), st)     # the default picks the stage kernels for this width
+    assert out.shape == (2, 64)
+
+
 def test_graphed_step_equals_the_eager_step_on_every_replay():
     """The block's step captured in a graph (no memset nodes: every kernel writes what it later reads) and replayed
     with the program's own eager work between the replays; outputs and both states equal the eager step's bit for bit."""

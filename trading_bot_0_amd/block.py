@@ -37,6 +37,8 @@ def _lib():
         lib.ssd_block_proj_fwd.argtypes = [c_int64, c_int64, c_int64, c_int64, c_int, P, P, P, P]
         lib.ssd_block_post_proj_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, c_int64, c_int64, P, P]
         lib.ssd_block_post_proj_fwd.restype = c_int
+        lib.ssd_block_step_fwd.argtypes = [POINTER(SsdBlockDims), c_int, c_int64, P, P, P, P, P, P, P, P, c_float, P, P, P, P, P]
+        lib.ssd_block_step_fwd.restype = c_int
         lib.ssd_block_pre_reset_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_block_pre_reset_fwd.restype = c_int
         lib.ssd_block_bwd_workspace_bytes.argtypes = [POINTER(SsdBlockDims), c_int, POINTER(c_size_t)]
@@ -185,6 +187,53 @@ def block_post_proj(y, zxbcdt, norm_w, weight, nheads, headdim, dstate, ngroups,
     ssd._check(lib, lib.ssd_block_post_proj_fwd(byref(dims), ssd.SSD_DTYPE_BF16, y.data_ptr(), zxbcdt.data_ptr(),
                                                 norm_w.data_ptr(), c_float(eps), weight.data_ptr(), weight.shape[0], 0,
                                                 out.data_ptr(), ssd._stream_ptr(zxbcdt)))
+    return out
+
+
+# batches up to which one workgroup per stream (each reading both weight matrices whole) beats the stage kernels
+FUSED_STEP_MAX_BATCH = 64
+
+
+def block_step_supported(u_t: torch.Tensor, d_inner: int, dstate: int) -> bool:
+    """Whether `block_step` takes this step (else the stage kernels, one launch each)."""
+    return (u_t.is_cuda and u_t.dtype in (torch.bfloat16, torch.float32) and u_t.dim() == 2
+            and u_t.shape[1] in (128, 256) and d_inner in (128, 256) and dstate % 16 == 0)
+
+
+def block_step(u_t, w_in, conv_w, conv_b, dt_bias, A, D, norm_w, w_out, conv_state, ssm_state, nheads, headdim, dstate,
+               ngroups, eps=1e-5, out=None):
+    """One timestep of the whole block for every stream as one launch: u_t [B,d_model] -> out [B,d_model]; `conv_state`
+    [B,d_conv-1,C] (activation dtype) and `ssm_state` [B,H,P,N] (float32) advance in place.  w_in [E,d_model] and
+    w_out [d_model,H*P] in the activation dtype."""
+    lib = _lib()
+    Bsz, d_model = u_t.shape
+    H, P, N, G = nheads, headdim, dstate, ngroups
+    C = H * P + 2 * G * N
+    E = in_proj_width(H, P, N, G)
+    dtype = u_t.dtype
+    code = ssd._dtype_code(u_t)
+    d_conv = conv_w.shape[1]
+    ssd._require(u_t, "u_t", (Bsz, d_model), dtype)
+    ssd._require(w_in, "w_in", (E, d_model), dtype)
+    ssd._require(w_out, "w_out", (d_model, H * P), dtype)
+    ssd._require(conv_w, "conv_w", (C, d_conv), torch.float32)
+    ssd._require(conv_b, "conv_b", (C,), torch.float32)
+    ssd._require(dt_bias, "dt_bias", (H,), torch.float32)
+    ssd._require(A, "A", (H,), torch.float32)
+    if D is not None:
+        ssd._require(D, "D", (H,), torch.float32)
+    ssd._require(norm_w, "norm_w", (H * P,), torch.float32)
+    ssd._require(conv_state, "conv_state", (Bsz, d_conv - 1, C), dtype)
+    ssd._require(ssm_state, "ssm_state", (Bsz, H, P, N), torch.float32)
+    if out is None:
+        out = torch.empty((Bsz, d_model), dtype=dtype, device=u_t.device)
+    else:
+        ssd._require(out, "out", (Bsz, d_model), dtype)
+    dims = SsdBlockDims(Bsz, 1, H, P, N, G, d_conv, 0)
+    ssd._check(lib, lib.ssd_block_step_fwd(byref(dims), code, d_model, u_t.data_ptr(), w_in.data_ptr(), conv_w.data_ptr(),
+                                           conv_b.data_ptr(), dt_bias.data_ptr(), A.data_ptr(), ssd._ptr(D),
+                                           norm_w.data_ptr(), c_float(eps), w_out.data_ptr(), conv_state.data_ptr(),
+                                           ssm_state.data_ptr(), out.data_ptr(), ssd._stream_ptr(u_t)))
     return out
 
 
@@ -440,11 +489,27 @@ class Mamba2Block:
             self._weights_cache = cached
         return cached[1], cached[2]
 
-    def step(self, u_t: torch.Tensor, state: Mamba2StreamState) -> torch.Tensor:
-        """One timestep for every stream: u_t [B,d_model] -> [B,d_model]; advances `state` in place."""
+    def _A_cached(self) -> torch.Tensor:
+        """-exp(A_log), computed once per version of A_log (a launch of its own otherwise, per step)."""
+        key = (self.A_log._version, self.A_log.data_ptr())
+        cached = getattr(self, "_A_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, -torch.exp(self.A_log))
+            self._A_cache = cached
+        return cached[1]
+
+    def step(self, u_t: torch.Tensor, state: Mamba2StreamState, fused: Optional[bool] = None) -> torch.Tensor:
+        """One timestep for every stream: u_t [B,d_model] -> [B,d_model]; advances `state` in place.  `fused`: run the
+        step as one launch (default: for batches up to FUSED_STEP_MAX_BATCH of shapes the fused kernel takes) or as the
+        stage kernels with the projections on the BLAS behind torch."""
         if u_t.dim() != 2 or u_t.shape[1] != self.d_model:
             raise ValueError(f"block step input must be [batch, {self.d_model}], got {tuple(u_t.shape)}")
         w_in, w_out = self._weights(u_t.dtype)
+        if fused is None:
+            fused = u_t.shape[0] <= FUSED_STEP_MAX_BATCH and block_step_supported(u_t, self.d_inner, self.N)
+        if fused:   # the whole step as one launch: what a step costs at a few streams is issuing its launches
+            return block_step(u_t.contiguous(), w_in, self.conv_w, self.conv_b, self.dt_bias, self._A_cached(), self.D,
+                              self.norm_w, w_out, state.conv, state.ssm.state, self.H, self.P, self.N, self.G, self.eps)
         zxbcdt = torch.matmul(u_t, w_in.t()).unsqueeze(1).contiguous()
         x, Bm, Cm, dt, _ = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N,
                                      self.G, conv_state=state.conv, conv_state_out=state.conv)  # in place

@@ -978,4 +978,35 @@ int ssd_block_post_proj_fwd(const ssd_block_dims *dims, int dtype, const void *y
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block post-scan + out-projection launch");
 }
 
+int ssd_block_step_fwd(const ssd_block_dims *dims, int dtype, int64_t d_model, const void *u, const void *w_in,
+                       const float *conv_w, const float *conv_b, const float *dt_bias, const float *A, const float *D,
+                       const float *norm_w, float eps, const void *w_out, void *conv_state, float *ssm_state, void *out,
+                       void *hip_stream) {
+    ssd::BlockShape s;
+    if (int rc = make_block_shape(dims, dtype, &s)) return rc;
+    if (dtype != SSD_DTYPE_F32 && dtype != SSD_DTYPE_BF16)
+        return fail(SSD_ERR_UNSUPPORTED, "ssd: the fused block step takes dtype 0 (float32) or 1 (bfloat16), got %d", dtype);
+    if (s.L != 1) return fail(SSD_ERR_INVALID, "ssd: the fused block step advances one timestep, got seqlen %d", s.L);
+    if (d_model <= 0 || d_model > 0x7fffffff || !ssd::block_step_supported(s, (int)d_model))
+        return fail(SSD_ERR_UNSUPPORTED,
+                    "ssd: the fused block step needs d_model and nheads*headdim of 128 or 256 and dstate a multiple of 16, "
+                    "got d_model %lld, nheads*headdim %d, dstate %d", (long long)d_model, s.H * s.P, s.N);
+    REQUIRE_PTR(u);
+    REQUIRE_PTR(w_in);
+    REQUIRE_PTR(conv_w);
+    REQUIRE_PTR(conv_b);
+    REQUIRE_PTR(dt_bias);
+    REQUIRE_PTR(A);
+    REQUIRE_PTR(norm_w);
+    REQUIRE_PTR(w_out);
+    REQUIRE_PTR(conv_state);
+    REQUIRE_PTR(ssm_state);
+    REQUIRE_PTR(out);
+    OPTIONAL_PTR(D);
+    if (!(eps > 0.f)) return fail(SSD_ERR_INVALID, "ssd: eps must be positive");
+    hipError_t e = ssd::launch_block_step(s, dtype == SSD_DTYPE_F32 ? 0 : 1, (int)d_model, u, w_in, conv_w, conv_b, dt_bias,
+                                          A, D, norm_w, eps, w_out, conv_state, ssm_state, out, (hipStream_t)hip_stream);
+    return e == hipSuccess ? SSD_OK : hip_fail(e, "fused block step launch");
+}
+
 }  // extern "C"

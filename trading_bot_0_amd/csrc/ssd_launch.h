@@ -129,6 +129,10 @@ hipError_t launch_block_proj(long long rows, int in_features, int out_features, 
 hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w,
                             const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
                             const unsigned char *reset, void *x, void *Bm, void *Cm, void *dt, hipStream_t stream);
+bool block_step_supported(const BlockShape &s, int d_model);
+hipError_t launch_block_step(const BlockShape &s, int dtype, int d_model, const void *u, const void *w_in, const float *conv_w,
+                             const float *conv_b, const float *dt_bias, const float *A, const float *D, const float *norm_w,
+                             float eps, const void *w_out, void *conv_state, float *ssm_state, void *out, hipStream_t st);
 bool block_post_proj_supported(const BlockShape &s, int out_features);
 hipError_t launch_block_post_proj(const BlockShape &s, const void *y, const void *zxbcdt, const float *norm_w, float eps,
                                   const void *w, int out_features, int out_ld, void *out, hipStream_t st);

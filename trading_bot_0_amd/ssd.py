@@ -53,6 +53,7 @@ EXPORTED_SYMBOLS = (
     "ssd_block_post_bwd",
     "ssd_block_pre_bwd",
     "ssd_block_post_proj_fwd",
+    "ssd_block_step_fwd",
 )
 
 
