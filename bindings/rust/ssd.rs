@@ -117,10 +117,6 @@ extern "C" {
     pub fn ssd_block_post_proj_fwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
         norm_w: *const f32, eps: f32, w: *const c_void, out_features: i64, out_ld: i64, out: *mut c_void,
         hip_stream: *mut c_void) -> c_int;
-    pub fn ssd_block_in_proj_pre_fwd(dims: *const SsdBlockDims, dtype: c_int, d_model: i64, u: *const c_void,
-        w_in: *const c_void, conv_w: *const f32, conv_b: *const f32, dt_bias: *const f32, conv_state_in: *const c_void,
-        conv_state_out: *mut c_void, write_raw: c_int, zxbcdt: *mut c_void, x: *mut c_void, bm: *mut c_void,
-        cm: *mut c_void, dt: *mut c_void, hip_stream: *mut c_void) -> c_int;
     pub fn ssd_block_step_fwd(dims: *const SsdBlockDims, dtype: c_int, d_model: i64, u: *const c_void, w_in: *const c_void,
         conv_w: *const f32, conv_b: *const f32, dt_bias: *const f32, a: *const f32, d: *const f32, norm_w: *const f32,
         eps: f32, w_out: *const c_void, conv_state: *mut c_void, ssm_state: *mut f32, out: *mut c_void,

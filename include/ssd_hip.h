@@ -277,20 +277,6 @@ int ssd_block_proj_fwd(int64_t rows, int64_t in_features, int64_t out_features, 
 int ssd_block_post_fwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt,
                        const float *norm_w, float eps, void *out, void *hip_stream);
 
-/* The in-projection with ssd_block_pre_fwd in its epilogue, as one kernel: zxbcdt [B*L, zxbcdt_ld] = u [B*L, d_model] .
- * w_in [2*H*P+2*G*N+H, d_model]^T, and from its x | B | C | dt channels, before they leave the chip, x [B,L,H,P], Bm, Cm
- * [B,L,G,N] = silu(conv + bias) and dt [B,L,H] = softplus(dt_raw + dt_bias) (the reference's counterparts are the input
- * linear layer and the causal depthwise mix of its temporal mixer, trading_bots/src/torch/model/blocks/gqa.rs:82-109,
- * 172-178).  zxbcdt receives its z channels; its raw x | B | C | dt channels only when write_raw != 0 (the backward
- * pass reads them), else they are left unwritten.  Results equal ssd_block_proj_fwd followed by ssd_block_pre_fwd bit
- * for bit.  bfloat16 only (dtype 1), d_model 128 or 256, seqlen a multiple of 256, nheads a multiple of 8, nheads*headdim
- * and ngroups*dstate multiples of 64, more than 160 channels per row, no restarts inside the window; SSD_ERR_UNSUPPORTED otherwise (run the two stages).
- * conv_state_in / conv_state_out [B, d_conv-1, C] or NULL, as in ssd_block_pre_fwd. */
-int ssd_block_in_proj_pre_fwd(const ssd_block_dims *dims, int dtype, int64_t d_model, const void *u, const void *w_in,
-                              const float *conv_w, const float *conv_b, const float *dt_bias, const void *conv_state_in,
-                              void *conv_state_out, int write_raw, void *zxbcdt, void *x, void *Bm, void *Cm, void *dt,
-                              void *hip_stream);
-
 /* ssd_block_post_fwd and the out-projection behind it as one kernel: out [B*L, out_features] (row stride out_ld
  * elements, 0 = out_features) = rmsnorm(y * silu(z)) * norm_w . w [out_features, H*P]^T, so that the normalised rows
  * never reach memory (the reference's counterpart is the output linear layer of its temporal mixer,

@@ -6,8 +6,7 @@ import pytest
 import torch
 
 from oracle import mamba2_block_oracle as blk
-from trading_bot_0_amd import (Mamba2Block, SsdError, block_in_proj_pre, block_post, block_post_proj, block_pre,
-                                block_proj)
+from trading_bot_0_amd import Mamba2Block, SsdError, block_post, block_post_proj, block_pre, block_proj
 
 from _util import np64, rel_err
 
@@ -127,36 +126,6 @@ def test_stages_take_padded_rows(shape, dtype):
         block_pre(buf[:, :, 1:E + 1], p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G)
     with pytest.raises(ValueError):       # elements of a row not adjacent
         block_pre(buf[:, :, :2 * E:2], p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G)
-
-
-@pytest.mark.parametrize("shape", [(2, 512, 256, 8, 32, 64, 1, 4), (3, 256, 128, 8, 16, 32, 2, 3), (1, 768, 256, 16, 16, 128, 2, 2),
-                                   (9, 256, 256, 8, 32, 64, 1, 4), (2, 2048, 128, 8, 32, 64, 1, 4), (17, 256, 128, 8, 16, 64, 1, 2)])
-@pytest.mark.parametrize("with_state,keep_raw", [(False, False), (True, True)])
-def test_in_projection_with_pre_scan_in_one_kernel(shape, with_state, keep_raw):
-    """ssd_block_in_proj_pre_fwd against the two stages it fuses (ssd_block_proj_fwd into rows of whole lines, then
-    ssd_block_pre_fwd), which are themselves checked against float64: every output bit for bit -- z (and, when kept,
-    the raw x | B | C | dt channels) of zxbcdt, x, B, C, dt and the returned conv state.  Shapes: runs that start a
-    sequence and runs inside one (history from the 32 rows in front), a carried conv state, filter lengths 2 to 4,
-    column blocks of four and of five chunks, row counts off the workgroups' 2 048."""
-    Bsz, L, dm, H, P, N, G, K = shape
-    p = params(H, P, N, G, K)
-    DI, C, E = H * P, H * P + 2 * G * N, 2 * H * P + 2 * G * N + H
-    g = torch.Generator().manual_seed(L + dm + K)
-    u = torch.randn(Bsz, L, dm, generator=g).to(torch.bfloat16).cuda()
-    w = (torch.randn(E, dm, generator=g) / dm ** 0.5).to(torch.bfloat16).cuda()
-    st = torch.randn(Bsz, K - 1, C, generator=g).to(torch.bfloat16).cuda() if with_state else None
-    zx_ref = block_proj(u, w, pad_rows=True)
-    ref = block_pre(zx_ref, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=st, return_conv_state=True)
-    got = block_in_proj_pre(u, w, p["conv_w"], p["conv_b"], p["dt_bias"], H, P, N, G, conv_state=st,
-                            return_conv_state=True, keep_raw=keep_raw)
-    torch.cuda.synchronize()
-    zx = got[0]
-    assert zx.shape == zx_ref.shape and zx.stride() == zx_ref.stride()
-    assert torch.equal(zx[..., :DI], zx_ref[..., :DI]), "z channels"
-    if keep_raw:
-        assert torch.equal(zx, zx_ref), "raw x | B | C | dt channels"
-    for name, a, b in zip(("x", "B", "C", "dt", "conv state"), got[1:], ref):
-        assert a.shape == b.shape and torch.equal(a, b), name
 
 
 @pytest.mark.parametrize("shape", [(2, 50, 8, 32, 64, 1, 256), (3, 700, 8, 32, 64, 1, 256), (1, 2049, 8, 16, 16, 1, 128),

@@ -17,5 +17,5 @@ from .ssd import (  # noqa: F401
     workspace_bytes,
 )
 from .stream_state import SsdStreamState  # noqa: F401
-from .block import (GraphedBlockStep, block_in_proj_pre, Mamba2Block, Mamba2StreamState, block_post, block_post_bwd, block_post_proj, block_pre,  # noqa: F401
+from .block import (GraphedBlockStep, Mamba2Block, Mamba2StreamState, block_post, block_post_bwd, block_post_proj, block_pre,  # noqa: F401
                     block_pre_bwd, block_proj, block_step)

@@ -39,8 +39,6 @@ def _lib():
         lib.ssd_block_post_proj_fwd.restype = c_int
         lib.ssd_block_step_fwd.argtypes = [POINTER(SsdBlockDims), c_int, c_int64, P, P, P, P, P, P, P, P, c_float, P, P, P, P, P]
         lib.ssd_block_step_fwd.restype = c_int
-        lib.ssd_block_in_proj_pre_fwd.argtypes = [POINTER(SsdBlockDims), c_int, c_int64, P, P, P, P, P, P, P, c_int, P, P, P, P, P, P]
-        lib.ssd_block_in_proj_pre_fwd.restype = c_int
         lib.ssd_block_pre_reset_fwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, P, P, P, P, P, P, P, P, P]
         lib.ssd_block_pre_reset_fwd.restype = c_int
         lib.ssd_block_bwd_workspace_bytes.argtypes = [POINTER(SsdBlockDims), c_int, POINTER(c_size_t)]
@@ -190,52 +188,6 @@ def block_post_proj(y, zxbcdt, norm_w, weight, nheads, headdim, dstate, ngroups,
                                                 norm_w.data_ptr(), c_float(eps), weight.data_ptr(), weight.shape[0], 0,
                                                 out.data_ptr(), ssd._stream_ptr(zxbcdt)))
     return out
-
-
-def block_in_proj_pre_supported(u: torch.Tensor, nheads, headdim, dstate, ngroups) -> bool:
-    """Whether `block_in_proj_pre` takes this window (else `block_proj`, then `block_pre`)."""
-    return (u.is_cuda and u.dtype == torch.bfloat16 and u.dim() == 3 and u.shape[2] in (128, 256) and u.shape[1] % 256 == 0
-            and nheads % 8 == 0 and (nheads * headdim) % 64 == 0 and (ngroups * dstate) % 64 == 0
-            and in_proj_width(nheads, headdim, dstate, ngroups) > 160)
-
-
-def block_in_proj_pre(u, w_in, conv_w, conv_b, dt_bias, nheads, headdim, dstate, ngroups, conv_state=None,
-                      return_conv_state=False, keep_raw=False):
-    """In-projection and pre-scan stage as one kernel: u [B,L,d_model] (bf16) -> (zxbcdt [B,L,E] with rows of whole
-    128-byte lines, x [B,L,H,P], Bm, Cm [B,L,G,N], dt [B,L,H][, conv state]).  Of zxbcdt only the z channels are written
-    unless `keep_raw` (the backward pass reads the raw x | B | C | dt channels).  Equal to `block_proj(u, w_in,
-    pad_rows=True)` followed by `block_pre` bit for bit."""
-    lib = _lib()
-    Bsz, L, d_model = u.shape
-    H, P, N, G = nheads, headdim, dstate, ngroups
-    C = H * P + 2 * G * N
-    E = in_proj_width(H, P, N, G)
-    if u.dtype != torch.bfloat16 or w_in.dtype != torch.bfloat16:
-        raise ValueError("block_in_proj_pre takes bfloat16 tensors")
-    ssd._require(u, "u", (Bsz, L, d_model), torch.bfloat16)
-    ssd._require(w_in, "w_in", (E, d_model), torch.bfloat16)
-    d_conv = conv_w.shape[1]
-    ssd._require(conv_w, "conv_w", (C, d_conv), torch.float32)
-    ssd._require(conv_b, "conv_b", (C,), torch.float32)
-    ssd._require(dt_bias, "dt_bias", (H,), torch.float32)
-    if conv_state is not None:
-        ssd._require(conv_state, "conv_state", (Bsz, d_conv - 1, C), torch.bfloat16)
-    dev = u.device
-    ld = (E + 63) // 64 * 64
-    buf = torch.empty((Bsz, L, ld), dtype=torch.bfloat16, device=dev)
-    x = torch.empty((Bsz, L, H, P), dtype=torch.bfloat16, device=dev)
-    Bm = torch.empty((Bsz, L, G, N), dtype=torch.bfloat16, device=dev)
-    Cm = torch.empty((Bsz, L, G, N), dtype=torch.bfloat16, device=dev)
-    dt = torch.empty((Bsz, L, H), dtype=torch.bfloat16, device=dev)
-    new_state = torch.empty((Bsz, d_conv - 1, C), dtype=torch.bfloat16, device=dev) if return_conv_state else None
-    dims = SsdBlockDims(Bsz, L, H, P, N, G, d_conv, ld)
-    ssd._check(lib, lib.ssd_block_in_proj_pre_fwd(byref(dims), ssd.SSD_DTYPE_BF16, d_model, u.data_ptr(), w_in.data_ptr(),
-                                                  conv_w.data_ptr(), conv_b.data_ptr(), dt_bias.data_ptr(),
-                                                  ssd._ptr(conv_state), ssd._ptr(new_state), 1 if keep_raw else 0,
-                                                  buf.data_ptr(), x.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), dt.data_ptr(),
-                                                  ssd._stream_ptr(u)))
-    zxbcdt = buf[..., :E] if ld != E else buf
-    return (zxbcdt, x, Bm, Cm, dt, new_state) if return_conv_state else (zxbcdt, x, Bm, Cm, dt)
 
 
 # batches up to which one workgroup per stream (each reading both weight matrices whole) beats the stage kernels
@@ -464,31 +416,16 @@ class Mamba2Block:
             raise ValueError(f"block input must be [batch, seqlen, {self.d_model}], got {tuple(u.shape)}")
         if reset is not None and state is not None:
             raise ValueError("restarts inside the window and a carried conv state cannot be combined")
-        w_in = self._weights(u.dtype)[0]
-        fuse_in = (reset is None and u.is_contiguous() and u.shape[0] * u.shape[1] >= 16384
-                   and block_in_proj_pre_supported(u, self.H, self.P, self.N, self.G))
-        if fuse_in:
-            # in-projection with the pre-scan stage in its epilogue: the x | B | C | dt channels of zxbcdt leave the chip
-            # only for a forward that keeps its tensors for the backward pass, which reads them
-            got = block_in_proj_pre(u, w_in, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G,
-                                    conv_state=None if state is None else state.conv, return_conv_state=state is not None,
-                                    keep_raw=save_for_backward)
-            zxbcdt, x, Bm, Cm, dt = got[:5]
-            if state is not None:
-                state.conv = got[5]
-        else:
-            zxbcdt = self._project(u, w_in, pad_rows=True)  # internal to the block: rows of whole lines
-            if state is None:
-                x, Bm, Cm, dt = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G,
-                                          reset=reset)
-            else:
-                x, Bm, Cm, dt, conv = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N,
-                                                self.G, conv_state=state.conv, return_conv_state=True)
-                state.conv = conv
+        zxbcdt = self._project(u, self._weights(u.dtype)[0], pad_rows=True)  # internal to the block: rows of whole lines
         if state is None:
+            x, Bm, Cm, dt = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N, self.G,
+                                      reset=reset)
             y, _ = ssd.ssd_chunk_scan(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk, return_final_states=False,
                                       reset=reset)
         else:
+            x, Bm, Cm, dt, conv = block_pre(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, self.H, self.P, self.N,
+                                            self.G, conv_state=state.conv, return_conv_state=True)
+            state.conv = conv
             y = state.ssm.init_from_prefix(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk)
         w_out = self._weights(u.dtype)[1]
         if not save_for_backward and block_post_proj_supported(y, w_out) and y.numel() // self.d_inner >= 8192:

@@ -978,38 +978,6 @@ int ssd_block_post_proj_fwd(const ssd_block_dims *dims, int dtype, const void *y
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block post-scan + out-projection launch");
 }
 
-int ssd_block_in_proj_pre_fwd(const ssd_block_dims *dims, int dtype, int64_t d_model, const void *u, const void *w_in,
-                              const float *conv_w, const float *conv_b, const float *dt_bias, const void *conv_state_in,
-                              void *conv_state_out, int write_raw, void *zxbcdt, void *x, void *Bm, void *Cm, void *dt,
-                              void *hip_stream) {
-    ssd::BlockShape s;
-    if (int rc = make_block_shape(dims, dtype, &s)) return rc;
-    if (dtype != SSD_DTYPE_BF16)
-        return fail(SSD_ERR_UNSUPPORTED, "ssd: the fused in-projection + pre-scan takes dtype 1 (bfloat16), got %d", dtype);
-    if (d_model <= 0 || d_model > 0x7fffffff || !ssd::block_in_proj_pre_supported(s, (int)d_model))
-        return fail(SSD_ERR_UNSUPPORTED,
-                    "ssd: the fused in-projection + pre-scan needs d_model 128 or 256, seqlen a multiple of 256, nheads a "
-                    "multiple of 8 and more than 160 channels per row, got d_model %lld, seqlen %d, nheads %d",
-                    (long long)d_model, s.L, s.H);
-    REQUIRE_PTR(u);
-    REQUIRE_PTR(w_in);
-    REQUIRE_PTR(conv_w);
-    REQUIRE_PTR(conv_b);
-    REQUIRE_PTR(dt_bias);
-    REQUIRE_PTR(zxbcdt);
-    REQUIRE_PTR(x);
-    REQUIRE_PTR(Bm);
-    REQUIRE_PTR(Cm);
-    REQUIRE_PTR(dt);
-    OPTIONAL_PTR(conv_state_in);
-    OPTIONAL_PTR(conv_state_out);
-    if (conv_state_in != nullptr && conv_state_in == conv_state_out)
-        return fail(SSD_ERR_INVALID, "ssd: conv_state_in and conv_state_out must not alias here");
-    hipError_t e = ssd::launch_block_in_proj_pre(s, (int)d_model, u, w_in, conv_w, conv_b, dt_bias, conv_state_in,
-                                                 conv_state_out, write_raw, zxbcdt, x, Bm, Cm, dt, (hipStream_t)hip_stream);
-    return e == hipSuccess ? SSD_OK : hip_fail(e, "fused in-projection + pre-scan launch");
-}
-
 int ssd_block_step_fwd(const ssd_block_dims *dims, int dtype, int64_t d_model, const void *u, const void *w_in,
                        const float *conv_w, const float *conv_b, const float *dt_bias, const float *A, const float *D,
                        const float *norm_w, float eps, const void *w_out, void *conv_state, float *ssm_state, void *out,

@@ -129,10 +129,6 @@ hipError_t launch_block_proj(long long rows, int in_features, int out_features, 
 hipError_t launch_block_pre(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w,
                             const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
                             const unsigned char *reset, void *x, void *Bm, void *Cm, void *dt, hipStream_t stream);
-bool block_in_proj_pre_supported(const BlockShape &s, int d_model);
-hipError_t launch_block_in_proj_pre(const BlockShape &s, int d_model, const void *u, const void *w, const float *conv_w,
-                                    const float *conv_b, const float *dt_bias, const void *state_in, void *state_out,
-                                    int write_raw, void *zx, void *x, void *Bm, void *Cm, void *dt, hipStream_t st);
 bool block_step_supported(const BlockShape &s, int d_model);
 hipError_t launch_block_step(const BlockShape &s, int dtype, int d_model, const void *u, const void *w_in, const float *conv_w,
                              const float *conv_b, const float *dt_bias, const float *A, const float *D, const float *norm_w,

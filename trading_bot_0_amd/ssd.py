@@ -54,7 +54,6 @@ EXPORTED_SYMBOLS = (
     "ssd_block_pre_bwd",
     "ssd_block_post_proj_fwd",
     "ssd_block_step_fwd",
-    "ssd_block_in_proj_pre_fwd",
 )
 
 
