@@ -9,7 +9,7 @@ from oracle import ssd_oracle as orc
 from trading_bot_0_amd import SsdError, ssd_chunk_scan, ssd_chunk_scan_onepass
 from trading_bot_0_amd.synthetic import WORKLOADS, Workload, make_inputs
 
-from _util import assert_close, check_y, np64, oracle_scan, rel_err, to_dev
+from _util import assert_close, assert_stored_bf16_close, check_y, np64, oracle_scan, rel_err, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -294,3 +294,31 @@ def test_partial_last_round_runs_as_a_batch_of_its_own(batch, seqlen, dtype):
     assert torch.equal(y32[:256], y1[:256]) and torch.equal(final[:256], f1[:256])     # the whole round is that kernel
     tol = 1e-4 if dtype == "bf16" else 1e-5
     assert rel_err(y32[256:], np64(y1[256:])) <= tol and rel_err(final[256:], np64(f1[256:])) <= tol
+
+
+@pytest.mark.parametrize("heads", [(4, 32, 64, 1), (2, 64, 64, 1), (8, 32, 32, 2)])
+def test_groups_of_four_units_take_the_one_pass_kernel(heads):
+    """Four units per group (four heads of 32 columns, two of 64, eight in two groups): workgroups of four waves, two
+    to a CU.  The whole-forward entry point picks that path from mid-size batches on (it is the faster one there: 144
+    against 263 us for 256 sequences of 2 048 steps) and the staged kernels for small ones; rows against the oracle
+    with an initial state, a ragged length and restarts, and the bf16 y as the rounded float32 y."""
+    from trading_bot_0_amd.ssd import chunk_scan_is_onepass
+    H, P, N, G = heads
+    assert chunk_scan_is_onepass(300, 1000, H, P, N, G, 128)
+    assert not chunk_scan_is_onepass(16, 1000, H, P, N, G, 128)
+    w = Workload("four_units", 300, 1000, H, P, N, G, 128, init_std=0.5)
+    dev = make_inputs(w, seed=8, device="cuda")
+    m = (np.random.default_rng(4).random((w.batch, w.seqlen)) < 0.003).astype(np.uint8)
+    m[2, 0] = 1
+    reset = torch.from_numpy(m).cuda()
+    y32, final = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                                initial_states=dev["init"], y_dtype=torch.float32, reset=reset)
+    y16, final16 = ssd_chunk_scan(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], chunk=w.chunk,
+                                  initial_states=dev["init"], reset=reset)
+    assert torch.equal(y16, y32.to(torch.bfloat16)) and torch.equal(final, final16)
+    rows = [0, 2, 299]
+    yr, fr = orc.ssd_sequential(*(np64(dev[k][rows]) for k in ("x", "dt")), np64(dev["A"]), np64(dev["B"][rows]),
+                                np64(dev["C"][rows]), np64(dev["D"]), np64(dev["init"][rows]), reset=m[rows])
+    assert_close(y32[rows], yr, torch.bfloat16, "four-wave one-pass y (float32 y)")
+    assert_close(final[rows], fr, torch.bfloat16, "four-wave one-pass final")
+    assert_stored_bf16_close(y16[rows], yr, "four-wave one-pass stored y")

@@ -51,6 +51,19 @@ int fused_scan_plan(const ScanShape &s, int dtype, int *segments) {
         return whole < staged ? 1 : 0;
     }
     const int waves = fused_scan_waves(s, dtype);
+    if (waves == 4 && s.N != 128) {
+        // groups of four units (four heads of 32, two of 64 ...): workgroups of four waves, two to a CU.  A workgroup
+        // alone on its CU walks a tile in about 4.2 (one wave per SIMD), two sharing it in about 7.0 each; a round is 512
+        // workgroups.  Measured at 2 048 steps, 4 heads of 32, state 64: 256 sequences 144 (staged 263), 512 221
+        // (503), 1 024 459 (1 010); 128 sequences 125 against 124, below that the staged kernels win.  Not cut into
+        // segments (the states-only instance is the eight-wave one).
+        const long long groups = (long long)s.B * s.G * ((s.H / s.G) * (s.P / 32) / 4);
+        const int nc = tiles_of(s);
+        const double staged = 20.0 + 510.0 * ((double)groups * 4 * nc) / (2048.0 * 32.0);
+        const long long rounds = groups / 512, rest = groups % 512;
+        const double per_tile = 7.0 * rounds + (rest == 0 ? 0.0 : rest <= 256 ? 4.2 : 4.2 + 2.8 * (double)(rest - 256) / 256.0);
+        return 5.0 + per_tile * nc < staged ? 1 : 0;
+    }
     const int full = s.N == 128 ? 4 : 8;  // waves of a workgroup that fills a CU
     if (waves != full) return 0;
     const long long groups = (long long)s.B * s.G * ((s.H / s.G) * (s.P / 32) / full);
@@ -79,6 +92,7 @@ int fused_scan_plan(const ScanShape &s, int dtype, int *segments) {
 int fused_scan_tail_rows(const ScanShape &s, int dtype) {
     int segments;
     if (fused_scan_plan(s, dtype, &segments) != 1) return 0;
+    if (dtype != 0 && s.N != 128 && fused_scan_waves(s, dtype) == 4) return 0;  // (four-wave workgroups: whole rounds only)
     const int full = (dtype != 0 && s.N == 128) ? 4 : 8;
     const int per_row = s.G * ((s.H / s.G) * (s.P / 32) / full);  // workgroups per batch row
     const long long groups = (long long)s.B * per_row;
