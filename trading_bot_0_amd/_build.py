@@ -14,7 +14,7 @@ SOURCES = [CSRC / "ssd_stream_kernels.hip", CSRC / "ssd_chunk_state.hip", CSRC /
            CSRC / "ssd_chunk_scan_f32.hip",
            CSRC / "ssd_chunk_scan_bf16.hip", CSRC / "ssd_chunk_scan_bf16_y32.hip",
            CSRC / "ssd_fused_scan_bf16.hip", CSRC / "ssd_fused_scan_bf16_y32.hip", CSRC / "ssd_fused_scan_f32.hip",
-           CSRC / "ssd_fused_scan_segments.hip", CSRC / "ssd_fused_scan_transposed.hip", CSRC / "ssd_fused_scan_adjoint_rows.hip", CSRC / "ssd_block_proj.hip",
+           CSRC / "ssd_fused_scan_segments.hip", CSRC / "ssd_fused_scan_wide.hip", CSRC / "ssd_fused_scan_transposed.hip", CSRC / "ssd_fused_scan_adjoint_rows.hip", CSRC / "ssd_block_proj.hip",
            CSRC / "ssd_block_kernels.hip", CSRC / "ssd_block_step.hip", CSRC / "ssd_block_backward.hip", CSRC / "ssd_backward_kernels.hip", CSRC / "ssd_api.cpp"]
 OBJ_DIR = PKG_DIR / "build"
 

@@ -7,6 +7,11 @@ hipError_t launch_fused_scan_y32(const ScanShape &, int, const void *, const voi
                                  const void *, const float *, const float *, const unsigned char *, void *, float *,
                                  float *, hipStream_t);
 
+bool fused_scan_wide_supported(const ScanShape &);
+hipError_t launch_fused_scan_wide(const ScanShape &, int, const void *, const void *, const float *, const void *,
+                                  const void *, const float *, const float *, const unsigned char *, void *, float *,
+                                  hipStream_t);
+
 int fused_scan_waves(const ScanShape &s, int dtype) {
     if (dtype == 0) return 0;                         // float inputs take the staged kernels
     if (s.P % 32 != 0) return 0;
@@ -36,6 +41,10 @@ hipError_t launch_fused_scan(const ScanShape &s, int dtype, const void *x, const
     ScanShape t = s;  // the kernel's own tiling of time; the caller's chunk length does not enter
     t.Q = kOnePassTile;
     t.nc = (s.L + kOnePassTile - 1) / kOnePassTile;
+    // a 128-wide state: two waves per unit (the one-wave-per-unit instance stays for callers that want the state
+    // entering every tile, which that kernel can write)
+    if (tile_states == nullptr && fused_scan_wide_supported(t))
+        return launch_fused_scan_wide(t, dtype, x, dt, A, Bm, Cm, D, init, reset, y, final_states, st);
     if (dtype == 2)
         return launch_fused_scan_y32(t, waves, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
     return fused_dispatch<__bf16>(t, waves, x, dt, A, Bm, Cm, D, init, reset, y, final_states, tile_states, st);
