@@ -645,7 +645,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 refl[lb] = readlane_f(lo[0], (32 * lb) / EPL);
                 endh[lb] = readlane_f(hi[EPL - 1], (32 * lb + 31) / EPL);
                 endl[lb] = readlane_f(lo[EPL - 1], (32 * lb + 31) / EPL);
-                if (lane == 0) {
+                if (!STATES_ONLY && lane == 0) {
                     blk_s[lb] = exp2_hw(refh[lb] + refl[lb]);
                     blk_s[8 + lb] = fmaxf(alpha_diff(refh[lb], refl[lb], endh[lb], endl[lb]), 0.f);
                 }
@@ -656,21 +656,25 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 const int l = lane * EPL + e;
                 if (Q >= 64 || l < Q) {
                     const int blk = l >> 5;
-                    ah_s[l] = hi[e];
-                    alo_s[l] = lo[e];
-                    dt_s[l] = dtv[e];
-                    w_s[l] = exp2_hw(fminf(alpha_diff(endh[QB - 1], endl[QB - 1], hi[e], lo[e]), 0.f)) * dtv[e];
-                    float rh = refh[0], rl = refl[0];
-#pragma unroll
-                    for (int lb = 1; lb < QB; ++lb) {
-                        rh = (blk >= lb) ? refh[lb] : rh;
-                        rl = (blk >= lb) ? refl[lb] : rl;
+                    if constexpr (!STATES_ONLY) {
+                        ah_s[l] = hi[e];
+                        alo_s[l] = lo[e];
+                        dt_s[l] = dtv[e];
                     }
-                    E_s[l] = exp2_hw(fminf(alpha_diff(hi[e], lo[e], rh, rl), 0.f));
+                    w_s[l] = exp2_hw(fminf(alpha_diff(endh[QB - 1], endl[QB - 1], hi[e], lo[e]), 0.f)) * dtv[e];
+                    if constexpr (!STATES_ONLY) {  // (phase 1's tables: the states-only pass has no phase 1)
+                        float rh = refh[0], rl = refl[0];
 #pragma unroll
-                    for (int lb = 0; lb < QB; ++lb)
-                        if (lb >= blk)
-                            F_s[lb * Q + l] = exp2_hw(fminf(alpha_diff(refh[lb], refl[lb], hi[e], lo[e]), 126.f)) * dtv[e];
+                        for (int lb = 1; lb < QB; ++lb) {
+                            rh = (blk >= lb) ? refh[lb] : rh;
+                            rl = (blk >= lb) ? refl[lb] : rl;
+                        }
+                        E_s[l] = exp2_hw(fminf(alpha_diff(hi[e], lo[e], rh, rl), 0.f));
+#pragma unroll
+                        for (int lb = 0; lb < QB; ++lb)
+                            if (lb >= blk)
+                                F_s[lb * Q + l] = exp2_hw(fminf(alpha_diff(refh[lb], refl[lb], hi[e], lo[e]), 126.f)) * dtv[e];
+                    }
                 }
             }
         }
