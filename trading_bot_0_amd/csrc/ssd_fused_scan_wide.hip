@@ -14,8 +14,8 @@
 //     diagonal block) -- so the masked, decayed score tiles, the part of a tile's work that does not shrink with the
 //     state, are each formed once, and no partial sums cross waves.
 // A workgroup is four units (eight waves, two per SIMD: wave w and w + 4 are the two halves of unit w, on SIMD w),
-// sharing the B and C tiles of their (batch, group) as before.  The scan of dt*A and the decay tables are computed by
-// both waves of a unit (each in its own LDS rows): 250 vector instructions of 750 per wave and tile.
+// sharing the B and C tiles of their (batch, group) as before.  The scan of dt*A and the decay tables of a unit are
+// computed by its first wave for both (250 vector instructions, about what the second wave's extra score block costs).
 //
 // Everything else -- tiling of time by 64 steps whatever chunk length the caller names, the separable decay factors
 // with the exact path for blocks that decay by more than 2^-120, hi + lo operands for everything the kernel
@@ -29,14 +29,14 @@ namespace {
 
 constexpr int kWideN = 128, kWideNK = 8, kWideUnits = 4, kWideWaves = 8, kWideQ = kOnePassTile, kWideQB = kWideQ / 32;
 // LDS: B and C tiles [Q][128], four x tiles [Q][32], the units' states in operand form ([unit][K step][hi, lo]
-// [lane] 16 bytes), per-wave tables
+// [lane] 16 bytes), per-unit tables
 constexpr int kWideTableFloats = (5 + kWideQB) * kWideQ + 16;
 // (the x tiles keep the eight-unit layout's offsets, fused_scan_xtile_base: by the hardware's bank-conflict counter the
 // staging writes of four units are free of conflicts with them, and were not with the second pair of units 128 instead
 // of 64 bytes further)
 constexpr int kWideXArea = kWideUnits * fused_scan_xtile_elems(kWideQ);
 constexpr size_t kWideLdsBytes = (size_t)2 * kWideQ * kWideN * 2 + (size_t)kWideXArea * 2 +
-                                 (size_t)kWideUnits * kWideNK * 2 * 64 * 16 + (size_t)kWideWaves * kWideTableFloats * 4;
+                                 (size_t)kWideUnits * kWideNK * 2 * 64 * 16 + (size_t)kWideUnits * kWideTableFloats * 4;
 
 template <typename TO>
 __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
@@ -64,9 +64,9 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
     T *const Cs = Bs + Q * N;
     T *const xs_all = Cs + Q * N;
     T *const hfrag = xs_all + kWideXArea;       // [UNITS][NK][2][64][8]
-    float *const wf = reinterpret_cast<float *>(hfrag + UNITS * NK * 2 * 64 * 8) + wave * kWideTableFloats;
+    float *const wf = reinterpret_cast<float *>(hfrag + UNITS * NK * 2 * 64 * 8) + ul * kWideTableFloats;  // (per unit)
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
-    float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [8..8+QB): log2-decay across block lb
+    float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [4]: exp2(alpha[Q-1]); [8..8+QB): log2-decay across block lb
     T *const xs = xs_all + fused_scan_xtile_base(Q, ul);
     T *const hf_unit = hfrag + (size_t)ul * NK * 2 * 64 * 8;
 
@@ -210,9 +210,9 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
             *reinterpret_cast<uint4 *>(dst) = make_uint4(fh.u[0], fh.u[1], fh.u[2], fh.u[3]);
             *reinterpret_cast<uint4 *>(dst + 64 * 8) = make_uint4(fl.u[0], fl.u[1], fl.u[2], fl.u[3]);
         }
-        // ---- scan of dt*A over the tile and the decay tables (both waves of a unit, each in its own rows) ----
-        float a_end;  // exp2(alpha[Q-1]): the tile's total decay
-        {
+        // ---- scan of dt*A over the tile and the decay tables: the unit's first wave, for both (the second has one
+        // more score block in phase 1, about as much work) ----
+        if (role == 0) {
             constexpr double kLog2e = 1.4426950408889634;
             const float dtv = (float)__builtin_bit_cast(__bf16, dq);
             const double run = (double)dtv * a_h - (rq ? kResetDrop : 0.0);
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
                     blk_s[8 + lb] = fmaxf(alpha_diff(refh[lb], refl[lb], endh[lb], endl[lb]), 0.f);
                 }
             }
-            a_end = exp2_hw(endh[QB - 1] + endl[QB - 1]);
+            if (lane == 0) blk_s[4] = exp2_hw(endh[QB - 1] + endl[QB - 1]);  // the tile's total decay
             const int l = lane, blk = l >> 5;
             ah_s[l] = hi;
             alo_s[l] = lo;
@@ -243,6 +243,7 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
                 if (lb >= blk) F_s[lb * Q + l] = exp2_hw(fminf(alpha_diff(refh[lb], refl[lb], hi, lo), 126.f)) * dtv;
         }
         block_sync_lds();  // tiles, operand fragments and tables are visible
+        const float a_end = blk_s[4];  // exp2(alpha[Q-1])
         // the next tile's inputs: requested here, in flight during both phases, stored to LDS at the top of the next tile
         if (c + 1 < s.nc) prefetch(c + 1);
         __builtin_amdgcn_sched_barrier(0);  // (left alone, the scheduler moves the loads down to where their values are used)
