@@ -448,7 +448,10 @@ def main():
         out["backward"] = {"ms": round(t_bwd * 1e3, 4), "alg_bytes": bwd_bytes,
                            "GBps": round(bwd_bytes / t_bwd / 1e9, 1),
                            "hbm_frac": round(bwd_bytes / t_bwd / 1e9 / HBM_PEAK_GBS, 4),
-                           "workspace_bytes": wsb.numel(), "units_per_s": round(BL / t_bwd, 1)}
+                           "workspace_bytes": wsb.numel(), "units_per_s": round(BL / t_bwd, 1),
+                           "parity": "against this repository's float64 adjoint, pinned by central differences of the forward "
+                                     "oracle (tests/test_oracle_backward.py); the reference holds no backward of this op: "
+                                     "unpinned by the reference"}
         del dyb, wsb
 
     # ---- the other workloads at full size: forward only, one row each -----------------------------------
@@ -705,6 +708,8 @@ def main():
         t_in_blas = timed(lambda: torch.matmul(u, w_in.t()))
         t_out_blas = timed(lambda: torch.matmul(yn, w_out.t()))
         out["mamba2_block"] = {"d_model": blk.d_model, "ms": round(t_block, 4),
+                               "parity": "against this repository's float64 block oracle (tests/test_oracle_block.py pins it); "
+                                         "the reference holds no source or vector of this layer: unpinned by the reference",
                                "in_proj_ms": round(t_in, 4), "in_proj_GBps": round(in_bytes / t_in / 1e6, 1),
                                "in_proj_dense_rows_ms": round(t_in_dense, 4), "in_proj_blas_ms": round(t_in_blas, 4),
                                "pre_ms": round(t_pre, 4), "pre_GBps": round(pre_bytes / t_pre / 1e6, 1),

@@ -116,7 +116,9 @@ int ssd_chunk_state_passing_fwd(const ssd_dims *dims, int dtype, const void *x, 
  * state of 32 head-dim columns of one (batch, head) in registers while it walks the chunks, so no workspace
  * is needed and nothing but x, dt, B, C is read and y, final_states written.  Same arguments (with the
  * optional reset mask of ssd_chunk_scan_reset_fwd) and results as ssd_chunk_scan_fwd.  Parallel over
- * (batch, head) sequences only; ssd_chunk_scan_fwd takes this path by itself when there are enough of them.  SSD_ERR_UNSUPPORTED unless headdim is a
+ * (batch, head) sequences only; ssd_chunk_scan_fwd takes this path by itself when there are enough of them (groups of
+ * eight such units in workgroups of eight waves; groups of four in workgroups of four waves, two to a CU; a 128-wide
+ * state with two waves per unit, half of the state each).  SSD_ERR_UNSUPPORTED unless headdim is a
  * multiple of 32 and, for bf16 inputs (dtype 1 or 2), dstate is 32, 64 or 128 and (nheads/ngroups)*(headdim/32) a
  * multiple of 4; for float32 inputs (every operand enters the matrix cores as three bf16 terms, six products per
  * multiplication: float accuracy at three eighths of the float instruction's cost), dstate is 32 or 64 and
