@@ -71,12 +71,13 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # Reads come out below the compulsory bytes because inputs that stay in the 256 MB last-level cache from one call
 # of the loop to the next are not fetched from HBM again.
 MEASURED_TRAFFIC_BYTES = {("policy_bf16", 256): 491.9e6,          # 201 100 + 279 300 KiB, one launch
-                          ("long_lookback_bf16", 32): 2012.4e6,   # 900 200 + 1 065 000 KiB, one launch
-                          ("decay_extreme", 64): 325.0e6}         # states only 63 060 + 12 290, forward 106 700 + 135 400 KiB
-TRAFFIC_MEASURED_AT = "c6b6689"   # the library revision the counter runs in profiles/ were made at
-# matrix-pipe busy fraction of the same kernels from the same counter runs (SQ_VALU_MFMA_BUSY_CYCLES over
-# SQ_BUSY_CU_CYCLES): what the north star's "MFMA utilisation" reads as on the hardware's own counters
-MEASURED_MFMA_PIPE_BUSY = {("policy_bf16", 256): 0.27, ("long_lookback_bf16", 32): 0.238}
+                          ("long_lookback_bf16", 32): 1992.8e6,   # 881 100 + 1 065 000 KiB, one launch
+                          ("decay_extreme", 64): 324.9e6}         # states only 63 050 + 12 290, forward 106 700 + 135 300 KiB
+TRAFFIC_MEASURED_AT = "60c9700"   # the library revision the counter runs in profiles/ were made at
+# matrix-pipe busy fraction of the same kernels from the same counter runs (SQ_VALU_MFMA_BUSY_CYCLES over the
+# SIMD-cycles of the launch, GRBM_GUI_ACTIVE / 8 x 1 024 SIMDs): what the north star's "MFMA utilisation" reads as
+# on the hardware's own counters
+MEASURED_MFMA_PIPE_BUSY = {("policy_bf16", 256): 0.267, ("long_lookback_bf16", 32): 0.306, ("decay_extreme", 64): 0.213}
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 
@@ -339,8 +340,9 @@ def main():
                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, w.batch)),
                     "traffic_measured_at": TRAFFIC_MEASURED_AT if (w.name, w.batch) in MEASURED_TRAFFIC_BYTES else None,
                     "mfma_pipe_busy": MEASURED_MFMA_PIPE_BUSY.get((w.name, w.batch)),
-                    "mfma_pipe_busy_note": "SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CU_CYCLES of the same kernel, from the "
-                                           "rocprofv3 --pmc run of the same revision (profiles/)"}
+                    "mfma_pipe_busy_note": "SQ_VALU_MFMA_BUSY_CYCLES over the launch's SIMD-cycles (GRBM_GUI_ACTIVE / 8 x "
+                                           "1024) of the same kernel, from the rocprofv3 --pmc run of that revision "
+                                           "(profiles/)"}
         if w.dtype == "bf16":
             # the float32-y instance of the same kernel: the output err_y is measured on (bf16 inputs, y in float32,
             # so its compulsory traffic holds y at four bytes per element)
