@@ -200,8 +200,11 @@ constexpr double kResetDrop = kResetLog2 / 1.4426950408889634;
 // ------------------------------------------------------------------------------------------
 template <int CTRL, int ROWMASK> __device__ inline double dpp_move(double v) {
     int lo = __double2loint(v), hi = __double2hiint(v);
-    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROWMASK, 0xf, false);
-    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROWMASK, 0xf, false);
+    // With every row enabled the hardware's own zero for a lane without a source (bound_ctrl) does what the zero
+    // "old" value does, and the destination needs no clearing first (two moves per step less).
+    constexpr bool kBound = ROWMASK == 0xf;
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROWMASK, 0xf, kBound);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROWMASK, 0xf, kBound);
     return __hiloint2double(hi, lo);  // lanes the row mask disables, or with no source lane, get +0.0
 }
 // Inclusive sum across the 64 lanes with DPP data movement: shifts inside rows of 16, then the
@@ -381,6 +384,36 @@ __device__ inline void split_pair(float a0, float f0, float a1, float f1, unsign
     const bf16x2 h = __builtin_bit_cast(bf16x2, hi);
     lo = pack_bf16x2(__builtin_amdgcn_fdot2_f32_bf16(h, __builtin_bit_cast(bf16x2, first), m0, false),
                      __builtin_amdgcn_fdot2_f32_bf16(h, __builtin_bit_cast(bf16x2, second), m1, false));
+}
+// The same split of eight plain values that stay live afterwards (the running state), as one operand fragment pair.
+// The three-operand form of the dot product writes the remainder to a register of its own, where the two-operand form
+// above accumulates in place and the compiler has to copy each value first (two moves per pair).  The compiler does not
+// select that form, so it is written out; and since it does not look inside such a block, the wait the hardware needs
+// between a dot product and the next instruction that reads its result (three wait states, which the compiler inserts
+// by itself behind the two-operand form) stands at the end of the block, behind eight independent products.
+__device__ inline void split8_keep(const float (&a)[8], unsigned (&hi)[4], unsigned (&lo)[4]) {
+    unsigned first = 0x0000bf80u, second = 0xbf800000u;
+    asm("" : "+s"(first));
+    asm("" : "+s"(second));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) hi[k] = pack_bf16x2(a[2 * k], a[2 * k + 1]);
+    float l0, l1, l2, l3, l4, l5, l6, l7;
+    asm("v_dot2_f32_bf16 %0, %8, %12, %14\n\t"
+        "v_dot2_f32_bf16 %1, %8, %13, %15\n\t"
+        "v_dot2_f32_bf16 %2, %9, %12, %16\n\t"
+        "v_dot2_f32_bf16 %3, %9, %13, %17\n\t"
+        "v_dot2_f32_bf16 %4, %10, %12, %18\n\t"
+        "v_dot2_f32_bf16 %5, %10, %13, %19\n\t"
+        "v_dot2_f32_bf16 %6, %11, %12, %20\n\t"
+        "v_dot2_f32_bf16 %7, %11, %13, %21\n\t"
+        "s_nop 2"
+        : "=&v"(l0), "=&v"(l1), "=&v"(l2), "=&v"(l3), "=&v"(l4), "=&v"(l5), "=&v"(l6), "=&v"(l7)
+        : "v"(hi[0]), "v"(hi[1]), "v"(hi[2]), "v"(hi[3]), "s"(first), "s"(second), "v"(a[0]), "v"(a[1]), "v"(a[2]),
+          "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7]));
+    lo[0] = pack_bf16x2(l0, l1);
+    lo[1] = pack_bf16x2(l2, l3);
+    lo[2] = pack_bf16x2(l4, l5);
+    lo[3] = pack_bf16x2(l6, l7);
 }
 struct FragBits {  // an operand fragment as four packed pairs
     unsigned u[4];

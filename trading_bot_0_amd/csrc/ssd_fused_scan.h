@@ -690,11 +690,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             for (int sk = 0; sk < SL * NK; ++sk) {  // slice sk / NK, K step sk % NK
                 const int kk = sk % NK, sn = (sk / NK) * NB + kk / 2;
                 FragBits fh, fl;
+                float sv[8];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int v = 8 * (kk % 2) + 2 * i;
-                    split_pair(st[sn][v], 1.f, st[sn][v + 1], 1.f, fh.u[i], fl.u[i]);
-                }
+                for (int i = 0; i < 8; ++i) sv[i] = st[sn][8 * (kk % 2) + i];
+                split8_keep(sv, fh.u, fl.u);
                 Hhi[sk] = fh.frag();
                 Hlo[sk] = fl.frag();
             }
@@ -744,9 +743,14 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     for (int vg = 0; vg < 4; ++vg) aq[vg] = *reinterpret_cast<const uint2 *>(ar + 8 * vg);
                     wt = (float)dt[((size_t)b * trows + arow) * s.H + h];
                 }
+                // The tiles' swizzles repeat every 32 rows, so a row's address is its block's base plus the offset of
+                // the row inside its block -- the same lane-derived offsets for every block, B or C tile alike, which
+                // stay in registers across the blocks and tiles (computed from the full row index they were formed
+                // again per block: 50 address instructions per column block).
+                const T *const Cs_lb = Cs + lb * 32 * N, *const xs_lb = xs + lb * 32 * 32;
                 Frag<T> Cf[NK];
 #pragma unroll
-                for (int kk = 0; kk < NK; ++kk) Cf[kk] = BT::split_frag(Cs, l, 16 * kk + 4 * half);
+                for (int kk = 0; kk < NK; ++kk) Cf[kk] = BT::split_frag(Cs_lb, r, 16 * kk + 4 * half);
                 f32x16 accs[SL];  // one output tile per slice
 #pragma unroll
                 for (int sl = 0; sl < SL; ++sl) {
@@ -767,7 +771,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 auto block = [&](int sb, bool diag) {
                     Frag<T> Bf[NK];
 #pragma unroll
-                    for (int kk = 0; kk < NK; ++kk) Bf[kk] = BT::split_frag(Bs, sb * 32 + r, 16 * kk + 4 * half);
+                    for (int kk = 0; kk < NK; ++kk) Bf[kk] = BT::split_frag(Bs + sb * 32 * N, r, 16 * kk + 4 * half);
                     f32x16 sc = {0};
 #pragma unroll
                     for (int kk = 0; kk < NK; ++kk) sc = mma32(Bf[kk], Cf[kk], sc);
@@ -777,16 +781,17 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     for (int sl = 0; sl < SL; ++sl) {
 #pragma unroll
                         for (int j = 0; j < 2; ++j)  // K order of mh[j]: rows 32 sb + 16 j + 4 half + {0..3} and the same + 8
-                            xf[sl][j] = XT::frag(xs + sl * XS, sb * 32 + 16 * j + 4 * half, 8, 0, lane);
+                            xf[sl][j] = XT::frag(xs + sl * XS + sb * 32 * 32, 16 * j + 4 * half, 8, 0, lane);
                     }
                     float4 fv[4];
                     if (!diag || fast) {
 #pragma unroll
                         for (int vg = 0; vg < 4; ++vg) fv[vg] = *reinterpret_cast<const float4 *>(F_row + sb * 32 + 8 * vg + 4 * half);
                     }
-                    float El = 1.f;
+                    float El = 1.f, Eend = 1.f;  // Eend: what scales the finished sum (1 on the exact path, which scales first)
                     if (diag) {
                         El = E_s[l];
+                        Eend = fast ? El : 1.f;
                         if (!fast) {
 #pragma unroll
                             for (int sl = 0; sl < SL; ++sl) accs[sl] = accs[sl] * El;
@@ -816,7 +821,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                             accs[sl] = mma32(xf[sl][j], ml[j], accs[sl]);
 #endif
                         }
-                        if (diag && fast) accs[sl] = accs[sl] * El;  // everything summed so far shares the factor E[l]
+                        if (diag) accs[sl] = accs[sl] * Eend;  // everything summed so far shares the factor E[l]
                     }
                 };
                 // compile-time block index: every LDS address is a lane offset plus an immediate
@@ -885,7 +890,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     float o[16], pe = 0.f, pd = 0.f;
 #pragma unroll
                     for (int vg = 0; vg < 4; ++vg) {
-                        const bf16x4 x4 = XT::row4(xs, ll, 8 * vg + 4 * he);
+                        const bf16x4 x4 = XT::row4(xs_lb, le & 31, 8 * vg + 4 * he);
                         const bf16x4 a4 = __builtin_bit_cast(bf16x4, aq[vg]);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
@@ -907,9 +912,12 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     float o[16];
 #pragma unroll
                     for (int vg = 0; vg < 4; ++vg) {
-                        const bf16x4 x4 = XT::row4(xs, ll, 8 * vg + 4 * he);
+                        const bf16x4 x4 = XT::row4(xs_lb, le & 31, 8 * vg + 4 * he);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) o[vg * 4 + i] = acc[vg * 4 + i] + dh * (float)x4[i];
+                        // (an explicit fused multiply-add: left to the compiler, the scaling of acc by E[l] just above and
+                        // this sum contract one way in the bf16-y instance and the other in the float-y one, and the
+                        // stored bf16 y is no longer the float y rounded once)
+                        for (int i = 0; i < 4; ++i) o[vg * 4 + i] = __builtin_fmaf(dh, (float)x4[i], acc[vg * 4 + i]);
                     }
                     const int yrow = ADJ ? s.L - 1 - (t0 + ll) : t0 + ll;
                     store_column_buffer<TO>(ybuf, (unsigned)yrow * (unsigned)(HP * sizeof(TO)) + ycol_bytes, o, he,
