@@ -201,11 +201,10 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
 #pragma unroll
         for (int k4 = 0; k4 < 2 * HNB; ++k4) {  // K step 4 role + k4: block k4 / 2 of the half, accumulator rows 8 (k4 % 2) ..
             FragBits fh, fl;
+            float sv[8];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int v = 8 * (k4 % 2) + 2 * i;
-                split_pair(st[k4 / 2][v], 1.f, st[k4 / 2][v + 1], 1.f, fh.u[i], fl.u[i]);
-            }
+            for (int i = 0; i < 8; ++i) sv[i] = st[k4 / 2][8 * (k4 % 2) + i];
+            split8_keep(sv, fh.u, fl.u);
             T *dst = hf_unit + ((size_t)(4 * role + k4) * 2) * 64 * 8 + lane * 8;
             *reinterpret_cast<uint4 *>(dst) = make_uint4(fh.u[0], fh.u[1], fh.u[2], fh.u[3]);
             *reinterpret_cast<uint4 *>(dst + 64 * 8) = make_uint4(fl.u[0], fl.u[1], fl.u[2], fl.u[3]);
@@ -308,9 +307,10 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
 #pragma unroll
                     for (int vg = 0; vg < 4; ++vg) fv[vg] = *reinterpret_cast<const float4 *>(F_row + sb * 32 + 8 * vg + 4 * half);
                 }
-                float El = 1.f;
+                float El = 1.f, Eend = 1.f;  // Eend: what scales the finished sum (1 on the exact path, which scales first)
                 if (diag) {
                     El = E_s[l];
+                    Eend = fast ? El : 1.f;
                     if (!fast) {
                         acc = acc * El;
                         const float al_hi = ah_s[l], al_lo = alo_s[l];
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
                     acc = mma32(xf[j], mh[j], acc);
                     acc = mma32(xf[j], ml[j], acc);
                 }
-                if (diag && fast) acc = acc * El;  // everything summed so far shares the factor E[l]
+                if (diag) acc = acc * Eend;  // everything summed so far shares the factor E[l]
                 __builtin_amdgcn_sched_barrier(0);  // (one block's fragments at a time)
             };
             if constexpr (lb == 1) block(std::integral_constant<int, 0>{}, std::false_type{});
@@ -346,7 +346,8 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
             for (int vg = 0; vg < 4; ++vg) {
                 const bf16x4 x4 = XT::row4(xs, l, 8 * vg + 4 * half);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) o[vg * 4 + i] = acc[vg * 4 + i] + dh * (float)x4[i];
+                // (an explicit fused multiply-add, so that the bf16-y and the float-y instance round alike)
+                for (int i = 0; i < 4; ++i) o[vg * 4 + i] = __builtin_fmaf(dh, (float)x4[i], acc[vg * 4 + i]);
             }
             const int yrow = t0 + l;
             store_column_buffer<TO>(ybuf, (unsigned)yrow * (unsigned)(HP * sizeof(TO)) + ycol_bytes, o, half, l < rows);
