@@ -718,7 +718,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 }
             };
             // rolled where registers are tight; the 128-wide-state instance has a wave's whole register file
-            constexpr int kUnrollBlocks = NK == 8 ? QB : 1;
+            constexpr int kUnrollBlocks = (NK == 8 || ((KIND == 0 || KIND == 5) && WAVES == 8)) ? QB : 1;
 #pragma unroll kUnrollBlocks
             for (int lb = 0; lb < QB; ++lb) {
                 const int l = lb * 32 + r;
@@ -1046,6 +1046,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         }
         return true;
     };
+    // Nothing in flight when the tile loop is entered: the wait for a tile's inputs at the loop's head is then counted
+    // from the loop's own path alone -- they are older than the tile's stores of y, so the wave need not wait for
+    // those to be acknowledged -- instead of from the prologue's, where they are the youngest requests.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     if constexpr (kTwoSets) {
         for (int c = c_first; c < c_end; c += 2) {
             if (!tile(c, std::integral_constant<int, 0>{})) break;
