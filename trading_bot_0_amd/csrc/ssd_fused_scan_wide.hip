@@ -167,6 +167,10 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
 
     const int lane = lane0, r = lane & 31, half = lane >> 5;
 
+    // Nothing in flight when the tile loop is entered: the wait for a tile's inputs at the loop's head is then counted
+    // along the loop's own path, where they are older than the tile's stores of y (which the wave need not see
+    // acknowledged), not along the prologue's, where they are the youngest requests.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     for (int c = 0; c < s.nc; ++c) {
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
