@@ -199,9 +199,15 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     using BT = ChunkTile<N>;
     // static, so that LDS addresses are compile-time offsets
     constexpr int XS = SL == 2 ? wide_transposed_tile_elems(Q) : fused_scan_xtile_elems(Q);
+    // The eight units of a workgroup are the eight heads (or head slices) of one group: they share B and C, and so the
+    // scores B . C^T of a tile -- three blocks of 32 x 32 with tiles of 64 steps.  Three waves form one block each and
+    // leave it in LDS in the accumulator's own layout, every wave reads the three from there: 12 matrix instructions
+    // per tile and workgroup instead of 96, for 12 KB of LDS and a second barrier per tile (behind the first block's
+    // readout, where the scores are first needed).
+    constexpr bool kSharedScores = !TR && KIND != 2 && WAVES == 8 && QB == 2 && NK <= 4;
     __shared__ __attribute__((aligned(16))) unsigned char smem[SL == 2 ? wide_transposed_scan_lds_bytes(Q)
                                                                         : TR ? transposed_scan_lds_bytes(Q)
-                                                                             : fused_scan_lds_bytes(N, Q, WAVES)];  // (kind 5 uses one set of the two)
+                                                                             : fused_scan_lds_bytes(N, Q, WAVES) + (kSharedScores ? 3 * 32 * 32 * 4 : 0)];  // (kind 5 uses one set of the two)
     const int tid = threadIdx.x;
     const int lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -222,6 +228,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     float *wf = wf0 + wave * ((5 + QB) * Q + 16);
     // transposed only: every head's output tile, [WAVES][Q][33], or [WAVES][32][64] (swizzled) with two slices per wave
     float *red = wf0 + WAVES * ((5 + QB) * Q + 16);
+    float *const G_s = red;  // shared scores (not transposed): [3 blocks][4 quarters][64 lanes][4 floats]
     constexpr int RS = SL == 2 ? 64 : 33;
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
     float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [8..8+QB): log2-decay across block lb
@@ -681,6 +688,31 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         if (kEarlyPrefetch && c + 1 < c_end) prefetch(c + 1);
         block_sync_lds();  // tiles and tables are visible
 
+        if constexpr (kSharedScores) {
+            if (wave < 3) {  // block g = sb + lb: (0,0), (0,1), (1,1)
+                const int lane = phase_tid() & 63, r = lane & 31, half = lane >> 5;
+                // (the wave index hidden from the compiler here: it would otherwise keep the sixteen addresses below,
+                // which differ from the ones every wave uses by a wave-uniform offset only, in registers of their own
+                // across the tile loop, and spill them)
+                int pw = wave;
+                asm volatile("" : "+s"(pw));
+                const int psb = pw == 2 ? 1 : 0, plb = pw == 0 ? 0 : 1;
+                Frag<T> Cp[NK], Bp[NK];
+#pragma unroll
+                for (int kk = 0; kk < NK; ++kk) {
+                    Cp[kk] = BT::split_frag(Cs + plb * 32 * N, r, 16 * kk + 4 * half);
+                    Bp[kk] = BT::split_frag(Bs + psb * 32 * N, r, 16 * kk + 4 * half);
+                }
+                f32x16 sc = {0};
+#pragma unroll
+                for (int kk = 0; kk < NK; ++kk) sc = mma32(Bp[kk], Cp[kk], sc);
+                float *gd = G_s + pw * 1024 + lane * 4;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<float4 *>(gd + q * 256) = make_float4(sc[4 * q], sc[4 * q + 1], sc[4 * q + 2], sc[4 * q + 3]);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // (the producers' fragments are dead before the state's operand form is made)
+        }
         // ---- phase 1: outputs of this chunk from the state entering it ----
         if constexpr (!STATES_ONLY) {
             const int lane = phase_tid() & 63;
@@ -764,17 +796,32 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                     }
                     accs[sl] = accs[sl] * blk_s[lb];
                 }
+                if constexpr (kSharedScores) {
+                    if (lb == 0) block_sync_lds();  // the three blocks of scores are in LDS
+                }
                 f32x16 &acc = accs[0];
                 const float *F_row = F_s + lb * Q;
                 // one s-block.  On the separable path the diagonal block is one more term of the sum that E[l]
                 // scales at the end; on the exact path the sum is scaled first and the block carries its full factors.
                 auto block = [&](int sb, bool diag) {
-                    Frag<T> Bf[NK];
-#pragma unroll
-                    for (int kk = 0; kk < NK; ++kk) Bf[kk] = BT::split_frag(Bs + sb * 32 * N, r, 16 * kk + 4 * half);
                     f32x16 sc = {0};
+                    if constexpr (kSharedScores) {
+                        const float *gs = G_s + (sb + lb) * 1024 + lane * 4;
 #pragma unroll
-                    for (int kk = 0; kk < NK; ++kk) sc = mma32(Bf[kk], Cf[kk], sc);
+                        for (int q = 0; q < 4; ++q) {
+                            const float4 t = *reinterpret_cast<const float4 *>(gs + q * 256);
+                            sc[4 * q] = t.x;
+                            sc[4 * q + 1] = t.y;
+                            sc[4 * q + 2] = t.z;
+                            sc[4 * q + 3] = t.w;
+                        }
+                    } else {
+                        Frag<T> Bf[NK];
+#pragma unroll
+                        for (int kk = 0; kk < NK; ++kk) Bf[kk] = BT::split_frag(Bs + sb * 32 * N, r, 16 * kk + 4 * half);
+#pragma unroll
+                        for (int kk = 0; kk < NK; ++kk) sc = mma32(Bf[kk], Cf[kk], sc);
+                    }
                     // requested while the score MFMAs run
                     Frag<T> xf[SL][2];
 #pragma unroll
