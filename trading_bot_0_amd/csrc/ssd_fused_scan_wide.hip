@@ -35,8 +35,11 @@ constexpr int kWideTableFloats = (5 + kWideQB) * kWideQ + 16;
 // staging writes of four units are free of conflicts with them, and were not with the second pair of units 128 instead
 // of 64 bytes further)
 constexpr int kWideXArea = kWideUnits * fused_scan_xtile_elems(kWideQ);
+// ... and the tile's three blocks of scores B . C^T, which the workgroup's four units share (one group's B and C): three
+// waves form a block each, in the accumulator's layout ([block][quarter][lane] 16 bytes), and every wave reads its blocks
 constexpr size_t kWideLdsBytes = (size_t)2 * kWideQ * kWideN * 2 + (size_t)kWideXArea * 2 +
-                                 (size_t)kWideUnits * kWideNK * 2 * 64 * 16 + (size_t)kWideUnits * kWideTableFloats * 4;
+                                 (size_t)kWideUnits * kWideNK * 2 * 64 * 16 + (size_t)kWideUnits * kWideTableFloats * 4 +
+                                 (size_t)3 * 32 * 32 * 4;
 
 template <typename TO>
 __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
@@ -65,6 +68,7 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
     T *const xs_all = Cs + Q * N;
     T *const hfrag = xs_all + kWideXArea;       // [UNITS][NK][2][64][8]
     float *const wf = reinterpret_cast<float *>(hfrag + UNITS * NK * 2 * 64 * 8) + ul * kWideTableFloats;  // (per unit)
+    float *const G_s = reinterpret_cast<float *>(hfrag + UNITS * NK * 2 * 64 * 8) + UNITS * kWideTableFloats;
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
     float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [4]: exp2(alpha[Q-1]); [8..8+QB): log2-decay across block lb
     T *const xs = xs_all + fused_scan_xtile_base(Q, ul);
@@ -247,6 +251,24 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
         }
         block_sync_lds();  // tiles, operand fragments and tables are visible
         const float a_end = blk_s[4];  // exp2(alpha[Q-1])
+        // ---- the tile's scores, once per workgroup: block g = sb + lb, (0,0), (0,1), (1,1), by the first waves of three
+        // units (which have one score block to apply in phase 1 where the second waves have two) ----
+        if (wave < 3) {
+            // (the wave index hidden from the compiler: it would keep these sixteen addresses, which differ from the
+            // ones every wave uses by a wave-uniform offset only, in registers of their own across the tile loop)
+            int pw = wave;
+            asm volatile("" : "+s"(pw));
+            const int psb = pw == 2 ? 1 : 0, plb = pw == 0 ? 0 : 1;
+            f32x16 sc = {0};
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk)
+                sc = mma32(BT::split_frag(Bs + psb * 32 * N, r, 16 * kk + 4 * half), BT::split_frag(Cs + plb * 32 * N, r, 16 * kk + 4 * half), sc);
+            float *gd = G_s + pw * 1024 + lane * 4;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<float4 *>(gd + q * 256) = make_float4(sc[4 * q], sc[4 * q + 1], sc[4 * q + 2], sc[4 * q + 3]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         // the next tile's inputs: requested here, in flight during both phases, stored to LDS at the top of the next tile
         if (c + 1 < s.nc) prefetch(c + 1);
         __builtin_amdgcn_sched_barrier(0);  // (left alone, the scheduler moves the loads down to where their values are used)
@@ -274,6 +296,7 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
             // (the readout's fragments are out of the registers before the score blocks' are requested: with two waves
             // on the SIMD the other wave covers the wait, and both sets at once do not fit)
             __builtin_amdgcn_sched_barrier(0);
+            block_sync_lds();  // the three blocks of scores are in LDS
             const float *F_row = F_s + lb * Q;
             auto make_m = [&](const f32x16 &sc, const float4 (&fv)[4], bool masked, Frag<T>(&mh)[2], Frag<T>(&ml)[2]) {
 #pragma unroll
@@ -297,12 +320,18 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
             auto block = [&](auto sbc, auto diagc) {
                 constexpr int sb = decltype(sbc)::value;
                 constexpr bool diag = decltype(diagc)::value;
-                Frag<T> Bf[NK];
+                f32x16 sc;
+                {
+                    const float *gs = G_s + (sb + lb) * 1024 + lane * 4;
 #pragma unroll
-                for (int kk = 0; kk < NK; ++kk) Bf[kk] = BT::split_frag(Bs, sb * 32 + r, 16 * kk + 4 * half);
-                f32x16 sc = {0};
-#pragma unroll
-                for (int kk = 0; kk < NK; ++kk) sc = mma32(Bf[kk], Cf[kk], sc);
+                    for (int q = 0; q < 4; ++q) {
+                        const float4 t = *reinterpret_cast<const float4 *>(gs + q * 256);
+                        sc[4 * q] = t.x;
+                        sc[4 * q + 1] = t.y;
+                        sc[4 * q + 2] = t.z;
+                        sc[4 * q + 3] = t.w;
+                    }
+                }
                 Frag<T> xf[2];
 #pragma unroll
                 for (int j = 0; j < 2; ++j) xf[j] = XT::frag(xs, sb * 32 + 16 * j + 4 * half, 8, 0, lane);
