@@ -35,9 +35,11 @@ constexpr int f32_table_floats() { return 6 * kFloatTile + 16; }
 // LDS read (whose two offsets are multiples of 512 bytes) reaches from one term into another -- the compiler
 // would pair reads of different terms that way and then move the halves of every fragment into place
 constexpr int f32_bcterm_elems(int N) { return kFloatTile * N + 8; }
+// ... and the tile's scores B . C^T, which the workgroup's eight units share (one group's B and C), as two partial
+// sums over half of the state dimension each, in the accumulator's layout ([half][quarter][lane] 16 bytes)
 constexpr size_t fused_scan_f32_lds_bytes(int N, int waves) {
     return (size_t)2 * 3 * f32_bcterm_elems(N) * 2 + (size_t)waves * 3 * f32_xterm_elems() * 2 +
-           (size_t)waves * f32_xfloat_elems() * 4 + (size_t)waves * f32_table_floats() * 4;
+           (size_t)waves * f32_xfloat_elems() * 4 + (size_t)waves * f32_table_floats() * 4 + (size_t)2 * 32 * 32 * 4;
 }
 
 // Where unit u's tiles start inside their regions (waves * f32_xterm_elems() bf16 elements per term, waves *
@@ -123,6 +125,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
     T *xt_all = Cs + 3 * TB;               // [3][WAVES][XS]
     float *xf_all = reinterpret_cast<float *>(xt_all + 3 * WAVES * XS);  // [WAVES][XF]
     float *wf = xf_all + WAVES * XF + wave * WF;
+    float *const G_s = xf_all + WAVES * XF + WAVES * WF;  // [2][4][64][4] floats
     T *xt = xt_all + f32_xterm_base(wave);  // term t of this wave's unit: xt + t * WAVES * XS
     float *xf = xf_all + f32_xfloat_base(wave);
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
@@ -281,6 +284,34 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
         if (c + 1 < c_end) prefetch(c + 1);
         block_sync_lds();  // tiles and tables are visible
 
+        // ---- the tile's scores S[s, l] = B_s . C_l, once per workgroup: six products per float product make them a
+        // quarter of a tile's matrix instructions.  Two waves sum half of the state dimension each; every wave adds the
+        // two partial sums where it needs the scores (behind a second barrier, after its state readout) ----
+        if constexpr (!STATES_ONLY) {
+            if (wave < 2) {
+                // (the wave index hidden from the compiler, which would otherwise keep these addresses -- a wave-uniform
+                // offset from the ones every wave uses -- in registers of their own across the tile loop)
+                int pw = wave;
+                asm volatile("" : "+s"(pw));
+                f32x16 part = {0};
+#pragma unroll
+                for (int j = 0; j < NK / 2; ++j) {
+                    const int col = 16 * (pw * (NK / 2) + j) + 4 * half;
+                    Frag3 Bf, Cp;
+#pragma unroll
+                    for (int t = 0; t < 3; ++t) {
+                        Bf.t[t] = BT::split_frag(Bs + t * TB, r, col);
+                        Cp.t[t] = BT::split_frag(Cs + t * TB, r, col);
+                    }
+                    part = mma6(Bf, Cp, part);
+                }
+                float *gd = G_s + pw * 1024 + lane * 4;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<float4 *>(gd + q * 256) = make_float4(part[4 * q], part[4 * q + 1], part[4 * q + 2], part[4 * q + 3]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
         // ---- phase 1: y of this tile from the state entering it ----
         if constexpr (!STATES_ONLY) {
             const bool fast = __builtin_amdgcn_readfirstlane(__float_as_int(span)) <= __float_as_int(kFloatFastSpan);
@@ -302,14 +333,20 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fused_scan_f32_kernel(
                 }
                 acc = mma6(hb.frags(), Cf[kk], acc);
             }
-            // scores S[s, l] = B_s . C_l
-            f32x16 sc = {0};
+            // scores S[s, l] = B_s . C_l: the two partial sums the workgroup shares
+            block_sync_lds();
+            f32x16 sc;
+            {
+                const float *gs = G_s + lane * 4;
 #pragma unroll
-            for (int kk = 0; kk < NK; ++kk) {
-                Frag3 Bf;
-#pragma unroll
-                for (int t = 0; t < 3; ++t) Bf.t[t] = BT::split_frag(Bs + t * TB, r, 16 * kk + 4 * half);
-                sc = mma6(Bf, Cf[kk], sc);
+                for (int q = 0; q < 4; ++q) {
+                    const float4 t0 = *reinterpret_cast<const float4 *>(gs + q * 256);
+                    const float4 t1 = *reinterpret_cast<const float4 *>(gs + 1024 + q * 256);
+                    sc[4 * q] = t0.x + t1.x;
+                    sc[4 * q + 1] = t0.y + t1.y;
+                    sc[4 * q + 2] = t0.z + t1.z;
+                    sc[4 * q + 3] = t0.w + t1.w;
+                }
             }
             Frag3 xfr[2];  // x^T: K order rows 16 j + 4 half + {0..3} and the same + 8
 #pragma unroll
