@@ -7,12 +7,13 @@
 // of one batch row -- belongs to TWO waves on the same SIMD, 256 registers each:
 //   * each holds half of the state (64 of the 128 state columns, 32 accumulator registers) and, in phase 2, adds the
 //     tile's B^T . (w o x) to its half;
-//   * at the top of a tile each splits its half into hi + lo bf16 operand fragments and puts them in LDS, where both
-//     find the whole state in operand form;
-//   * phase 1 is divided by output block: wave 0 of the unit produces the tile's first 32 timesteps (state readout
-//     over all 128 columns, the diagonal score block), wave 1 the second 32 (readout, one block below the diagonal, the
-//     diagonal block) -- so the masked, decayed score tiles, the part of a tile's work that does not shrink with the
-//     state, are each formed once, and no partial sums cross waves.
+//   * the state readout C . H of a tile is divided by the state dimension: each wave splits its own half into hi + lo
+//     bf16 operands in registers and multiplies it by its 64 columns of C for BOTH 32-step output blocks; the partial
+//     sum of the block that is not its own goes to the other wave through LDS (4 KB each way per tile, at the barrier
+//     the workgroup holds anyway; the state's operand form through LDS would be 16 KB written and 32 KB read);
+//   * the rest of phase 1 is divided by output block: wave 0 of the unit produces the tile's first 32 timesteps (the
+//     diagonal score block), wave 1 the second 32 (one block below the diagonal, the diagonal block) -- so the masked,
+//     decayed score tiles, the part of a tile's work that does not shrink with the state, are each formed once.
 // A workgroup is four units (eight waves, two per SIMD: wave w and w + 4 are the two halves of unit w, on SIMD w),
 // sharing the B and C tiles of their (batch, group) as before.  The scan of dt*A and the decay tables of a unit are
 // computed by its first wave for both (250 vector instructions, about what the second wave's extra score block costs).
@@ -28,8 +29,8 @@ namespace ssd {
 namespace {
 
 constexpr int kWideN = 128, kWideNK = 8, kWideUnits = 4, kWideWaves = 8, kWideQ = kOnePassTile, kWideQB = kWideQ / 32;
-// LDS: B and C tiles [Q][128], four x tiles [Q][32], the units' states in operand form ([unit][K step][hi, lo]
-// [lane] 16 bytes), per-unit tables
+// LDS: B and C tiles [Q][128], four x tiles [Q][32], the partial readout sums the two waves of a unit hand each other
+// ([unit][sending wave][quarter][lane] 16 bytes, the accumulator's layout), per-unit tables
 constexpr int kWideTableFloats = (5 + kWideQB) * kWideQ + 16;
 // (the x tiles keep the eight-unit layout's offsets, fused_scan_xtile_base: by the hardware's bank-conflict counter the
 // staging writes of four units are free of conflicts with them, and were not with the second pair of units 128 instead
@@ -38,7 +39,7 @@ constexpr int kWideXArea = kWideUnits * fused_scan_xtile_elems(kWideQ);
 // ... and the tile's three blocks of scores B . C^T, which the workgroup's four units share (one group's B and C): three
 // waves form a block each, in the accumulator's layout ([block][quarter][lane] 16 bytes), and every wave reads its blocks
 constexpr size_t kWideLdsBytes = (size_t)2 * kWideQ * kWideN * 2 + (size_t)kWideXArea * 2 +
-                                 (size_t)kWideUnits * kWideNK * 2 * 64 * 16 + (size_t)kWideUnits * kWideTableFloats * 4 +
+                                 (size_t)kWideUnits * 2 * 32 * 32 * 4 + (size_t)kWideUnits * kWideTableFloats * 4 +
                                  (size_t)3 * 32 * 32 * 4;
 
 template <typename TO>
@@ -66,13 +67,15 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
     T *const Bs = reinterpret_cast<T *>(smem);
     T *const Cs = Bs + Q * N;
     T *const xs_all = Cs + Q * N;
-    T *const hfrag = xs_all + kWideXArea;       // [UNITS][NK][2][64][8]
-    float *const wf = reinterpret_cast<float *>(hfrag + UNITS * NK * 2 * 64 * 8) + ul * kWideTableFloats;  // (per unit)
-    float *const G_s = reinterpret_cast<float *>(hfrag + UNITS * NK * 2 * 64 * 8) + UNITS * kWideTableFloats;
+    // what a unit's two waves hand each other: each one's readout of ITS half of the state for the OTHER's output block,
+    // in the accumulator's layout ([unit][wave of the unit][quarter][lane] 16 bytes)
+    float *const part_all = reinterpret_cast<float *>(xs_all + kWideXArea);
+    float *const wf = part_all + UNITS * 2 * 1024 + ul * kWideTableFloats;  // (per unit)
+    float *const G_s = part_all + UNITS * 2 * 1024 + UNITS * kWideTableFloats;
     float *ah_s = wf, *alo_s = wf + Q, *dt_s = wf + 2 * Q, *w_s = wf + 3 * Q, *E_s = wf + 4 * Q, *F_s = wf + 5 * Q;
     float *blk_s = wf + (5 + QB) * Q;  // [0..QB): exp2(alpha[32 lb]); [4]: exp2(alpha[Q-1]); [8..8+QB): log2-decay across block lb
     T *const xs = xs_all + fused_scan_xtile_base(Q, ul);
-    T *const hf_unit = hfrag + (size_t)ul * NK * 2 * 64 * 8;
+    float *const part_unit = part_all + ul * 2 * 1024;
 
     // ---- which units this workgroup owns ----
     const int PBn = s.P / 32, HG = s.H / s.G;
@@ -205,18 +208,6 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
             *reinterpret_cast<uint2 *>(xs_all + xw[0] + u * XRP * 32) = make_uint2(xq[u].x, xq[u].y);
             *reinterpret_cast<uint2 *>(xs_all + xw[1] + u * XRP * 32) = make_uint2(xq[u].z, xq[u].w);
         }
-        // ---- this half of the state entering the tile, in operand form, for both waves of the unit ----
-#pragma unroll
-        for (int k4 = 0; k4 < 2 * HNB; ++k4) {  // K step 4 role + k4: block k4 / 2 of the half, accumulator rows 8 (k4 % 2) ..
-            FragBits fh, fl;
-            float sv[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) sv[i] = st[k4 / 2][8 * (k4 % 2) + i];
-            split8_keep(sv, fh.u, fl.u);
-            T *dst = hf_unit + ((size_t)(4 * role + k4) * 2) * 64 * 8 + lane * 8;
-            *reinterpret_cast<uint4 *>(dst) = make_uint4(fh.u[0], fh.u[1], fh.u[2], fh.u[3]);
-            *reinterpret_cast<uint4 *>(dst + 64 * 8) = make_uint4(fl.u[0], fl.u[1], fl.u[2], fl.u[3]);
-        }
         // ---- scan of dt*A over the tile and the decay tables: the unit's first wave, for both (the second has one
         // more score block in phase 1, about as much work) ----
         if (role == 0) {
@@ -279,24 +270,48 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
             const int l = lb * 32 + r;
             // non-negative floats order like their bit patterns: a scalar compare
             const bool fast = __builtin_amdgcn_readfirstlane(__float_as_int(blk_s[8 + lb])) <= __float_as_int(kFastDiagSpan);
-            Frag<T> Cf[NK];
+            // State readout, divided by the state dimension: this wave holds columns 64 role .. + 63 of the state and reads
+            // out both output blocks over them -- its own block's sum stays in registers, the other block's goes to LDS
+            // for the unit's other wave, which does the same for its half.  (A readout of the own block over the whole
+            // state needs the other half in operand form: 16 KB written and 32 KB read per unit and tile, where the
+            // partial sums are 4 KB each way.)
+            f32x16 acc = {0}, oth = {0};
 #pragma unroll
-            for (int kk = 0; kk < NK; ++kk) Cf[kk] = BT::split_frag(Cs, l, 16 * kk + 4 * half);
-            f32x16 acc = {0};
+            for (int k4 = 0; k4 < NK / 2; ++k4) {
+                const int col = 16 * (4 * role + k4) + 4 * half;
+                const Frag<T> Cown = BT::split_frag(Cs, l, col), Coth = BT::split_frag(Cs, (1 - lb) * 32 + r, col);
+                FragBits fh, fl;
+                float sv[8];
 #pragma unroll
-            for (int kk = 0; kk < NK; ++kk) {
-                Frag<T> Hh, Hl;
-                const T *src = hf_unit + ((size_t)kk * 2) * 64 * 8 + lane * 8;
-                Hh.v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(src));
-                Hl.v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(src + 64 * 8));
-                acc = mma32(Hh, Cf[kk], acc);
-                acc = mma32(Hl, Cf[kk], acc);
+                for (int i = 0; i < 8; ++i) sv[i] = st[k4 / 2][8 * (k4 % 2) + i];
+                split8_keep(sv, fh.u, fl.u);
+                const Frag<T> Hh = fh.frag(), Hl = fl.frag();
+                acc = mma32(Hh, Cown, acc);
+                oth = mma32(Hh, Coth, oth);
+                acc = mma32(Hl, Cown, acc);
+                oth = mma32(Hl, Coth, oth);
+            }
+            {
+                float *pd = part_unit + role * 1024 + lane * 4;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<float4 *>(pd + q * 256) = make_float4(oth[4 * q], oth[4 * q + 1], oth[4 * q + 2], oth[4 * q + 3]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            block_sync_lds();  // the unit's other partial sum, and the three blocks of scores, are in LDS
+            {
+                const float *ps = part_unit + (1 - role) * 1024 + lane * 4;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 t = *reinterpret_cast<const float4 *>(ps + q * 256);
+                    acc[4 * q] += t.x;
+                    acc[4 * q + 1] += t.y;
+                    acc[4 * q + 2] += t.z;
+                    acc[4 * q + 3] += t.w;
+                }
             }
             acc = acc * blk_s[lb];
-            // (the readout's fragments are out of the registers before the score blocks' are requested: with two waves
-            // on the SIMD the other wave covers the wait, and both sets at once do not fit)
             __builtin_amdgcn_sched_barrier(0);
-            block_sync_lds();  // the three blocks of scores are in LDS
             const float *F_row = F_s + lb * Q;
             auto make_m = [&](const f32x16 &sc, const float4 (&fv)[4], bool masked, Frag<T>(&mh)[2], Frag<T>(&ml)[2]) {
 #pragma unroll
