@@ -212,6 +212,63 @@ def test_head_sums_taken_on_chip(w, with_D, with_init, with_dfinal):
     run_case(w, seed=21, with_D=with_D, with_init=with_init, with_dfinal=with_dfinal)
 
 
+@pytest.mark.parametrize("w", [
+    Workload("bwd_far_anchors_wide", 192, 64 * 19 + 5, 8, 32, 64, 1, 64, dtype="bf16", init_std=0.5),    # 20 tiles: runs of 8, 8, 4
+    Workload("bwd_far_anchors_narrow", 192, 64 * 10 + 33, 8, 32, 32, 1, 64, dtype="bf16", init_std=0.5),  # 11 tiles: 8, 3
+    Workload("bwd_far_anchors_whole_runs", 192, 64 * 16, 8, 32, 64, 1, 64, dtype="bf16", init_std=0.5),
+    Workload("bwd_far_anchors_strong_decay", 192, 64 * 12 + 1, 8, 32, 64, 1, 64, dtype="bf16", a_log_range=(0.01, 64.0),
+             dt_law="mixture", x_law="student-t3"),
+], ids=lambda w: w.name)
+def test_decay_gradient_between_far_anchors(w):
+    """Where the adjoint scan carries the row products, the two transposed scans' states meet only at every eighth
+    tile boundary, and the decay gradient sums its per-step terms over runs of up to 512 steps: sequences of more than
+    eight tiles, with a ragged last run and a ragged last tile, restarts on tile and run borders, an initial state and
+    a gradient on the final state; both kinds of transposed scan (the one that keeps its tile states runs forward in
+    time for a 64-wide state, backward for a 32-wide one).  Rows against the oracle; dA through additivity over the
+    batch rows (a batch of three takes the general path, whose anchors stand at every tile)."""
+    dev = make_inputs(w, seed=6, device="cuda")
+    m = (np.random.default_rng(2).random((w.batch, w.seqlen)) < 0.004).astype(np.uint8)
+    m[0] = 0
+    for t in (63, 64, 511, 512, 513, 1023, 1024, w.seqlen - 1):   # tile and run borders
+        if t < w.seqlen:
+            m[1, t] = 1
+    m[2, 0] = 1
+    g = torch.Generator(device="cuda").manual_seed(4)
+    dy = torch.randn(dev["x"].shape, generator=g, device="cuda").to(torch.bfloat16)
+    dfin = torch.randn(w.batch, w.nheads, w.headdim, w.dstate, generator=g, device="cuda")
+    reset = torch.from_numpy(m).cuda()
+    got = ssd_chunk_scan_backward(dev["x"], dev["dt"], dev["A"], dev["B"], dev["C"], dev["D"], dy, chunk=w.chunk,
+                                  initial_states=dev["init"], dfinal_states=dfin, need_dinitial_states=True, reset=reset)
+    rows = [0, 1, 2]
+    sub = lambda t: None if t is None else t[rows].contiguous()
+    ref = bwd.ssd_backward_sequential(np64(sub(dev["x"])), np64(sub(dev["dt"])), np64(dev["A"]), np64(sub(dev["B"])),
+                                      np64(sub(dev["C"])), np64(dev["D"]), np64(sub(dev["init"])), np64(sub(dy)),
+                                      np64(sub(dfin)), reset=m[rows])
+    for k_out, k_ref in (("dx", "dx"), ("ddt", "ddt"), ("dB", "dB"), ("dC", "dC"), ("dinitial_states", "dinit")):
+        check(got[k_out][rows], ref[k_ref], torch.bfloat16, f"{w.name} {k_out}")
+    # the same rows as a batch of their own: the general path.  ddt agrees to the bf16 rounding of either.
+    small = ssd_chunk_scan_backward(sub(dev["x"]), sub(dev["dt"]), dev["A"], sub(dev["B"]), sub(dev["C"]), dev["D"], sub(dy),
+                                    chunk=w.chunk, initial_states=sub(dev["init"]), dfinal_states=sub(dfin),
+                                    need_dinitial_states=True, reset=reset[rows].contiguous())
+    check(small["dA"], ref["dA"], torch.bfloat16, f"{w.name} dA (general path)", ref["dA_scale"])
+    a, b_ = got["ddt"][rows].double(), small["ddt"].double()
+    rms = b_.pow(2).mean().sqrt().item()
+    assert ((a - b_).abs() <= 2.0 ** -7 * b_.abs() + 1e-3 * rms).all()
+    # dA over the whole batch = the sum of dA over its halves (each half still takes the path under test)
+    half = w.batch // 2
+    total = torch.zeros_like(got["dA"], dtype=torch.float64)
+    for i in range(2):
+        sl = slice(i * half, (i + 1) * half)
+        c = lambda t: None if t is None else t[sl].contiguous()
+        part = ssd_chunk_scan_backward(c(dev["x"]), c(dev["dt"]), dev["A"], c(dev["B"]), c(dev["C"]), dev["D"], c(dy),
+                                       chunk=w.chunk, initial_states=c(dev["init"]), dfinal_states=c(dfin), reset=c(reset))
+        total += part["dA"].double()
+        if i == 0:
+            assert torch.equal(part["ddt"][rows], got["ddt"][rows])
+    scale = got["dA"].double().abs().max().item()
+    assert (got["dA"].double() - total).abs().max().item() <= 1e-5 * scale
+
+
 def test_restarts_on_the_one_pass_adjoint_scan():
     """Enough bf16 sequences for the adjoint recurrence to take the one-pass kernel: rows against the oracle."""
     w = Workload("bwd_reset_onepass", 96, 200, 8, 32, 64, 1, 128, dtype="bf16")

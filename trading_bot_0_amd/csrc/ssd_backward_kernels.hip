@@ -386,20 +386,30 @@ __global__ __launch_bounds__(256) void bwd_ddt_kernel(const T *__restrict__ dt, 
 // contiguous run of 64 elements of a [B, L, H] array (a wave per head touches a cache line per lane instead).
 // NP: the pieces of C . yC per element when they are 1..4 (then e1 holds the (e1, dd) pairs and the loads are
 // straight-line code); 0: any other form of the inputs, through conditions uniform over the launch.
+// stride (a power of two, at most kDdtMaxStride): the anchors stand at every stride-th chunk boundary and at the end
+// of the sequence only.  The chunks between two of them are a run; a run's waves sit in one workgroup (of
+// max(4, stride) waves: whole runs), hand each other their chunks' sums of u through LDS, and spread the run's
+// mismatch over all of its steps.
+constexpr int kDdtMaxStride = 8;
 template <typename T, int NH, int NP>
-__global__ __launch_bounds__(256) void bwd_ddt_heads_kernel(const T *__restrict__ dt, const float *__restrict__ A,
-                                                            const float *__restrict__ e1, const float *__restrict__ u,
-                                                            const float *__restrict__ dd, const double *__restrict__ anchor,
-                                                            T *__restrict__ ddt, double *__restrict__ dA_part,
-                                                            double *__restrict__ dD_part, ScanShape s,
-                                                            const float *__restrict__ parts, int nparts,
-                                                            const unsigned char *__restrict__ reset, int raw_anchors) {
+__global__ __launch_bounds__(64 * kDdtMaxStride) void bwd_ddt_heads_kernel(
+    const T *__restrict__ dt, const float *__restrict__ A, const float *__restrict__ e1, const float *__restrict__ u,
+    const float *__restrict__ dd, const double *__restrict__ anchor, T *__restrict__ ddt, double *__restrict__ dA_part,
+    double *__restrict__ dD_part, ScanShape s, const float *__restrict__ parts, int nparts,
+    const unsigned char *__restrict__ reset, int raw_anchors, int stride) {
     constexpr int TL = 64 / NH, R = 64 / TL;
-    const int lane = threadIdx.x & 63;
-    const long long id = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (id >= (long long)s.B * s.nc) return;
-    const int c = (int)(id % s.nc);
-    const long long b = id / s.nc;
+    __shared__ double run_sums[kDdtMaxStride][NH];  // [wave of the workgroup][head]: the chunk's sum of u
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int runs = (s.nc + stride - 1) / stride;  // per sequence
+    const long long run_id = (long long)blockIdx.x * ((blockDim.x >> 6) / stride) + wave / stride;
+    const int cw = wave % stride;  // this wave's chunk of the run
+    const int run = (int)(run_id % runs);
+    // a wave past the last chunk (of its run, or of the launch) walks the last chunk of its sequence and keeps nothing:
+    // every wave of a workgroup reaches the barrier below
+    const long long b = min(run_id / runs, (long long)s.B - 1);
+    const bool live = run_id < (long long)s.B * runs && run * stride + cw < s.nc;
+    const int c = min(run * stride + cw, s.nc - 1);
+    const long long id = b * s.nc + c;
     const int h = lane % NH, tl = lane / NH;
     const int t0 = c * 64, len = min(64, s.L - t0);
     const size_t row0 = ((size_t)b * s.L + t0) * NH;  // this chunk's first element of a [B, L, H] array
@@ -440,12 +450,13 @@ __global__ __launch_bounds__(256) void bwd_ddt_heads_kernel(const T *__restrict_
     unsigned char an_rs[2];
     const int ra = max(raw_anchors, 1);  // (the launcher keeps raw_anchors within kMaxPieces)
     const unsigned char *rs_or_any = reset != nullptr ? reset : reinterpret_cast<const unsigned char *>(dt);
+    const int run_c[2] = {run * stride, min(run * stride + stride, s.nc)};  // the chunk boundaries the run lies between
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
-        const size_t at = ((size_t)b * (s.nc + 1) + c + e) * NH + h;
+        const size_t at = ((size_t)b * (s.nc + 1) + run_c[e]) * NH + h;
 #pragma unroll
         for (int i = 0; i < kMaxPieces; ++i) an_q[e][i] = anchor[at * ra + min(i, ra - 1)];
-        const size_t t = (size_t)b * s.L + (size_t)min(c + e, s.nc - 1) * 64;
+        const size_t t = (size_t)b * s.L + (size_t)min(run_c[e], s.nc - 1) * 64;
         an_dt[e] = dt[t * NH + h];
         an_rs[e] = rs_or_any[t];
     }
@@ -454,7 +465,7 @@ __global__ __launch_bounds__(256) void bwd_ddt_heads_kernel(const T *__restrict_
 #pragma unroll
         for (int i = 0; i < kMaxPieces; ++i) v += i < ra ? an_q[e][i] : 0.0;
         const double first = (reset != nullptr && an_rs[e] != 0) ? 0.0 : exp((double)(float)an_dt[e] * a);
-        return (raw_anchors != 0 && c + e < s.nc) ? v * first : v;
+        return (raw_anchors != 0 && run_c[e] < s.nc) ? v * first : v;
     };
     const double q0 = anchor_at(0), q1 = anchor_at(1);
     float e1v[R], ddv[R], dtv[R];
@@ -496,13 +507,29 @@ __global__ __launch_bounds__(256) void bwd_ddt_heads_kernel(const T *__restrict_
         before[r] = carry + v - uv[r];
         carry += __shfl(v, 64 - NH + h, 64);
     }
-    const double mismatch = q0 - carry - q1;
+    // the run: the sum of u over its earlier chunks and over all of them, its steps before this chunk and in all
+    double run_before = 0.0, run_total = carry;
+    int steps_before = 0, run_len = len;
+    if (stride > 1) {  // (uniform)
+        if (tl == 0) run_sums[wave][h] = live ? carry : 0.0;
+        __syncthreads();
+        run_total = 0.0;
+        for (int k = 0; k < stride; ++k) {
+            const double v = run_sums[wave - cw + k][h];
+            run_before += k < cw ? v : 0.0;
+            run_total += v;
+        }
+        steps_before = cw * 64;
+        run_len = min(stride * 64, s.L - run * stride * 64);
+    }
+    if (!live) return;
+    const double mismatch = q0 - run_total - q1;
     double da = 0.0, sdd = 0.0;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int t = r * TL + tl;
         if (t < len) {
-            const double q = q0 - before[r] - mismatch * (double)t / (double)len;
+            const double q = q0 - run_before - before[r] - mismatch * (double)(steps_before + t) / (double)run_len;
             ddt[row0 + (size_t)r * 64 + lane] = (T)(float)((double)e1v[r] + a * q);
             da += (double)dtv[r] * q;
             sdd += (double)ddv[r];
@@ -636,15 +663,20 @@ hipError_t anchors_t(const ScanShape &s, const void *dt, const float *A, const f
 template <typename T>
 hipError_t ddt_t(const ScanShape &s, const void *dt, const float *A, const float *e1, const float *u, const float *dd,
                  const double *anchor, void *ddt, double *dA_part, double *dD_part, const float *parts, int nparts,
-                 const unsigned char *reset, int raw_anchors, hipStream_t st) {
+                 const unsigned char *reset, int raw_anchors, int anchor_stride, hipStream_t st) {
     if (s.Q > 64) return hipErrorInvalidValue;  // one pass of the wave per chunk
-    if (s.Q == 64 && (s.H == 4 || s.H == 8 || s.H == 16) && raw_anchors <= 4) {
-        const long long chunks = (long long)s.B * s.nc;
-        const dim3 grid((unsigned)((chunks + 3) / 4)), block(256);
+    if (anchor_stride < 1 || (anchor_stride & (anchor_stride - 1)) != 0 || anchor_stride > kDdtMaxStride ||
+        (anchor_stride > 1 && !bwd_ddt_anchor_stride_supported(s, raw_anchors)))
+        return hipErrorInvalidValue;
+    if (bwd_ddt_anchor_stride_supported(s, raw_anchors)) {
+        const int waves = max(4, anchor_stride);  // per workgroup: whole runs
+        const long long runs = (long long)s.B * ((s.nc + anchor_stride - 1) / anchor_stride);
+        const long long per_group = waves / anchor_stride;
+        const dim3 grid((unsigned)((runs + per_group - 1) / per_group)), block(64 * waves);
 #define SSD_DDT_HEADS_NP(NH, NP)                                                                                       \
     bwd_ddt_heads_kernel<T, NH, NP><<<grid, block, 0, st>>>(static_cast<const T *>(dt), A, e1, u, dd, anchor,           \
                                                             static_cast<T *>(ddt), dA_part, dD_part, s, parts, nparts,   \
-                                                            reset, raw_anchors)
+                                                            reset, raw_anchors, anchor_stride)
 #define SSD_DDT_HEADS(NH)                                           \
     do {                                                            \
         if (parts != nullptr && nparts == 1) SSD_DDT_HEADS_NP(NH, 1); \
@@ -728,11 +760,18 @@ hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, con
                  : anchors_t<float>(s, dt, A, fwd_prev, rev_prev, rev_final, init_t, fwd_final, dfin_t, reset, anchor, st);
 }
 
+bool bwd_ddt_anchor_stride_supported(const ScanShape &s, int raw_anchors) {  // (the kernel with a group's heads per wave)
+    return s.Q == 64 && (s.H == 4 || s.H == 8 || s.H == 16) && raw_anchors <= 4;
+}
+
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
                           const float *dd, const double *anchor, void *ddt, double *dA_part, double *dD_part,
-                          hipStream_t st, const float *parts, int nparts, const unsigned char *reset, int raw_anchors) {
-    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, reset, raw_anchors, st)
-                 : ddt_t<float>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, reset, raw_anchors, st);
+                          hipStream_t st, const float *parts, int nparts, const unsigned char *reset, int raw_anchors,
+                          int anchor_stride) {
+    return dtype ? ddt_t<__bf16>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, reset, raw_anchors,
+                                 anchor_stride, st)
+                 : ddt_t<float>(s, dt, A, e1, u, dd, anchor, ddt, dA_part, dD_part, parts, nparts, reset, raw_anchors,
+                                anchor_stride, st);
 }
 
 hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,

@@ -529,10 +529,18 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         const float *g = j == 0 ? an.other_final : j == s.nc ? an.other_init : an.other_tiles;
         zero = g == nullptr;
         const bool tiles = zero || (j != 0 && j != s.nc);
-        const size_t bh = tiles ? ((size_t)b * s.nc + (zero ? 0 : s.nc - j)) * s.H + h : (size_t)b * s.H + h;
+        // (the other scan kept the states entering its tiles phase, phase + stride, ..: anchor_here says which j meet one)
+        const int kept = s.nc > an.phase ? (s.nc - 1 - an.phase) / an.stride + 1 : 1;
+        const size_t bh = tiles ? ((size_t)b * kept + (zero ? 0 : (s.nc - j - an.phase) / an.stride)) * s.H + h
+                                : (size_t)b * s.H + h;
         return (zero ? an.other_tiles : g) + (bh * s.P + pb * 32 + (lane0 & 31)) * N + 4 * (lane0 >> 5);
     };
     // one slice at a time, so that at most one slice of the other scan's state is held in registers
+    // whether the two scans meet where this scan's tile j starts (j = nc: where it ends)
+    auto anchor_here = [&](int j) {
+        const int o = s.nc - j - an.phase;  // the other scan's tile that starts there, counted from its first kept one
+        return j == 0 || j == s.nc || (o >= 0 && o % an.stride == 0);
+    };
     auto load_other = [&](const float *g, int sl, float4 (&gq)[NB][4]) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
@@ -576,7 +584,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         const int t0 = c * Q;
         const int rows = min(Q, s.L - t0);
         // the state entering every tile, for a caller that needs it (the backward pass): [B, nc, H, P, N]
-        if (tile_states) store_state(tile_states + (((size_t)b * s.nc + c) * s.H + h) * s.P * N);
+        // (of every an.stride-th tile from an.phase on, where the backward pass's other scan asks for fewer)
+        if (tile_states && c >= an.phase && (c - an.phase) % an.stride == 0) {
+            const int kept = (s.nc - 1 - an.phase) / an.stride + 1;
+            store_state(tile_states + (((size_t)b * kept + (c - an.phase) / an.stride) * s.H + h) * s.P * N);
+        }
         if (!kTwoSets) block_sync_lds();  // every wave is done reading the previous chunk's tiles
         // ---- registers -> LDS tiles ----
         // where the pieces go: the swizzle repeats every 32 rows, so all passes of a thread share the
@@ -1008,8 +1020,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         float4 gq[ANCH ? NB : 1][4];
         bool gzero = false;
         const float *gnext = nullptr;
+        const bool anchor_next = ANCH && an.out != nullptr && anchor_here(c + 1);
         if constexpr (ANCH) {
-            if (an.out != nullptr) {
+            if (anchor_next) {
                 gnext = adjoint_state(c + 1, gzero);
                 load_other(gnext, 0, gq);
             }
@@ -1068,7 +1081,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             }
         }
         if constexpr (ANCH) {
-            if (an.out != nullptr) {
+            if (anchor_next) {
                 // (the other scan's values are used from here on, not before: left alone, the compiler converts them to
                 // float64 right behind their loads, in front of phase 2, and the wave waits for them there)
                 auto pin = [&](float4 (&q)[NB][4]) {

@@ -30,13 +30,17 @@ hipError_t launch_transposed_scan(const ScanShape &sT, bool adjoint, const void 
     t.nc = (sT.L + kOnePassTile - 1) / kOnePassTile;
     if (an.out != nullptr && adjoint != wide(sT)) return hipErrorInvalidValue;
     if (an.out != nullptr && an.other_tiles == nullptr) return hipErrorInvalidValue;  // (the kernel reads it without asking)
+    if (an.stride < 1 || an.phase < 0 || an.phase >= an.stride) return hipErrorInvalidValue;
+    ScanAnchors keep;  // the scan that runs first: which of its tile states it keeps
+    keep.stride = an.stride;
+    keep.phase = an.phase;
     if (wide(sT))
         return adjoint ? fused_launch_transposed<__bf16, 7>(t, x, dt, A, Bm, Cm, nullptr, init, reset, out, final_states,
                                                             tile_states, nullptr, an, st)
                        : fused_launch_transposed<__bf16, 6>(t, x, dt, A, Bm, Cm, aux, init, reset, out, final_states,
-                                                            tile_states, parts, ScanAnchors{}, st);
+                                                            tile_states, parts, keep, st);
     return adjoint ? fused_launch_transposed<__bf16, 4>(t, x, dt, A, Bm, Cm, nullptr, init, reset, out, final_states,
-                                                        tile_states, nullptr, ScanAnchors{}, st)
+                                                        tile_states, nullptr, keep, st)
                    : fused_launch_transposed<__bf16, 3>(t, x, dt, A, Bm, Cm, aux, init, reset, out, final_states,
                                                         tile_states, parts, an, st);
 }

@@ -163,9 +163,15 @@ hipError_t launch_block_pre_bwd(const BlockShape &s, int dtype, const void *zxbc
 // states at the start of forward tile k (k = nc: the end of the sequence): its own state entering its tile j with
 // other_tiles[b, nc - j, h] for 0 < j < nc, its initial state with other_final (zero without an initial state), its
 // final state with other_init (zero when NULL).  out [B, nc+1, H, P/32], float64.
+// stride > 1: the two scans meet at every stride-th tile boundary of forward time only (k = 0, stride, 2 stride, ..
+// and nc); the other entries of `out` are left alone.  The scan that runs first then keeps only the states entering
+// its tiles c = phase, phase + stride, .. in tile_states [B, (nc - 1 - phase) / stride + 1, H, P, N] (phase = 0 for
+// the forward scan, nc % stride for the adjoint one, whose tile c starts where forward tile nc - c ends), and is
+// given stride and phase in `an` as well (its `out` stays NULL).
 struct ScanAnchors {
     const float *other_tiles = nullptr, *other_final = nullptr, *other_init = nullptr;
     double *out = nullptr;
+    int stride = 1, phase = 0;
 };
 bool transposed_scan_anchors_in_adjoint(const ScanShape &sT);
 bool transposed_scan_supported(const ScanShape &sT, int x_groups);
@@ -225,10 +231,14 @@ hipError_t launch_bwd_anchors(const ScanShape &s, int dtype, const void *dt, con
 // With raw_anchors > 0, anchor holds that many pieces per (b, c, h) ([B, nc+1, H, raw_anchors], as ScanAnchors
 // writes them) of the two states' inner product, and the first step's decay exp(dt A) -- zero where `reset` marks
 // the chunk's first step -- is applied here.
+// anchor_stride > 1 (a power of two up to 8, where bwd_ddt_anchor_stride_supported): q is known only at every
+// anchor_stride-th chunk boundary and at the end of the sequence, the u are summed over the chunks in between and
+// their mismatch is spread over all of those steps.
+bool bwd_ddt_anchor_stride_supported(const ScanShape &s, int raw_anchors);
 hipError_t launch_bwd_ddt(const ScanShape &s, int dtype, const void *dt, const float *A, const float *e1, const float *u,
                           const float *dd, const double *anchor, void *ddt, double *dA_part, double *dD_part,
                           hipStream_t stream, const float *parts = nullptr, int nparts = 0,
-                          const unsigned char *reset = nullptr, int raw_anchors = 0);
+                          const unsigned char *reset = nullptr, int raw_anchors = 0, int anchor_stride = 1);
 // dA[h], dD[h] (NULL allowed) = the sums over batch and chunks of the parts
 hipError_t launch_bwd_head_sums(const ScanShape &s, const double *dA_part, const double *dD_part, float *dA, float *dD,
                                 hipStream_t stream);
