@@ -157,15 +157,16 @@ constexpr size_t fused_scan_lds_bytes(int N, int Q, int waves) {
 // KIND 6 and 7 are 3 and 4 for a 64-wide transposed state (dstate 64) with both 32-column slices of a head in one
 // wave: the head's masked, decayed score tile -- the part of a tile's work that does not shrink with the state's
 // width -- and its B and C tiles are then formed and staged once instead of once per slice.  Their LDS holds two x
-// tiles and two tiles of the second operand of C . y, all tiles 8 elements apart instead of 16 to make room, and a
+// tiles and two tiles of the second operand of C . y, 4 elements apart (a staging write puts 8-byte halves of one row
+// into both tiles of a pair: one takes the even 8-byte slots of the row's banks, the other the odd ones), and a
 // float tile per wave of 32 rows only: the workgroup writes its sums out after every block of 32 rows.  That tile's
 // rows are 64 floats with their 16-byte pieces XOR-swizzled by the row's low four bits, so that a lane's four
 // consecutive columns go out and come back as one 16-byte access and 16 consecutive rows of one logical piece
 // cover 256 bytes of banks.
-constexpr int wide_transposed_tile_elems(int Q) { return Q * 32 + 8; }
+constexpr int wide_transposed_tile_elems(int Q) { return Q * 32 + 4; }
 constexpr size_t wide_transposed_scan_lds_bytes(int Q) {
-    return (size_t)(2 * 8 + 4) * wide_transposed_tile_elems(Q) * 2 + (size_t)8 * ((5 + Q / 32) * Q * 4 + 64) +
-           (size_t)8 * 32 * 64 * 4;
+    return (size_t)(2 * 8) * fused_scan_xtile_elems(Q) * 2 + (size_t)4 * wide_transposed_tile_elems(Q) * 2 +
+           (size_t)8 * ((5 + Q / 32) * Q * 4 + 64) + (size_t)8 * 32 * 64 * 4;
 }
 constexpr size_t transposed_scan_lds_bytes(int Q) {
     return (size_t)(2 * 8 + 2) * fused_scan_xtile_elems(Q) * 2 + (size_t)8 * ((5 + Q / 32) * Q * 4 + 64) +
@@ -220,9 +221,12 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
     constexpr bool kTwoSets = !TR && KIND != 5 && fused_scan_two_tile_sets(N, WAVES);
     constexpr int SETS = kTwoSets ? 2 : 1;
     T *tiles = reinterpret_cast<T *>(smem);
-    T *const Bs0 = TR ? tiles + wave * XS : tiles;
-    T *const Cs0 = TR ? tiles + (WAVES + wave) * XS : tiles + SETS * Q * N;
-    T *const xs_all0 = TR ? tiles + 2 * WAVES * XS : tiles + 2 * SETS * Q * N;
+    // (transposed: the heads' B tiles, then their C tiles, each set laid out like the forward's x tiles -- the staging
+    // writes are the same, a row of every head's tile at once -- then the shared tiles, XS apart)
+    constexpr int TRB = WAVES * fused_scan_xtile_elems(Q);  // the eight heads' B (or C) tiles
+    T *const Bs0 = TR ? tiles + fused_scan_xtile_base(Q, wave) : tiles;
+    T *const Cs0 = TR ? tiles + TRB + fused_scan_xtile_base(Q, wave) : tiles + SETS * Q * N;
+    T *const xs_all0 = TR ? tiles + 2 * TRB : tiles + 2 * SETS * Q * N;
     T *aux_s = xs_all0 + SL * XS;  // transposed only (one tile per slice, behind the x tiles)
     float *wf0 = reinterpret_cast<float *>(TR ? xs_all0 + 2 * SL * XS : xs_all0 + SETS * WAVES * XS);
     float *wf = wf0 + wave * ((5 + QB) * Q + 16);
@@ -600,7 +604,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
             bw[hf] = BT::off(tw / BPR, (tw % BPR) * 8 + 4 * hf);
 #pragma unroll
             for (int par = 0; par < 2; ++par)
-                xw[par][hf] = (TR ? ((tw % XPR) / 4) * XS : fused_scan_xtile_base(Q, (tw % XPR) / 4)) +
+                xw[par][hf] = fused_scan_xtile_base(Q, (tw % XPR) / 4) +
                               XT::off(tw / XPR + 16 * par, ((tw % XPR) % 4) * 8 + 4 * hf);
         }
         if constexpr (TR) {
@@ -609,8 +613,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
                 T *tb = tiles + xw[u & 1][0] + (u >> 1) * 1024, *tb1 = tiles + xw[u & 1][1] + (u >> 1) * 1024;
                 *reinterpret_cast<uint2 *>(tb) = make_uint2(bq[u].x, bq[u].y);
                 *reinterpret_cast<uint2 *>(tb1) = make_uint2(bq[u].z, bq[u].w);
-                *reinterpret_cast<uint2 *>(tb + WAVES * XS) = make_uint2(cq[u].x, cq[u].y);
-                *reinterpret_cast<uint2 *>(tb1 + WAVES * XS) = make_uint2(cq[u].z, cq[u].w);
+                *reinterpret_cast<uint2 *>(tb + TRB) = make_uint2(cq[u].x, cq[u].y);
+                *reinterpret_cast<uint2 *>(tb1 + TRB) = make_uint2(cq[u].z, cq[u].w);
             }
             if (tw < Q * 4 * SL) {
                 const int col = (tw % (4 * SL)) * 8;
