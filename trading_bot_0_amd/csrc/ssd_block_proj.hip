@@ -89,6 +89,10 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
     // (a block takes CH chunks or one fewer -- 648 columns are 4 x 128 + 136 -- and the last chunk is the only piece
     // of a tile's work under a condition, a uniform one)
     const bool last_chunk = ncols > (CH - 1) * kProjChunk;
+    constexpr int kRing = KS < 8 ? KS : 8;
+    uint4 wq[kRing];  // the next kRing fragments of w
+#pragma unroll
+    for (int ks = 0; ks < kRing; ++ks) wq[ks] = *reinterpret_cast<const uint4 *>(wsm + r * ROWB + half * 16 + ks * 32);
     auto tile_product = [&](int t, const Frag<__bf16>(&uf)[KS]) {
         const unsigned trow = (unsigned)(t * (32 * kProjWaves) + wave * 32);  // the tile's first row within the workgroup's
         const long long m0 = tile_row0(t);
@@ -99,21 +103,34 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
             for (int sub = 0; sub < 2; ++sub) {
                 const int c = c0 + sub;
                 if (c >= CH || (c == CH - 1 && !last_chunk)) break;
+                // the chunk that follows this one (the next tile's first after the last)
+                const int cn = (c + 1 < CH && (c + 1 < CH - 1 || last_chunk)) ? c + 1 : 0;
                 const unsigned char *wb = wsm + (c * kProjChunk + r) * ROWB + half * 16;
+                const unsigned char *wn = wsm + (cn * kProjChunk + r) * ROWB + half * 16;
                 f32x16 acc = {0}, acc_odd = {0};  // two chains of dependent MFMAs instead of one
 #pragma unroll
                 for (int ks = 0; ks < KS; ks += 2) {
                     Frag<__bf16> wf0, wf1;
-                    wf0.v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(wb + ks * 32));
-                    wf1.v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(wb + ks * 32 + 32));
+                    wf0.v = __builtin_bit_cast(bf16x8, wq[ks % kRing]);
+                    wf1.v = __builtin_bit_cast(bf16x8, wq[(ks + 1) % kRing]);
                     acc = mma32(wf0, uf[ks], acc);
                     acc_odd = mma32(wf1, uf[ks + 1], acc_odd);
+                    // ... and the fragments of w kRing K steps further on (in this chunk or the next), each requested
+                    // into the registers of the one just used: kRing / 2 pairs of products lie between a request and
+                    // its use (requested right in front of its use, as the compiler orders them when left alone, every
+                    // pair of products waits out the LDS latency)
+                    const unsigned char *wa = ks + kRing < KS ? wb + kRing * 32 : wn + (kRing - KS) * 32;
+                    wq[ks % kRing] = *reinterpret_cast<const uint4 *>(wa + ks * 32);
+                    wq[(ks + 1) % kRing] = *reinterpret_cast<const uint4 *>(wa + ks * 32 + 32);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 acc = acc + acc_odd;
                 // acc[4 vg + i] = out[m, n0 + 32 c + 8 vg + 4 half + i]
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg)
-                    *reinterpret_cast<uint2 *>(tile + r * kTileRowB + (sub * 32 + 8 * vg + 4 * half) * 2) = make_uint2(
+                    // (rows 8 .. 15 and 24 .. 31 keep the 8-byte halves of every 16-byte piece the other way round: rows
+                    // are 144 bytes apart, so that rows r and r + 8, served together, would otherwise share their banks)
+                    *reinterpret_cast<uint2 *>(tile + r * kTileRowB + (sub * 32 + 8 * vg + 4 * (half ^ ((r >> 3) & 1))) * 2) = make_uint2(
                         pack_bf16x2(acc[4 * vg], acc[4 * vg + 1]), pack_bf16x2(acc[4 * vg + 2], acc[4 * vg + 3]));
             }
             // The tile was written by this wave's other lanes: LDS works a wave's requests off in order, so all that
@@ -123,7 +140,8 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_proj_kernel(const __bf1
 #pragma unroll
             for (int pass = 0; pass < 4; ++pass) {
                 const int row = pass * 8 + (lane >> 3), col = c0 * kProjChunk + (lane & 7) * 8;
-                const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + row * kTileRowB + (lane & 7) * 16);
+                const u32x4 q = *reinterpret_cast<const u32x4 *>(tile + row * kTileRowB + (lane & 7) * 16);
+                const u32x4 v = (pass & 1) ? u32x4{q.z, q.w, q.x, q.y} : q;
                 const bool ok = m0 + row < M && col < ncols;
                 const unsigned off = ((trow + (unsigned)row) * (unsigned)ldo + (unsigned)(n0 + col)) * 2u;
                 __builtin_amdgcn_raw_buffer_store_b128(v, obuf, ok ? off : kBufferDropOffset, 0, 0);
@@ -271,7 +289,7 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_post_proj_kernel(
                     for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
                         for (int vg = 0; vg < 4; ++vg)
-                            *reinterpret_cast<uint2 *>(tile + (r & 15) * kTileRowB + (sub * 32 + 8 * vg + 4 * half) * 2) = make_uint2(
+                            *reinterpret_cast<uint2 *>(tile + (r & 15) * kTileRowB + (sub * 32 + 8 * vg + 4 * (half ^ ((r >> 3) & 1))) * 2) = make_uint2(
                                 pack_bf16x2(acc[sub][4 * vg], acc[sub][4 * vg + 1]), pack_bf16x2(acc[sub][4 * vg + 2], acc[sub][4 * vg + 3]));
                     }
                 }
@@ -280,7 +298,8 @@ __global__ __launch_bounds__(64 * kProjWaves) void block_post_proj_kernel(
 #pragma unroll
                 for (int pass = 0; pass < 2; ++pass) {
                     const int trw = pass * 8 + (lane >> 3), row = rh * 16 + trw, col = c0 * kProjChunk + (lane & 7) * 8;
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + trw * kTileRowB + (lane & 7) * 16);
+                    const u32x4 q = *reinterpret_cast<const u32x4 *>(tile + trw * kTileRowB + (lane & 7) * 16);
+                    const u32x4 v = (pass & 1) ? u32x4{q.z, q.w, q.x, q.y} : q;  // (halves swapped in rows 8 .. 15)
                     const bool ok = m0 + row < M && col < N;
                     const unsigned off = ((trow + (unsigned)row) * (unsigned)ldo + (unsigned)col) * 2u;
                     __builtin_amdgcn_raw_buffer_store_b128(v, obuf, ok ? off : kBufferDropOffset, 0, 0);
