@@ -70,14 +70,14 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # script, so the figures are carried here, keyed by (workload, batch): a run at any other size reports null.
 # Reads come out below the compulsory bytes because inputs that stay in the 256 MB last-level cache from one call
 # of the loop to the next are not fetched from HBM again.
-MEASURED_TRAFFIC_BYTES = {("policy_bf16", 256): 493.7e6,          # 201 700 + 280 400 KiB, one launch
-                          ("long_lookback_bf16", 32): 2026.6e6,   # 914 100 + 1 065 000 KiB, one launch
-                          ("decay_extreme", 64): 326.7e6}         # states only 63 060 + 12 290, forward 107 200 + 136 500 KiB
-TRAFFIC_MEASURED_AT = "1955780"   # the library revision the counter runs in profiles/ were made at
+MEASURED_TRAFFIC_BYTES = {("policy_bf16", 256): 493.6e6,          # 201 600 + 280 400 KiB, one launch
+                          ("long_lookback_bf16", 32): 2116.6e6,   # 1 002 000 + 1 065 000 KiB, one launch
+                          ("decay_extreme", 64): 326.8e6}         # states only 63 050 + 12 290, forward 107 200 + 136 600 KiB
+TRAFFIC_MEASURED_AT = "4178078"   # the library revision the counter runs in profiles/ were made at
 # matrix-pipe busy fraction of the same kernels from the same counter runs (SQ_VALU_MFMA_BUSY_CYCLES over the
 # SIMD-cycles of the launch, GRBM_GUI_ACTIVE / 8 x 1 024 SIMDs): what the north star's "MFMA utilisation" reads as
 # on the hardware's own counters (decay-extreme: the forward launch of the two)
-MEASURED_MFMA_PIPE_BUSY = {("policy_bf16", 256): 0.234, ("long_lookback_bf16", 32): 0.249, ("decay_extreme", 64): 0.190}
+MEASURED_MFMA_PIPE_BUSY = {("policy_bf16", 256): 0.236, ("long_lookback_bf16", 32): 0.251, ("decay_extreme", 64): 0.189}
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 
