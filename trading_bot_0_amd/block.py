@@ -451,7 +451,7 @@ class Mamba2Block:
         E = in_proj_width(self.H, self.P, self.N, self.G)
         w_in, w_out = self._weights(act)
         dout2 = dout.reshape(Bsz * L, self.d_model)
-        dyn = torch.matmul(dout2, w_out).view(Bsz, L, self.d_inner)
+        dyn = self._project(dout2, self._out_proj_transposed(act)).view(Bsz, L, self.d_inner)
         dout_proj = _weight_gradient(dout2, yn.reshape(Bsz * L, self.d_inner))
         # the gradient of zxbcdt, with zxbcdt's own (padded) row stride
         ld = _row_stride(zxbcdt)
@@ -485,9 +485,16 @@ class Mamba2Block:
         key = (dtype, self.in_proj._version, self.out_proj._version, self.in_proj.data_ptr(), self.out_proj.data_ptr())
         cached = getattr(self, "_weights_cache", None)
         if cached is None or cached[0] != key:
-            cached = (key, self.in_proj.to(dtype).contiguous(), self.out_proj.to(dtype).contiguous())
+            w_out = self.out_proj.to(dtype).contiguous()
+            cached = (key, self.in_proj.to(dtype).contiguous(), w_out, w_out.t().contiguous())
             self._weights_cache = cached
         return cached[1], cached[2]
+
+    def _out_proj_transposed(self, dtype: torch.dtype) -> torch.Tensor:
+        """out_proj^T [d_inner, d_model] in the activation dtype (the backward's dyn = dout . out_proj is then a
+        product of the forward's form, which the library's projection kernel takes), cached with the others."""
+        self._weights(dtype)
+        return self._weights_cache[3]
 
     def _A_cached(self) -> torch.Tensor:
         """-exp(A_log), computed once per version of A_log (a launch of its own otherwise, per step)."""
