@@ -186,22 +186,29 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void fused_scan_wide_kernel(
         // where the staged pieces go: the swizzles repeat every 32 rows, and a pass is 32 rows.  Computed per tile from
         // a copy of the thread index that an empty asm hides from the compiler: hoisted out of the tile loop the
         // offsets would hold registers through both phases, which have none to spare.
+        // A B or C row is 256 bytes, twice the width of the banks, and the 16 lanes served together hold one row's 16
+        // pieces: writing the same 8-byte half of every piece at once would put 16 values on the even (or odd) 8-byte
+        // slots of 256 bytes, which fold onto 128 bytes of banks two by two.  So the lanes of the row's upper eight pieces
+        // write their halves in the other order (and odd rows the other way round, for the pair of rows that 32 lanes
+        // cover): each instruction then fills 128 bytes of banks exactly.
         int bw[2], xw[2];
+        bool swap;
         {
             int tw = tid;
             asm volatile("" : "+v"(tw));
+            swap = ((((tw % BPR) >> 3) ^ (tw / BPR)) & 1) != 0;
 #pragma unroll
             for (int hf = 0; hf < 2; ++hf) {
-                bw[hf] = BT::off(tw / BPR, (tw % BPR) * 8 + 4 * hf);
+                bw[hf] = BT::off(tw / BPR, (tw % BPR) * 8 + 4 * (swap ? 1 - hf : hf));
                 xw[hf] = fused_scan_xtile_base(Q, (tw % XPR) / 4) + XT::off(tw / XPR, ((tw % XPR) % 4) * 8 + 4 * hf);
             }
         }
 #pragma unroll
         for (int u = 0; u < UBC; ++u) {
-            *reinterpret_cast<uint2 *>(Bs + bw[0] + u * BRP * N) = make_uint2(bq[u].x, bq[u].y);
-            *reinterpret_cast<uint2 *>(Bs + bw[1] + u * BRP * N) = make_uint2(bq[u].z, bq[u].w);
-            *reinterpret_cast<uint2 *>(Cs + bw[0] + u * BRP * N) = make_uint2(cq[u].x, cq[u].y);
-            *reinterpret_cast<uint2 *>(Cs + bw[1] + u * BRP * N) = make_uint2(cq[u].z, cq[u].w);
+            *reinterpret_cast<uint2 *>(Bs + bw[0] + u * BRP * N) = swap ? make_uint2(bq[u].z, bq[u].w) : make_uint2(bq[u].x, bq[u].y);
+            *reinterpret_cast<uint2 *>(Bs + bw[1] + u * BRP * N) = swap ? make_uint2(bq[u].x, bq[u].y) : make_uint2(bq[u].z, bq[u].w);
+            *reinterpret_cast<uint2 *>(Cs + bw[0] + u * BRP * N) = swap ? make_uint2(cq[u].z, cq[u].w) : make_uint2(cq[u].x, cq[u].y);
+            *reinterpret_cast<uint2 *>(Cs + bw[1] + u * BRP * N) = swap ? make_uint2(cq[u].x, cq[u].y) : make_uint2(cq[u].z, cq[u].w);
         }
 #pragma unroll
         for (int u = 0; u < UX; ++u) {
