@@ -125,6 +125,9 @@ extern "C" {
     pub fn ssd_block_post_bwd(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
         norm_w: *const f32, eps: f32, dout: *const c_void, dy: *mut c_void, dzxbcdt: *mut c_void, dnorm_w: *mut f32,
         workspace: *mut c_void, workspace_bytes: usize, hip_stream: *mut c_void) -> c_int;
+    pub fn ssd_block_post_bwd_yn(dims: *const SsdBlockDims, dtype: c_int, y: *const c_void, zxbcdt: *const c_void,
+        norm_w: *const f32, eps: f32, dout: *const c_void, dy: *mut c_void, dzxbcdt: *mut c_void, dnorm_w: *mut f32,
+        yn_out: *mut c_void, workspace: *mut c_void, workspace_bytes: usize, hip_stream: *mut c_void) -> c_int;
     pub fn ssd_block_pre_bwd(dims: *const SsdBlockDims, dtype: c_int, zxbcdt: *const c_void, conv_w: *const f32,
         conv_b: *const f32, dt_bias: *const f32, conv_state_in: *const c_void, reset: *const u8, dx: *const c_void,
         db: *const c_void, dc: *const c_void, ddt: *const c_void, dconv_state_out: *const c_void,

@@ -319,6 +319,14 @@ int ssd_block_bwd_workspace_bytes(const ssd_block_dims *dims, int dtype, size_t 
 int ssd_block_post_bwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                        float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *workspace,
                        size_t workspace_bytes, void *hip_stream);
+/* The same, and with yn_out [B,L,H*P] (activation dtype; NULL allowed) also the forward's normalised rows, bit for bit
+ * what ssd_block_post_fwd writes: a training forward can then run gate, norm and out-projection as one kernel
+ * (ssd_block_post_proj_fwd, which never writes those rows) and the backward still has them for the out-projection's
+ * weight gradient dout^T yn, which is the only thing that reads them.  No counterpart in the reference, whose
+ * autograd keeps such tensors itself (trading_bots/src/torch/model/blocks/gqa.rs:172-178 is where its norm sits). */
+int ssd_block_post_bwd_yn(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                          float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *yn_out,
+                          void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /* Gradients of ssd_block_pre_reset_fwd: from dx [B,L,H,P], dB, dC [B,L,G,N], ddt [B,L,H] (what ssd_chunk_scan_bwd
  * returns) and, optionally, dconv_state_out [B,d_conv-1,C] (a gradient on the conv state the forward returned) to

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import mamba2_block_oracle as blk
-from trading_bot_0_amd import Mamba2Block, block_post_bwd, block_pre_bwd
+from trading_bot_0_amd import Mamba2Block, block_post, block_post_bwd, block_pre_bwd
 
 from _util import np64
 
@@ -76,12 +76,19 @@ def test_post_backward(shape, dtype):
     dzx2 = torch.empty_like(z)
     dy2, dw2 = block_post_bwd(y, z, p["norm_w"], dout, dzx2, H, P, N, G)
     assert torch.equal(dw, dw2) and torch.equal(dy, dy2)
+    # with yn_out, the forward's normalised rows on the way (for a forward that ran gate, norm and out-projection as
+    # one kernel and kept none): bit for bit what block_post writes, the gradients unchanged
+    yn = torch.full((Bsz, L, H * P), float("nan"), dtype=dtype, device="cuda")
+    dy4, dw4 = block_post_bwd(y, z, p["norm_w"], dout, dzx2, H, P, N, G, yn_out=yn)
+    assert torch.equal(yn, block_post(y, z, p["norm_w"], H, P, N, G)), "yn_out is not block_post's output"
+    assert torch.equal(dy4, dy) and torch.equal(dw4, dw)
     if dtype == torch.bfloat16:   # the scan's float32 y as the forward's input
         y32 = y.float() + 1e-3
-        dy3, dw3 = block_post_bwd(y32, z, p["norm_w"], dout, dzx2, H, P, N, G)
+        dy3, dw3 = block_post_bwd(y32, z, p["norm_w"], dout, dzx2, H, P, N, G, yn_out=yn)
         ry3, _, rw3 = blk.block_post_bwd(np64(y32), np64(z), np64(p["norm_w"]), 1e-5, np64(dout))
         check_act(dy3, ry3, dtype, "dy from float32 y")
         check_sum(dw3, rw3, scale, dtype, "dnorm_w from float32 y")
+        assert torch.equal(yn, block_post(y32, z, p["norm_w"], H, P, N, G)), "yn_out from float32 y"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -43,8 +43,9 @@ def _lib():
         lib.ssd_block_pre_reset_fwd.restype = c_int
         lib.ssd_block_bwd_workspace_bytes.argtypes = [POINTER(SsdBlockDims), c_int, POINTER(c_size_t)]
         lib.ssd_block_post_bwd.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, P, P, P, P, c_size_t, P]
+        lib.ssd_block_post_bwd_yn.argtypes = [POINTER(SsdBlockDims), c_int, P, P, P, c_float, P, P, P, P, P, P, c_size_t, P]
         lib.ssd_block_pre_bwd.argtypes = [POINTER(SsdBlockDims), c_int] + [P] * 17 + [c_size_t, P]
-        for name in ("ssd_block_bwd_workspace_bytes", "ssd_block_post_bwd", "ssd_block_pre_bwd"):
+        for name in ("ssd_block_bwd_workspace_bytes", "ssd_block_post_bwd", "ssd_block_post_bwd_yn", "ssd_block_pre_bwd"):
             getattr(lib, name).restype = c_int
         lib.ssd_block_pre_fwd.restype = c_int
         lib.ssd_block_post_fwd.restype = c_int
@@ -248,10 +249,12 @@ def block_bwd_workspace(batch, seqlen, nheads, headdim, dstate, ngroups, d_conv=
 
 
 def block_post_bwd(y, zxbcdt, norm_w, dout, dzxbcdt, nheads, headdim, dstate, ngroups, eps=1e-5, workspace=None,
-                   d_conv=4):
+                   d_conv=4, yn_out=None):
     """Gradients of block_post: returns (dy [B,L,H,P], dnorm_w [H*P]) and writes dz into the z channels of dzxbcdt
     (a tensor laid out like zxbcdt, same row stride).  `d_conv` is the block's filter length: the library sizes the
-    scratch both backward calls of a pass share from it, so it must be the one `workspace` was sized with."""
+    scratch both backward calls of a pass share from it, so it must be the one `workspace` was sized with.
+    With `yn_out` [B,L,H*P] (zxbcdt's dtype) the call also writes the forward's normalised rows into it, bit for bit
+    what `block_post` returns (for a forward that ran `block_post_proj` and kept none)."""
     lib = _lib()
     Bsz, L, E = zxbcdt.shape
     H, P, N, G = nheads, headdim, dstate, ngroups
@@ -272,9 +275,12 @@ def block_post_bwd(y, zxbcdt, norm_w, dout, dzxbcdt, nheads, headdim, dstate, ng
     if workspace is None:
         workspace = block_bwd_workspace(Bsz, L, H, P, N, G, d_conv, dtype, zxbcdt.device)
     dims = SsdBlockDims(Bsz, L, H, P, N, G, d_conv, ld)
-    ssd._check(lib, lib.ssd_block_post_bwd(byref(dims), code, y.data_ptr(), zxbcdt.data_ptr(), norm_w.data_ptr(), c_float(eps),
-                                           dout.data_ptr(), dy.data_ptr(), dzxbcdt.data_ptr(), dnorm_w.data_ptr(),
-                                           workspace.data_ptr(), workspace.numel(), ssd._stream_ptr(zxbcdt)))
+    if yn_out is not None:
+        ssd._require(yn_out, "yn_out", (Bsz, L, H * P), dtype)
+    ssd._check(lib, lib.ssd_block_post_bwd_yn(byref(dims), code, y.data_ptr(), zxbcdt.data_ptr(), norm_w.data_ptr(), c_float(eps),
+                                              dout.data_ptr(), dy.data_ptr(), dzxbcdt.data_ptr(), dnorm_w.data_ptr(),
+                                              None if yn_out is None else yn_out.data_ptr(),
+                                              workspace.data_ptr(), workspace.numel(), ssd._stream_ptr(zxbcdt)))
     return dy, dnorm_w
 
 
@@ -428,15 +434,17 @@ class Mamba2Block:
             state.conv = conv
             y = state.ssm.init_from_prefix(x, dt, self.A, Bm, Cm, self.D, chunk=self.chunk)
         w_out = self._weights(u.dtype)[1]
-        if not save_for_backward and block_post_proj_supported(y, w_out) and y.numel() // self.d_inner >= 8192:
+        if save_for_backward and state is not None:
+            raise ValueError("backward through a window that continues a carried state is not supported")
+        if block_post_proj_supported(y, w_out) and y.numel() // self.d_inner >= 8192:
             # gate, norm and out-projection as one kernel: the normalised rows never reach memory (the backward pass
-            # needs them, so a forward that keeps its tensors for it runs the two stages)
-            return block_post_proj(y, zxbcdt, self.norm_w, w_out, self.H, self.P, self.N, self.G, self.eps)
-        yn = block_post(y, zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
-        out = self._project(yn, w_out)
+            # needs them for one weight gradient only, and has its post stage write them on the way: yn=None)
+            out = block_post_proj(y, zxbcdt, self.norm_w, w_out, self.H, self.P, self.N, self.G, self.eps)
+            yn = None
+        else:
+            yn = block_post(y, zxbcdt, self.norm_w, self.H, self.P, self.N, self.G, self.eps)
+            out = self._project(yn, w_out)
         if save_for_backward:
-            if state is not None:
-                raise ValueError("backward through a window that continues a carried state is not supported")
             return out, dict(u=u, zxbcdt=zxbcdt, x=x, Bm=Bm, Cm=Cm, dt=dt, y=y, yn=yn, reset=reset)
         return out
 
@@ -452,14 +460,16 @@ class Mamba2Block:
         w_in, w_out = self._weights(act)
         dout2 = dout.reshape(Bsz * L, self.d_model)
         dyn = self._project(dout2, self._out_proj_transposed(act)).view(Bsz, L, self.d_inner)
-        dout_proj = _weight_gradient(dout2, yn.reshape(Bsz * L, self.d_inner))
+        # (a forward that ran gate, norm and out-projection as one kernel kept no normalised rows: post_bwd writes them)
+        yn_new = None if yn is not None else torch.empty((Bsz, L, self.d_inner), dtype=act, device=u.device)
         # the gradient of zxbcdt, with zxbcdt's own (padded) row stride
         ld = _row_stride(zxbcdt)
         dbuf = torch.empty((Bsz, L, ld), dtype=act, device=u.device)
         dzx = dbuf[..., :E] if ld != E else dbuf
         ws = block_bwd_workspace(Bsz, L, self.H, self.P, self.N, self.G, self.d_conv, act, u.device)
         dy, dnorm_w = block_post_bwd(y, zxbcdt, self.norm_w, dyn, dzx, self.H, self.P, self.N, self.G, self.eps, workspace=ws,
-                                     d_conv=self.d_conv)
+                                     d_conv=self.d_conv, yn_out=yn_new)
+        dout_proj = _weight_gradient(dout2, (yn if yn is not None else yn_new).reshape(Bsz * L, self.d_inner))
         g = ssd.ssd_chunk_scan_backward(x, dt, self.A, Bm, Cm, self.D, dy, chunk=self.chunk, reset=reset)
         dconv_w, dconv_b, ddt_bias, _ = block_pre_bwd(zxbcdt, self.conv_w, self.conv_b, self.dt_bias, g["dx"], g["dB"],
                                                       g["dC"], g["ddt"], dzx, self.H, self.P, self.N, self.G, reset=reset,

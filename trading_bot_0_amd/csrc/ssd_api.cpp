@@ -904,6 +904,13 @@ int ssd_block_bwd_workspace_bytes(const ssd_block_dims *dims, int dtype, size_t 
 int ssd_block_post_bwd(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                        float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *workspace,
                        size_t workspace_bytes, void *hip_stream) {
+    return ssd_block_post_bwd_yn(dims, dtype, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, nullptr, workspace,
+                                 workspace_bytes, hip_stream);
+}
+
+int ssd_block_post_bwd_yn(const ssd_block_dims *dims, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
+                          float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *yn_out,
+                          void *workspace, size_t workspace_bytes, void *hip_stream) {
     ssd::BlockShape s;
     if (int rc = make_block_shape(dims, dtype, &s)) return rc;
     REQUIRE_PTR(y);
@@ -918,8 +925,9 @@ int ssd_block_post_bwd(const ssd_block_dims *dims, int dtype, const void *y, con
     const size_t need = ssd::block_bwd_workspace_bytes(s);
     if (workspace_bytes < need)
         return fail(SSD_ERR_WORKSPACE, "ssd: block backward workspace has %zu bytes, %zu needed", workspace_bytes, need);
+    OPTIONAL_PTR(yn_out);
     hipError_t e = ssd::launch_block_post_bwd(s, dtype, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, workspace,
-                                              (hipStream_t)hip_stream);
+                                              (hipStream_t)hip_stream, yn_out);
     return e == hipSuccess ? SSD_OK : hip_fail(e, "block post-scan backward launch");
 }
 

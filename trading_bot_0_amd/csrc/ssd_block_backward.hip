@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
                                                              const float *__restrict__ norm_w, float eps,
                                                              const T *__restrict__ dout, T *__restrict__ dy,
                                                              T *__restrict__ dzxbcdt, float *__restrict__ dw_part,
-                                                             BlockShape s) {
+                                                             T *__restrict__ yn, BlockShape s) {
     const int DI = s.H * s.P;
     const int lane = threadIdx.x & (LPR - 1);
     constexpr int MAXP = PPL;
@@ -93,6 +93,7 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
         return o;
     };
     const float inv_di = 1.f / (float)DI;
+    const float di = (float)DI;
     const long long stride = (long long)gridDim.x * RPB;
     RowIn cur = fetch((long long)blockIdx.x * RPB + threadIdx.x / LPR);
     auto pass = [&](long long row0, auto whole_tag) {
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
         }
         ss = group_sum<LPR>(ss);
         gv = group_sum<LPR>(gv);
-        const float r = rsqrtf(ss * inv_di + eps);
+        const float r = rsqrtf(ss / di + eps);  // (the forward's expression: yn below is its output bit for bit)
         const float k3 = r * r * r * gv * inv_di;
 #pragma unroll
         for (int u = 0; u < MAXP; ++u) {
@@ -144,6 +145,12 @@ __global__ __launch_bounds__(256) void block_post_bwd_kernel(const TY *__restric
                 }
                 Pack8<T>::store(dy + (size_t)row * DI + c0, oy);
                 Pack8<T>::store(dzxbcdt + (size_t)row * s.ld + c0, oz);
+                if (yn != nullptr) {  // (uniform) the normalised row, for a forward that did not keep it
+                    float on[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) on[i] = yy[u][i] * silu(zz[u][i]) * r * wv[u][i];
+                    Pack8<T>::store(yn + (size_t)row * DI + c0, on);
+                }
             }
         }
     };
@@ -596,12 +603,13 @@ size_t block_bwd_workspace_bytes(const BlockShape &s) {
 
 template <typename T, typename TY>
 static hipError_t post_bwd_dispatch(const BlockShape &s, const void *y, const void *zxbcdt, const float *norm_w, float eps,
-                                    const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, float *part, hipStream_t st) {
+                                    const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, float *part, void *yn,
+                                    hipStream_t st) {
     const int DI = s.H * s.P, pieces = DI / 8;
     const long long rows = (long long)s.B * s.L;
     const TY *yy = static_cast<const TY *>(y);
     const T *zz = static_cast<const T *>(zxbcdt), *dd = static_cast<const T *>(dout);
-    T *oy = static_cast<T *>(dy), *oz = static_cast<T *>(dzxbcdt);
+    T *oy = static_cast<T *>(dy), *oz = static_cast<T *>(dzxbcdt), *on = static_cast<T *>(yn);
     // lanes per row and pieces per lane as in the forward
     const int lpr = pieces <= 16 * 4 ? 16 : pieces <= 32 * 4 ? 32 : 64;
     const int ppl = (pieces + lpr - 1) / lpr;
@@ -610,9 +618,9 @@ static hipError_t post_bwd_dispatch(const BlockShape &s, const void *y, const vo
 #define SSD_POST_BWD_CASE(LPRv, PPLv)                                                                                       \
     if (lpr == LPRv && ppl == PPLv) {                                                                                       \
         if (pieces == LPRv * PPLv)                                                                                          \
-            block_post_bwd_kernel<T, TY, LPRv, PPLv, true><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, s); \
+            block_post_bwd_kernel<T, TY, LPRv, PPLv, true><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, on, s); \
         else                                                                                                                \
-            block_post_bwd_kernel<T, TY, LPRv, PPLv, false><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, s); \
+            block_post_bwd_kernel<T, TY, LPRv, PPLv, false><<<dim3(blocks), dim3(256), 0, st>>>(yy, zz, norm_w, eps, dd, oy, oz, part, on, s); \
         launched = true;                                                                                                    \
     }
     SSD_POST_BWD_CASE(16, 1) SSD_POST_BWD_CASE(16, 2) SSD_POST_BWD_CASE(16, 3) SSD_POST_BWD_CASE(16, 4)
@@ -627,12 +635,12 @@ static hipError_t post_bwd_dispatch(const BlockShape &s, const void *y, const vo
 
 hipError_t launch_block_post_bwd(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                                  float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *workspace,
-                                 hipStream_t st) {
+                                 hipStream_t st, void *yn) {
     float *part = static_cast<float *>(workspace);
     switch (dtype) {
-        case 0: return post_bwd_dispatch<float, float>(s, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, part, st);
-        case 1: return post_bwd_dispatch<__bf16, __bf16>(s, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, part, st);
-        default: return post_bwd_dispatch<__bf16, float>(s, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, part, st);
+        case 0: return post_bwd_dispatch<float, float>(s, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, part, yn, st);
+        case 1: return post_bwd_dispatch<__bf16, __bf16>(s, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, part, yn, st);
+        default: return post_bwd_dispatch<__bf16, float>(s, y, zxbcdt, norm_w, eps, dout, dy, dzxbcdt, dnorm_w, part, yn, st);
     }
 }
 

@@ -141,11 +141,13 @@ hipError_t launch_block_post(const BlockShape &s, int dtype, const void *y, cons
 
 // Backward of the two stages (dtype as the forward's; dtype 2 = bf16 activations with the scan's float32 y in
 // post_bwd).  dzxbcdt [B,L,ld] is the gradient of zxbcdt: post_bwd writes its z channels, pre_bwd its x | B | C | dt
-// channels.  workspace: block_bwd_workspace_bytes (partial sums of the parameter gradients).
+// channels.  workspace: block_bwd_workspace_bytes (partial sums of the parameter gradients).  With yn given
+// ([B,L,H*P], the activation type) post_bwd also writes the forward's normalised rows, bit for bit what
+// launch_block_post writes, for a forward that did not keep them.
 size_t block_bwd_workspace_bytes(const BlockShape &s);
 hipError_t launch_block_post_bwd(const BlockShape &s, int dtype, const void *y, const void *zxbcdt, const float *norm_w,
                                  float eps, const void *dout, void *dy, void *dzxbcdt, float *dnorm_w, void *workspace,
-                                 hipStream_t stream);
+                                 hipStream_t stream, void *yn = nullptr);
 hipError_t launch_block_pre_bwd(const BlockShape &s, int dtype, const void *zxbcdt, const float *conv_w, const float *conv_b,
                                 const float *dt_bias, const void *state_in, const unsigned char *reset, const void *dx,
                                 const void *dB, const void *dC, const void *ddt, const void *dstate_out, void *dzxbcdt,

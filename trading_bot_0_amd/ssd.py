@@ -51,6 +51,7 @@ EXPORTED_SYMBOLS = (
     "ssd_block_pre_reset_fwd",
     "ssd_block_bwd_workspace_bytes",
     "ssd_block_post_bwd",
+    "ssd_block_post_bwd_yn",
     "ssd_block_pre_bwd",
     "ssd_block_post_proj_fwd",
     "ssd_block_step_fwd",
