@@ -589,9 +589,13 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 || NK == 8) ? 1 : 2) void f
         const int rows = min(Q, s.L - t0);
         // the state entering every tile, for a caller that needs it (the backward pass): [B, nc, H, P, N]
         // (of every an.stride-th tile from an.phase on, where the backward pass's other scan asks for fewer)
-        if (tile_states && c >= an.phase && (c - an.phase) % an.stride == 0) {
-            const int kept = (s.nc - 1 - an.phase) / an.stride + 1;
-            store_state(tile_states + (((size_t)b * kept + (c - an.phase) / an.stride) * s.H + h) * s.P * N);
+        if constexpr (TR) {
+            if (tile_states && c >= an.phase && (c - an.phase) % an.stride == 0) {
+                const int kept = (s.nc - 1 - an.phase) / an.stride + 1;
+                store_state(tile_states + (((size_t)b * kept + (c - an.phase) / an.stride) * s.H + h) * s.P * N);
+            }
+        } else {  // (the other kinds keep every tile's)
+            if (tile_states) store_state(tile_states + (((size_t)b * s.nc + c) * s.H + h) * s.P * N);
         }
         if (!kTwoSets) block_sync_lds();  // every wave is done reading the previous chunk's tiles
         // ---- registers -> LDS tiles ----
